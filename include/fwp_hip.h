@@ -1,0 +1,141 @@
+/*
+ * fwp_hip.h -- C ABI of libfwp_hip.so, the MI355X (gfx950) implementation of the
+ * fast-weight update operators of IDSIA/recurrent-fwp.
+ *
+ * Every entry point replaces one pybind11 function of the reference's CUDA
+ * extensions (cited per function).  Differences that hold for all of them:
+ *   - plain pointers to fp32 DEVICE memory and plain integers; no torch types;
+ *   - work is enqueued on the HIP stream handed in (`stream`, a hipStream_t cast
+ *     to void*; NULL = the default stream); nothing synchronises;
+ *   - outputs are fully overwritten (the reference accumulates with atomicAdd into
+ *     caller-zeroed buffers); results are deterministic;
+ *   - the return value is 0 on success, a negative FWP_E_* for a rejected call
+ *     (nothing was launched) or a positive hipError_t from the launch.
+ *
+ * Tensors are [N,H,L,*] as in the reference.  Inputs may be strided views
+ * (struct fwp_view: element strides of the N, H and L axes; the last axis must be
+ * contiguous).  Outputs, states and saved buffers are contiguous.
+ * The fast-weight state is W[N,H,E,M] with v_old[m] = sum_e W[e][m] k[e].
+ *
+ * Backward never rewinds the caller's W: forward stores the state at the end of
+ * every `chunk` steps in `ckpt[N,H,nchunk,E,M]`, nchunk = ceil(L/chunk), and
+ * v - v_old per step in `vdiff`; backward walks the chunks in reverse from those.
+ */
+#ifndef FWP_HIP_H
+#define FWP_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct fwp_view {
+    const float *ptr;   /* device pointer to element [0,0,0,0] */
+    int64_t sN, sH, sL; /* strides in elements; last-axis stride is 1 */
+} fwp_view;
+
+enum {
+    FWP_OK = 0,
+    FWP_E_NULL = -1,      /* a required pointer is NULL */
+    FWP_E_SHAPE = -2,     /* a dimension is < 1 or inconsistent */
+    FWP_E_CHUNK = -3,     /* chunk is not a positive multiple of FWP_Q_CHUNK_QUANTUM */
+    FWP_E_TOO_LARGE = -4, /* state does not fit the workgroup's LDS */
+    FWP_E_ARCH = -5       /* current device is not gfx950 */
+};
+
+enum {
+    FWP_Q_VERSION = 0,
+    FWP_Q_CHUNK_QUANTUM = 1, /* chunk must be a multiple of this */
+    FWP_Q_DEFAULT_CHUNK = 2,
+    FWP_Q_MAX_STATE_FLOATS = 3 /* largest E*M (delta) the library accepts */
+};
+
+const char *fwp_strerror(int code);
+int fwp_query(int what);
+
+/* 0 if the current HIP device is a gfx950 part, FWP_E_ARCH otherwise. */
+int fwp_check_device(void);
+
+/*
+ * Delta rule forward.  Replaces fast_weight_forward
+ * (algorithmic/fast_weight/fast_weight_cuda.cu:182-240, kernel :17-178).
+ *   q,k [N,H,L,E]  v [N,H,L,M]  beta [N,H,L,1]
+ *   W [N,H,E,M] in/out: initial state in, state after step L-1 out
+ *   out [N,H,L,M]; vdiff [N,H,L,M] = v - v_old; ckpt [N,H,nchunk,E,M]
+ * vdiff and ckpt may both be NULL for a forward that will not be differentiated.
+ */
+int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,
+                  float *out, float *vdiff, float *ckpt, int N, int H, int L,
+                  int E, int M, int chunk, void *stream);
+
+/*
+ * Delta rule backward.  Replaces fast_weight_backward
+ * (algorithmic/fast_weight/fast_weight_cuda.cu:564-664, kernels :397-560 and
+ * :244-393) with one fused reverse pass.
+ *   grad_out [N,H,L,M] (strided view allowed)
+ *   gq,gk [N,H,L,E]  gv [N,H,L,M]  gbeta [N,H,L,1]
+ */
+int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff,
+                  fwp_view grad_out, const float *ckpt, float *gq, float *gk,
+                  float *gv, float *gbeta, int N, int H, int L, int E, int M,
+                  int chunk, void *stream);
+
+/*
+ * Delta RNN v2 forward.  Replaces fast_rnn_v2_forward
+ * (algorithmic/fast_weight_rnn_v2/fast_rnn_cuda.cu:233-293, kernel :25-229).
+ *   z,k,v [N,H,L,D]  beta [N,H,L,1]  W [N,H,D,D] in/out  h [N,H,D] in/out
+ *   out [N,H,L,D]; vdiff, ckpt as above (E=M=D).
+ * The softmax of the previous output is exact (no epsilon in the denominator),
+ * as in the reference's PyTorch loop (fast_weight_rnn_v2/__init__.py:214).
+ */
+int fwp_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W,
+                float *h, float *out, float *vdiff, float *ckpt, int N, int H,
+                int L, int D, int chunk, void *stream);
+
+/*
+ * Delta RNN v2 backward.  Replaces fast_rnn_v2_backward
+ * (algorithmic/fast_weight_rnn_v2/fast_rnn_cuda.cu:592-659, kernel :297-588).
+ *   out [N,H,L,D] is the forward output, h_init [N,H,D] the state the forward
+ *   started from; softmax of the delayed output is recomputed from them.
+ */
+int fwp_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
+                const float *h_init, fwp_view grad_out, const float *ckpt,
+                float *gz, float *gk, float *gv, float *gbeta, int N, int H,
+                int L, int D, int chunk, void *stream);
+
+/*
+ * Recurrent Delta Net forward.  Replaces rec_update_fwm_tanh_forward
+ * (algorithmic/rec_update_fwm_tanh/rec_update_fwm_tanh.cu:349-444, kernel :25-345).
+ *   qx,kx,vx [N,H,L,D] and bx [N,H,L,1] are pre-activation
+ *   Rq,Rk,Rv [H,D,D] indexed [e_in][m_out], rb [H,D]  (contiguous)
+ *   W [N,H,D,D] in/out, h [N,H,D] in/out, out [N,H,L,D]
+ *   saved for backward: q_act,k_act [N,H,L,D] (after softmax), beta_act [N,H,L]
+ *   (after sigmoid), vdiff [N,H,L,D], ckpt.
+ */
+int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx,
+                const float *Rq, const float *Rk, const float *Rv,
+                const float *rb, float *W, float *h, float *out, float *q_act,
+                float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,
+                int H, int L, int D, int chunk, void *stream);
+
+/*
+ * Recurrent Delta Net backward.  Replaces rec_update_fwm_tanh_backward
+ * (algorithmic/rec_update_fwm_tanh/rec_update_fwm_tanh.cu:880-986, kernel :448-876).
+ *   gqx,gkx,gvx [N,H,L,D]  gbx [N,H,L,1]
+ *   gRq,gRk,gRv [H,D,D], grb [H,D]: summed over N and L in a fixed order.
+ *   workspace: N*H*(3*D*D+D) floats of scratch for the per-sequence partial sums
+ *   (the reference adds them with global atomics, :791-824).
+ */
+int fwp_rec_bwd(const float *q_act, const float *k_act, const float *beta_act,
+                const float *vdiff, const float *out, const float *h_init,
+                fwp_view grad_out, const float *Rq, const float *Rk,
+                const float *Rv, const float *rb, const float *ckpt, float *gqx,
+                float *gkx, float *gvx, float *gbx, float *gRq, float *gRk,
+                float *gRv, float *grb, float *workspace, int N, int H, int L,
+                int D, int chunk, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FWP_HIP_H */

@@ -1,0 +1,107 @@
+"""ctypes binding of libfwp_hip.so (the C ABI declared in include/fwp_hip.h).
+
+There is no fallback: if the shared library is missing or a call is rejected the
+caller gets an exception.
+"""
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "libfwp_hip.so")
+
+_F = ctypes.POINTER(ctypes.c_float)
+
+
+class View(ctypes.Structure):
+    """struct fwp_view: device pointer + element strides of the N, H, L axes."""
+    _fields_ = [("ptr", ctypes.c_void_p), ("sN", ctypes.c_int64), ("sH", ctypes.c_int64),
+                ("sL", ctypes.c_int64)]
+
+
+class FwpError(RuntimeError):
+    pass
+
+
+_P, _I, _V = ctypes.c_void_p, ctypes.c_int, View
+_SIGNATURES = {
+    "fwp_delta_fwd": [_V] * 4 + [_P] * 4 + [_I] * 6 + [_P],
+    "fwp_delta_bwd": [_V] * 3 + [_P, _V, _P] + [_P] * 4 + [_I] * 6 + [_P],
+    "fwp_rnn_fwd": [_V] * 4 + [_P] * 5 + [_I] * 5 + [_P],
+    "fwp_rnn_bwd": [_V, _V, _P, _P, _P, _V, _P] + [_P] * 4 + [_I] * 5 + [_P],
+    "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
+    "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
+}
+EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device"])
+
+_lib = None
+_checked_devices = set()
+
+
+def lib():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            raise FwpError(
+                f"{SO_PATH} is missing: build it with recurrent-fwp_amd/csrc/build.sh "
+                "(there is no CPU or PyTorch fallback for the fast-weight operators)")
+        handle = ctypes.CDLL(SO_PATH)
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        handle.fwp_strerror.argtypes = [ctypes.c_int]
+        handle.fwp_strerror.restype = ctypes.c_char_p
+        handle.fwp_query.argtypes = [ctypes.c_int]
+        handle.fwp_query.restype = ctypes.c_int
+        handle.fwp_check_device.restype = ctypes.c_int
+        _lib = handle
+    return _lib
+
+
+def query(what):
+    return int(lib().fwp_query(int(what)))
+
+
+Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
+
+
+def strerror(code):
+    return lib().fwp_strerror(int(code)).decode()
+
+
+def check(code, what):
+    if code != 0:
+        raise FwpError(f"{what} failed: {strerror(code)} (code {code})")
+
+
+def require_device(t):
+    """The operators exist for fp32 tensors on a gfx950 GPU only."""
+    if t.device.type != "cuda":
+        raise FwpError(f"fast-weight operators need tensors on an MI355X GPU, got device '{t.device}'")
+    idx = t.device.index if t.device.index is not None else torch.cuda.current_device()
+    if idx not in _checked_devices:
+        with torch.cuda.device(idx):
+            check(lib().fwp_check_device(), "device check")
+        _checked_devices.add(idx)
+
+
+def rows(t):
+    """A view argument for a 4-D fp32 tensor; copies only if the last axis is strided."""
+    if t.dtype != torch.float32:
+        raise FwpError(f"fast-weight operators are fp32 only, got {t.dtype}")
+    if t.dim() != 4:
+        raise FwpError(f"expected a 4-D [N,H,L,D] tensor, got {t.dim()}-D")
+    if t.shape[-1] != 1 and t.stride(-1) != 1:
+        t = t.contiguous()
+    return t, View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+
+def ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def stream_of(t):
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)

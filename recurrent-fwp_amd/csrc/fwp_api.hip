@@ -1,0 +1,135 @@
+// extern "C" entry points of libfwp_hip.so: argument checks and dispatch between
+// the register-state kernels (E = M in {16, 32}, 16-byte aligned rows) and the
+// LDS-state kernels (everything else).
+#include "fwp_common.hpp"
+
+#include <string.h>
+
+using namespace fwp;
+
+namespace {
+
+bool bad_view(const fwp_view &v) { return v.ptr == nullptr; }
+
+int check_dims(int N, int H, int L, int E, int M, int chunk) {
+    if (N < 1 || H < 1 || L < 1 || E < 1 || M < 1) return FWP_E_SHAPE;
+    if (chunk < kTile || chunk % kTile != 0) return FWP_E_CHUNK;
+    if ((int64_t)E * M > fwp_query(FWP_Q_MAX_STATE_FLOATS)) return FWP_E_TOO_LARGE;
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *fwp_strerror(int code) {
+    switch (code) {
+        case FWP_OK: return "ok";
+        case FWP_E_NULL: return "a required pointer is NULL";
+        case FWP_E_SHAPE: return "a dimension is < 1 or inconsistent";
+        case FWP_E_CHUNK: return "chunk is not a positive multiple of the chunk quantum";
+        case FWP_E_TOO_LARGE: return "the fast-weight state does not fit the workgroup's LDS";
+        case FWP_E_ARCH: return "the current device is not a gfx950 (MI355X) part";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString((hipError_t)code);
+    return "unknown error";
+}
+
+int fwp_query(int what) {
+    switch (what) {
+        case FWP_Q_VERSION: return 1;
+        case FWP_Q_CHUNK_QUANTUM: return kTile;
+        case FWP_Q_DEFAULT_CHUNK: return kDefaultChunk;
+        case FWP_Q_MAX_STATE_FLOATS: return 16384;
+        default: return -1;
+    }
+}
+
+int fwp_check_device(void) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    hipDeviceProp_t p;
+    e = hipGetDeviceProperties(&p, dev);
+    if (e != hipSuccess) return (int)e;
+    return strncmp(p.gcnArchName, "gfx950", 6) == 0 ? FWP_OK : FWP_E_ARCH;
+}
+
+int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                  float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
+                  void *stream) {
+    if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(beta) || !W || !out)
+        return FWP_E_NULL;
+    if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
+                             (hipStream_t)stream);
+}
+
+int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view grad_out,
+                  const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
+                  int L, int E, int M, int chunk, void *stream) {
+    if (bad_view(q) || bad_view(k) || bad_view(beta) || bad_view(grad_out) || !vdiff || !ckpt ||
+        !gq || !gk || !gv || !gbeta)
+        return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    return generic_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
+                             chunk, (hipStream_t)stream);
+}
+
+int fwp_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
+                float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, void *stream) {
+    if (bad_view(z) || bad_view(k) || bad_view(v) || bad_view(beta) || !W || !h || !out)
+        return FWP_E_NULL;
+    if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    return generic_rnn_fwd(z, k, v, beta, W, h, out, vdiff, ckpt, N, H, L, D, chunk,
+                           (hipStream_t)stream);
+}
+
+int fwp_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
+                const float *h_init, fwp_view grad_out, const float *ckpt, float *gz, float *gk,
+                float *gv, float *gbeta, int N, int H, int L, int D, int chunk, void *stream) {
+    if (bad_view(k) || bad_view(beta) || bad_view(grad_out) || !vdiff || !out || !h_init ||
+        !ckpt || !gz || !gk || !gv || !gbeta)
+        return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    return generic_rnn_bwd(k, beta, vdiff, out, h_init, grad_out, ckpt, gz, gk, gv, gbeta, N, H, L,
+                           D, chunk, (hipStream_t)stream);
+}
+
+int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,
+                float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,
+                int H, int L, int D, int chunk, void *stream) {
+    if (bad_view(qx) || bad_view(kx) || bad_view(vx) || bad_view(bx) || !Rq || !Rk || !Rv ||
+        !rb || !W || !h || !out)
+        return FWP_E_NULL;
+    const int saved = (q_act != nullptr) + (k_act != nullptr) + (beta_act != nullptr) +
+                      (vdiff != nullptr) + (ckpt != nullptr);
+    if (saved != 0 && saved != 5) return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    return generic_rec_fwd(qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act,
+                           vdiff, ckpt, N, H, L, D, chunk, (hipStream_t)stream);
+}
+
+int fwp_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, const float *vdiff,
+                const float *out, const float *h_init, fwp_view grad_out, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, const float *ckpt, float *gqx,
+                float *gkx, float *gvx, float *gbx, float *gRq, float *gRk, float *gRv,
+                float *grb, float *workspace, int N, int H, int L, int D, int chunk,
+                void *stream) {
+    if (!q_act || !k_act || !beta_act || !vdiff || !out || !h_init || bad_view(grad_out) || !Rq ||
+        !Rk || !Rv || !rb || !ckpt || !gqx || !gkx || !gvx || !gbx || !gRq || !gRk || !gRv ||
+        !grb || !workspace)
+        return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    int rc = generic_rec_bwd(q_act, k_act, beta_act, vdiff, out, h_init, grad_out, Rq, Rk, Rv, rb,
+                             ckpt, gqx, gkx, gvx, gbx, workspace, N, H, L, D, chunk,
+                             (hipStream_t)stream);
+    if (rc) return rc;
+    return reduce_rec_param_grads(workspace, gRq, gRk, gRv, grb, N, H, D, (hipStream_t)stream);
+}
+
+}  // extern "C"

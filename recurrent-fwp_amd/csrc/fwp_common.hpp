@@ -1,0 +1,47 @@
+// Shared declarations of the HIP sources of libfwp_hip.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "fwp_hip.h"
+
+namespace fwp {
+
+// Length of the LDS input tiles of the register-state kernels.  The state
+// checkpoint interval (`chunk` of the C ABI) must be a multiple of it.
+constexpr int kTile = 16;
+constexpr int kDefaultChunk = 64;
+
+__device__ __forceinline__ const float *row(const fwp_view &v, int n, int h, int t) {
+    return v.ptr + (int64_t)n * v.sN + (int64_t)h * v.sH + (int64_t)t * v.sL;
+}
+
+// Launchers of the LDS-state kernels (any E, M that fit the LDS).
+int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                      float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
+                      hipStream_t s);
+int generic_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
+                      const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N,
+                      int H, int L, int E, int M, int chunk, hipStream_t s);
+int generic_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h,
+                    float *out, float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
+                    hipStream_t s);
+int generic_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
+                    const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
+                    float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s);
+int generic_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
+                    const float *Rk, const float *Rv, const float *rb, float *W, float *h,
+                    float *out, float *q_act, float *k_act, float *beta_act, float *vdiff,
+                    float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+int generic_rec_bwd(const float *q_act, const float *k_act, const float *beta_act,
+                    const float *vdiff, const float *out, const float *h_init, fwp_view go,
+                    const float *Rq, const float *Rk, const float *Rv, const float *rb,
+                    const float *ckpt, float *gqx, float *gkx, float *gvx, float *gbx,
+                    float *workspace, int N, int H, int L, int D, int chunk, hipStream_t s);
+// gR*[H,D,D], grb[H,D] = sum over n of workspace[n,h,:] in ascending n.
+int reduce_rec_param_grads(const float *workspace, float *gRq, float *gRk, float *gRv,
+                           float *grb, int N, int H, int D, hipStream_t s);
+
+// Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
+constexpr size_t kMaxLds = 160 * 1024 - 1024;
+
+}  // namespace fwp

@@ -1,0 +1,78 @@
+"""Delta-rule fast weight memory: drop-in for the reference's ``fast_weight``
+package (algorithmic/fast_weight/__init__.py:26-96; the language-modelling copy
+is ``utils.fast_fast_weight``)."""
+import torch
+
+from . import _lib
+
+
+def _nchunk(L, chunk):
+    return (L + chunk - 1) // chunk
+
+
+class DeltaFastWeight(torch.autograd.Function):
+    """``out = fast_weight_delta(Q, K, V, beta, W)``.
+
+    Q, K ``[N,H,L,E]``; V ``[N,H,L,M]``; beta ``[N,H,L,1]``; W ``[N,H,E,M]`` is the
+    initial state on entry and the state after the last step on return (in place).
+    Gradients flow to Q, K, V and beta; W gets none, as in the reference (:92).
+    Unlike the reference, backward leaves W untouched.
+    """
+
+    @staticmethod
+    def forward(ctx, Q, K, V, beta, W):
+        _lib.require_device(Q)
+        N, H, L, E = Q.shape
+        M = V.shape[-1]
+        if K.shape != (N, H, L, E) or V.shape != (N, H, L, M) or beta.shape != (N, H, L, 1):
+            raise _lib.FwpError(f"shape mismatch: Q{tuple(Q.shape)} K{tuple(K.shape)} "
+                                f"V{tuple(V.shape)} beta{tuple(beta.shape)}")
+        if W.shape != (N, H, E, M) or not W.is_contiguous() or W.dtype != torch.float32:
+            raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
+        Q, qv = _lib.rows(Q.detach())
+        K, kv = _lib.rows(K.detach())
+        V, vv = _lib.rows(V.detach())
+        beta, bv = _lib.rows(beta.detach())
+        need_grad = any(ctx.needs_input_grad[:4])
+        chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
+        out = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
+        vdiff = ckpt = None
+        if need_grad:
+            vdiff = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
+            ckpt = torch.empty((N, H, _nchunk(L, chunk), E, M), device=Q.device, dtype=torch.float32)
+        with torch.cuda.device(Q.device):
+            rc = _lib.lib().fwp_delta_fwd(
+                qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out),
+                _lib.ptr(vdiff) if need_grad else None, _lib.ptr(ckpt) if need_grad else None,
+                N, H, L, E, M, chunk, _lib.stream_of(Q))
+        _lib.check(rc, "fwp_delta_fwd")
+        if need_grad:
+            ctx.save_for_backward(Q, K, beta, vdiff, ckpt)
+            ctx.dims = (N, H, L, E, M, chunk)
+        ctx.set_materialize_grads(False)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if grad_out is None:
+            return None, None, None, None, None
+        Q, K, beta, vdiff, ckpt = ctx.saved_tensors
+        N, H, L, E, M, chunk = ctx.dims
+        _, qv = _lib.rows(Q)
+        _, kv = _lib.rows(K)
+        _, bv = _lib.rows(beta)
+        grad_out, gv_ = _lib.rows(grad_out)
+        grad_Q = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
+        grad_K = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
+        grad_V = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
+        grad_beta = torch.empty((N, H, L, 1), device=Q.device, dtype=torch.float32)
+        with torch.cuda.device(Q.device):
+            rc = _lib.lib().fwp_delta_bwd(
+                qv, kv, bv, _lib.ptr(vdiff), gv_, _lib.ptr(ckpt), _lib.ptr(grad_Q),
+                _lib.ptr(grad_K), _lib.ptr(grad_V), _lib.ptr(grad_beta), N, H, L, E, M, chunk,
+                _lib.stream_of(Q))
+        _lib.check(rc, "fwp_delta_bwd")
+        return grad_Q, grad_K, grad_V, grad_beta, None
+
+
+fast_weight_delta = DeltaFastWeight.apply

@@ -1,0 +1,95 @@
+"""Recurrent Delta Net update with tanh feedback: drop-in for the reference's
+``rec_update_fwm_tanh`` package (algorithmic/rec_update_fwm_tanh/__init__.py:31-139)."""
+import torch
+
+from . import _lib
+from .fast_weight import _nchunk
+
+
+class FastWeightRecUpdateTanh(torch.autograd.Function):
+    """``out = rec_update_fwm_tanh(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0)``.
+
+    qx, kx, vx ``[N,H,L,D]`` and bx ``[N,H,L,1]`` are pre-activation; R_q, R_k, R_v
+    ``[1,H,D,D]`` (indexed ``[e_in][m_out]``) and r_b ``[1,H,1,D]`` feed
+    ``tanh(out_{t-1})`` back into them; softmax on q and k and sigmoid on beta are
+    applied inside.  W ``[N,H,D,D]`` and h0 ``[N,H,1,D]`` are in/out states.
+    Gradients flow to the first eight arguments.
+    """
+
+    @staticmethod
+    def forward(ctx, qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0):
+        _lib.require_device(qx)
+        N, H, L, E = qx.shape
+        M = vx.shape[-1]
+        # same preconditions as the reference (:52-56)
+        assert E == M, "Current kernel only support this case."
+        assert R_q.shape == (1, H, M, M), "Reshape/unsqueeze if needed."
+        assert R_k.shape == (1, H, M, M), "Reshape/unsqueeze if needed."
+        assert R_v.shape == (1, H, M, M), "Reshape/unsqueeze if needed."
+        assert r_b.shape == (1, H, 1, M), "Reshape/unsqueeze if needed."
+        assert kx.shape == (N, H, L, M) and vx.shape == (N, H, L, M) and bx.shape == (N, H, L, 1)
+        assert W.shape == (N, H, M, M) and h0.shape == (N, H, 1, M)
+        for name, t in (("W", W), ("h0", h0)):
+            if not t.is_contiguous() or t.dtype != torch.float32:
+                raise _lib.FwpError(f"{name} must be a contiguous fp32 tensor")
+        D = M
+        qx, qv = _lib.rows(qx.detach())
+        kx, kv = _lib.rows(kx.detach())
+        vx, vv = _lib.rows(vx.detach())
+        bx, bv = _lib.rows(bx.detach())
+        Rq, Rk, Rv, rb = (t.detach().contiguous().float() for t in (R_q, R_k, R_v, r_b))
+        need_grad = any(ctx.needs_input_grad)
+        chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
+        dev = qx.device
+        out = torch.empty((N, H, L, D), device=dev, dtype=torch.float32)
+        saved = [None] * 5
+        h_init = None
+        if need_grad:
+            h_init = h0.detach().clone()
+            saved = [torch.empty((N, H, L, D), device=dev, dtype=torch.float32),   # q after softmax
+                     torch.empty((N, H, L, D), device=dev, dtype=torch.float32),   # k after softmax
+                     torch.empty((N, H, L), device=dev, dtype=torch.float32),      # beta after sigmoid
+                     torch.empty((N, H, L, D), device=dev, dtype=torch.float32),   # v - v_old
+                     torch.empty((N, H, _nchunk(L, chunk), D, D), device=dev, dtype=torch.float32)]
+        with torch.cuda.device(dev):
+            rc = _lib.lib().fwp_rec_fwd(
+                qv, kv, vv, bv, _lib.ptr(Rq), _lib.ptr(Rk), _lib.ptr(Rv), _lib.ptr(rb),
+                _lib.ptr(W), _lib.ptr(h0), _lib.ptr(out),
+                *[(_lib.ptr(t) if t is not None else None) for t in saved],
+                N, H, L, D, chunk, _lib.stream_of(qx))
+        _lib.check(rc, "fwp_rec_fwd")
+        if need_grad:
+            ctx.save_for_backward(out, h_init, Rq, Rk, Rv, rb, *saved)
+            ctx.dims = (N, H, L, D, chunk)
+        ctx.set_materialize_grads(False)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        if grad_out is None:
+            return (None,) * 10
+        out, h_init, Rq, Rk, Rv, rb, q_act, k_act, beta_act, vdiff, ckpt = ctx.saved_tensors
+        N, H, L, D, chunk = ctx.dims
+        grad_out, gv_ = _lib.rows(grad_out)
+        dev = out.device
+        grad_qx, grad_kx, grad_vx = (torch.empty((N, H, L, D), device=dev, dtype=torch.float32)
+                                     for _ in range(3))
+        grad_bx = torch.empty((N, H, L, 1), device=dev, dtype=torch.float32)
+        grad_R_q, grad_R_k, grad_R_v = (torch.empty((1, H, D, D), device=dev, dtype=torch.float32)
+                                        for _ in range(3))
+        grad_r_b = torch.empty((1, H, 1, D), device=dev, dtype=torch.float32)
+        workspace = torch.empty((N, H, 3 * D * D + D), device=dev, dtype=torch.float32)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().fwp_rec_bwd(
+                _lib.ptr(q_act), _lib.ptr(k_act), _lib.ptr(beta_act), _lib.ptr(vdiff),
+                _lib.ptr(out), _lib.ptr(h_init), gv_, _lib.ptr(Rq), _lib.ptr(Rk), _lib.ptr(Rv),
+                _lib.ptr(rb), _lib.ptr(ckpt), _lib.ptr(grad_qx), _lib.ptr(grad_kx),
+                _lib.ptr(grad_vx), _lib.ptr(grad_bx), _lib.ptr(grad_R_q), _lib.ptr(grad_R_k),
+                _lib.ptr(grad_R_v), _lib.ptr(grad_r_b), _lib.ptr(workspace),
+                N, H, L, D, chunk, _lib.stream_of(out))
+        _lib.check(rc, "fwp_rec_bwd")
+        return (grad_qx, grad_kx, grad_vx, grad_bx,
+                grad_R_q, grad_R_k, grad_R_v, grad_r_b, None, None)
+
+
+rec_update_fwm_tanh = FastWeightRecUpdateTanh.apply

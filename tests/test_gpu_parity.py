@@ -1,0 +1,149 @@
+"""GPU parity: the HIP operators (through the autograd Functions, i.e. through the
+C ABI) against the float64 CPU oracle on the same seeded inputs.
+
+Tolerance (fp32, stated by the task): |hip - oracle| <= 1e-4 + 1e-3 * |oracle|
+elementwise, for outputs, final states and every gradient.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import delta_inputs, rec_inputs, rnn_inputs, within, max_abs
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 1e-4, 1e-3
+
+
+def dev(x, grad=False):
+    t = torch.from_numpy(np.asarray(x, np.float32)).to("cuda")
+    return t.requires_grad_(True) if grad else t
+
+
+def check(name, got, want):
+    got = got.detach().cpu().numpy()
+    assert got.shape == want.shape, (name, got.shape, want.shape)
+    assert np.all(np.isfinite(got)), name
+    assert within(got, want, ATOL, RTOL), f"{name}: max abs err {max_abs(got, want):.3e}"
+
+
+DELTA_SHAPES = [
+    (2, 2, 64, 16, 16, False),    # the CPU-runnable configuration of the benchmark list
+    (3, 5, 11, 64, 64, False),    # shape of the reference self test
+    (2, 3, 130, 16, 16, True),    # ragged tail chunk, carried-in state
+    (2, 2, 256, 32, 32, True),
+    (1, 2, 1, 16, 16, True),      # single step (RL-style stepping)
+    (2, 2, 37, 32, 97, True),     # E != M (Delta-Delta layer: M = 3D+1)
+    (1, 3, 70, 24, 8, False),     # E != M, M smaller
+    (1, 1, 20, 5, 3, True),       # odd sizes
+]
+
+
+@pytest.mark.parametrize("N,H,L,E,M,w0", DELTA_SHAPES)
+def test_delta(fwp, N, H, L, E, M, w0):
+    q, k, v, beta, W0, go = delta_inputs(100 + L + E, N, H, L, E, M, w0=w0)
+    tq, tk, tv, tb = (dev(x, True) for x in (q, k, v, beta))
+    W = dev(W0)
+    out = fwp.fast_weight_delta(tq, tk, tv, tb, W)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("q k v beta".split(), (tq, tk, tv, tb), oracle.delta_bwd(q, k, v, beta, W0, go)):
+        check("grad_" + name, t.grad, r)
+    check("W after backward", W, ref_W)     # backward does not rewind the caller's state
+
+
+def test_delta_strided_views_and_segments(fwp):
+    # inputs as the layers pass them: [L,N,H,*] storage permuted to [N,H,L,*], and a carried state
+    N, H, L, D = 2, 3, 48, 16
+    q, k, v, beta, W0, go = delta_inputs(7, N, H, L, D, D, w0=True)
+    def lnh(x):
+        return dev(np.ascontiguousarray(x.transpose(2, 0, 1, 3))).permute(1, 2, 0, 3)
+    tq, tk, tv, tb, tgo = lnh(q), lnh(k), lnh(v), lnh(beta), lnh(go)
+    for t in (tq, tk, tv, tb):
+        t.requires_grad_(True)
+    assert not tq.is_contiguous()
+    W = dev(W0)
+    a, b = slice(0, 20), slice(20, L)
+    o1 = fwp.fast_weight_delta(tq[:, :, a], tk[:, :, a], tv[:, :, a], tb[:, :, a], W)
+    o2 = fwp.fast_weight_delta(tq[:, :, b], tk[:, :, b], tv[:, :, b], tb[:, :, b], W)
+    out = torch.cat([o1, o2], dim=2)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    # gradients of the first segment alone (the carried state is detached, as in the reference)
+    o1.backward(tgo[:, :, a])
+    refs = oracle.delta_bwd(q[:, :, a], k[:, :, a], v[:, :, a], beta[:, :, a], W0, go[:, :, a])
+    check("grad_q", tq.grad[:, :, a], refs[0])
+    check("grad_beta", tb.grad[:, :, a], refs[3])
+
+
+def test_delta_no_grad_path(fwp):
+    q, k, v, beta, W0, _ = delta_inputs(8, 2, 2, 40, 16, 16)
+    with torch.no_grad():
+        W = dev(W0)
+        out = fwp.fast_weight_delta(dev(q), dev(k), dev(v), dev(beta), W)
+    check("out", out, oracle.delta_fwd(q, k, v, beta, W0)[0])
+
+
+RNN_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 64, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
+              (2, 3, 77, 8, True), (1, 1, 19, 5, True)]
+
+
+@pytest.mark.parametrize("N,H,L,D,w0", RNN_SHAPES)
+def test_rnn(fwp, N, H, L, D, w0):
+    z, k, v, W0, beta, h0, go = rnn_inputs(200 + L + D, N, H, L, D, w0=w0)
+    tz, tk, tv, tb = (dev(x, True) for x in (z, k, v, beta))
+    W, h = dev(W0), dev(h0)
+    out = fwp.fast_rnn_v2(tz, tk, tv, W, tb, h)
+    ref_out, ref_W, ref_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    check("h", h, ref_h)
+    out.backward(dev(go))
+    for name, t, r in zip("z k v beta".split(), (tz, tk, tv, tb), oracle.rnn_bwd(z, k, v, W0, beta, h0, go)):
+        check("grad_" + name, t.grad, r)
+
+
+REC_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 32, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
+              (2, 3, 77, 8, True), (1, 1, 19, 5, True), (1, 2, 30, 64, False)]
+
+
+@pytest.mark.parametrize("N,H,L,D,w0", REC_SHAPES)
+def test_rec(fwp, N, H, L, D, w0):
+    *x, go = rec_inputs(300 + L + D, N, H, L, D, w0=w0)
+    ts = [dev(a, True) for a in x[:8]]
+    W, h = dev(x[8]), dev(x[9])
+    out = fwp.rec_update_fwm_tanh(*ts, W, h)
+    ref_out, ref_W, ref_h = oracle.rec_fwd(*x)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    check("h", h, ref_h)
+    out.backward(dev(go))
+    names = "qx kx vx bx R_q R_k R_v r_b".split()
+    for name, t, r in zip(names, ts, oracle.rec_bwd(*x, go)):
+        check("grad_" + name, t.grad, r)
+
+
+def test_deterministic(fwp):
+    *x, go = rec_inputs(9, 4, 2, 50, 32)
+    res = []
+    for _ in range(2):
+        ts = [dev(a, True) for a in x[:8]]
+        out = fwp.rec_update_fwm_tanh(*ts, dev(x[8]), dev(x[9]))
+        out.backward(dev(go))
+        res.append([out.detach().clone()] + [t.grad.clone() for t in ts])
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+
+
+def test_rejects_cpu_tensors_and_bad_shapes(fwp):
+    q, k, v, beta, W0, _ = delta_inputs(1, 1, 1, 4, 4, 4)
+    cpu = [torch.from_numpy(a.astype(np.float32)) for a in (q, k, v, beta, W0)]
+    with pytest.raises(RuntimeError):
+        fwp.fast_weight_delta(*cpu)
+    with pytest.raises(RuntimeError):
+        fwp.fast_weight_delta(dev(q), dev(k[:, :, :3]), dev(v), dev(beta), dev(W0))
+    with pytest.raises(AssertionError):
+        fwp.fast_rnn_v2(dev(v), dev(k), dev(v), dev(W0), dev(beta), dev(v[:, :, :1, :3]))
