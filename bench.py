@@ -1,0 +1,289 @@
+#!/usr/bin/env python3
+"""Benchmark of the fast-weight update operators on one MI355X.
+
+A step is one forward + backward of the operator (through its autograd
+Function, allocations included) over one synthetic batch that is already
+resident in HBM.  Default workload: the delta rule at the LM-small shape
+B=96, H=8, T=256, D=16 (fp32).  Prints ONE JSON line.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload delta|rnn|rec]
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+METRIC = "fast-weight update tokens/s (fwd+bwd), % of FP32-VALU roofline, 1 GPU"
+PEAK_VALU = 157.3e12     # MI355X fp32 vector peak (packed), FLOP/s
+PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
+
+# name -> (B, H, T, D, algorithmic flops per token-head = c*D^2, fwd bytes, bwd bytes per token-head)
+WORKLOADS = {
+    "delta": dict(B=96, H=8, T=256, D=16, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
+                  bwd_bytes=lambda D: (7 * D + 2) * 4,
+                  label="delta-rule fast_weight fwd+bwd, B=96 H=8 T=256 D=16, fp32"),
+    "rnn": dict(B=64, H=8, T=256, D=32, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
+                bwd_bytes=lambda D: (8 * D + 2) * 4,
+                label="Delta RNN fast_rnn_v2 fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
+    "rec": dict(B=64, H=8, T=256, D=32, flop_c=38, fwd_bytes=lambda D: (4 * D + 1) * 4,
+                bwd_bytes=lambda D: (8 * D + 2) * 4,
+                label="Recurrent Delta Net rec_update_fwm_tanh fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
+}
+
+
+def make_inputs(name, w):
+    import numpy as np
+    from helpers import delta_inputs, rec_inputs, rnn_inputs
+    B, H, T, D = w["B"], w["H"], w["T"], w["D"]
+    if name == "delta":
+        return delta_inputs(0, B, H, T, D, D, dtype=np.float32)
+    if name == "rnn":
+        return rnn_inputs(0, B, H, T, D, dtype=np.float32)
+    return rec_inputs(0, B, H, T, D, dtype=np.float32)
+
+
+def gpu_step_fn(name, pkg, arrays):
+    """Returns (step, n_diff) where step() runs one fwd+bwd on the GPU."""
+    import torch
+    dev = [torch.from_numpy(a).to("cuda:0") for a in arrays]
+    go = dev[-1]
+    if name == "delta":
+        q, k, v, beta, W0 = dev[:5]
+        diff = [t.requires_grad_(True) for t in (q, k, v, beta)]
+        W = W0.clone()
+
+        def step():
+            W.copy_(W0)
+            out = pkg.fast_weight_delta(*diff, W)
+            torch.autograd.backward(out, go, inputs=diff)
+            return out
+    elif name == "rnn":
+        z, k, v, W0, beta, h0 = dev[:6]
+        diff = [t.requires_grad_(True) for t in (z, k, v, beta)]
+        W, h = W0.clone(), h0.clone()
+
+        def step():
+            W.copy_(W0)
+            h.copy_(h0)
+            out = pkg.fast_rnn_v2(diff[0], diff[1], diff[2], W, diff[3], h)
+            torch.autograd.backward(out, go, inputs=diff)
+            return out
+    else:
+        diff = [t.requires_grad_(True) for t in dev[:8]]
+        W0, h0 = dev[8], dev[9]
+        W, h = W0.clone(), h0.clone()
+
+        def step():
+            W.copy_(W0)
+            h.copy_(h0)
+            out = pkg.rec_update_fwm_tanh(*diff, W, h)
+            torch.autograd.backward(out, go, inputs=diff)
+            return out
+    return step, diff
+
+
+def kernel_times(name, pkg, arrays, iters):
+    """Average duration (s) of the forward and of the backward launch, timed with HIP
+    events on the stream the kernels are launched on (direct C-ABI calls, buffers preallocated)."""
+    import torch
+    L = pkg._lib
+    lib = L.lib()
+    dev = [torch.from_numpy(a).to("cuda:0") for a in arrays]
+    go = dev[-1]
+    stream = L.stream_of(go)
+    chunk = L.query(L.Q_DEFAULT_CHUNK)
+    f32 = dict(device="cuda:0", dtype=torch.float32)
+
+    def view(t):
+        return L.View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+
+    if name == "delta":
+        q, k, v, beta, W0 = dev[:5]
+        N, H, T, E = q.shape
+        M = v.shape[-1]
+        nch = (T + chunk - 1) // chunk
+        W = W0.clone()
+        out, vdiff = torch.empty_like(v), torch.empty_like(v)
+        ckpt = torch.empty((N, H, nch, E, M), **f32)
+        gq, gk, gv, gb = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(beta)
+
+        def fwd():
+            return lib.fwp_delta_fwd(view(q), view(k), view(v), view(beta), L.ptr(W), L.ptr(out), L.ptr(vdiff),
+                                     L.ptr(ckpt), N, H, T, E, M, chunk, stream)
+
+        def bwd():
+            return lib.fwp_delta_bwd(view(q), view(k), view(beta), L.ptr(vdiff), view(go), L.ptr(ckpt), L.ptr(gq),
+                                     L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, E, M, chunk, stream)
+        reset = lambda: W.copy_(W0)
+    elif name == "rnn":
+        z, k, v, W0, beta, h0 = dev[:6]
+        N, H, T, D = z.shape
+        nch = (T + chunk - 1) // chunk
+        W, h = W0.clone(), h0.clone()
+        out, vdiff = torch.empty_like(v), torch.empty_like(v)
+        ckpt = torch.empty((N, H, nch, D, D), **f32)
+        gz, gk, gv, gb = torch.empty_like(z), torch.empty_like(k), torch.empty_like(v), torch.empty_like(beta)
+
+        def fwd():
+            return lib.fwp_rnn_fwd(view(z), view(k), view(v), view(beta), L.ptr(W), L.ptr(h), L.ptr(out),
+                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream)
+
+        def bwd():
+            return lib.fwp_rnn_bwd(view(k), view(beta), L.ptr(vdiff), L.ptr(out), L.ptr(h0), view(go), L.ptr(ckpt),
+                                   L.ptr(gz), L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, D, chunk, stream)
+
+        def reset():
+            W.copy_(W0)
+            h.copy_(h0)
+    else:
+        qx, kx, vx, bx, Rq, Rk, Rv, rb, W0, h0 = dev[:10]
+        N, H, T, D = qx.shape
+        nch = (T + chunk - 1) // chunk
+        W, h = W0.clone(), h0.clone()
+        out, vdiff, qa, ka = (torch.empty_like(vx) for _ in range(4))
+        ba = torch.empty((N, H, T), **f32)
+        ckpt = torch.empty((N, H, nch, D, D), **f32)
+        g = [torch.empty_like(t) for t in (qx, kx, vx, bx, Rq, Rk, Rv, rb)]
+        ws = torch.empty((N, H, 3 * D * D + D), **f32)
+
+        def fwd():
+            return lib.fwp_rec_fwd(view(qx), view(kx), view(vx), view(bx), L.ptr(Rq), L.ptr(Rk), L.ptr(Rv),
+                                   L.ptr(rb), L.ptr(W), L.ptr(h), L.ptr(out), L.ptr(qa), L.ptr(ka), L.ptr(ba),
+                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream)
+
+        def bwd():
+            return lib.fwp_rec_bwd(L.ptr(qa), L.ptr(ka), L.ptr(ba), L.ptr(vdiff), L.ptr(out), L.ptr(h0), view(go),
+                                   L.ptr(Rq), L.ptr(Rk), L.ptr(Rv), L.ptr(rb), L.ptr(ckpt), *[L.ptr(t) for t in g],
+                                   L.ptr(ws), N, H, T, D, chunk, stream)
+
+        def reset():
+            W.copy_(W0)
+            h.copy_(h0)
+
+    def timed(fn, pre=None):
+        for _ in range(3):
+            if pre:
+                pre()
+            L.check(fn(), "warm-up launch")
+        torch.cuda.synchronize()
+        total = 0.0
+        for _ in range(iters):
+            if pre:
+                pre()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = fn()
+            e1.record()
+            L.check(rc, "timed launch")
+            e1.synchronize()
+            total += e0.elapsed_time(e1) * 1e-3
+        return total / iters
+
+    t_f = timed(fwd, reset)
+    reset()
+    L.check(fwd(), "forward before backward timing")
+    t_b = timed(bwd)
+    return t_f, t_b
+
+
+def cpu_baseline(name, arrays, w, reps):
+    """The reference's CPU path (its PyTorch step loop + autograd), restated, on the host cores."""
+    import torch
+    from oracle import torch_loop
+    cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        cores = min(cores, int(env))
+    torch.set_num_threads(cores)
+    ts = [torch.from_numpy(a) for a in arrays]
+    go = ts[-1]
+    if name == "delta":
+        loop, inputs, idx = torch_loop.delta_loop, ts[:5], [0, 1, 2, 3]
+    elif name == "rnn":
+        loop, inputs, idx = torch_loop.rnn_v2_loop, ts[:6], [0, 1, 2, 4]
+    else:
+        loop, inputs, idx = torch_loop.rec_update_loop, ts[:10], list(range(8))
+    torch_loop.grads(loop, inputs, idx, go)     # warm-up
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        torch_loop.grads(loop, inputs, idx, go)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    tokens = w["B"] * w["T"]
+    return {"value": tokens / med, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"full batch of the workload, PyTorch step loop fwd+bwd on the host, median of {reps} runs "
+                      f"({med * 1e3:.0f} ms each)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="delta")
+    ap.add_argument("--cpu-reps", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (sequences are independent; "
+                 "more GPUs would just split the batch). Use --gpus 1.")
+
+    import torch
+    from __graft_entry__ import package
+    pkg = package()
+    pkg._lib.lib()                       # fails loudly if the HIP library is not built
+    name = args.workload
+    w = WORKLOADS[name]
+    arrays = make_inputs(name, w)
+    B, H, T, D = w["B"], w["H"], w["T"], w["D"]
+    tokens = B * T
+    token_heads = tokens * H
+
+    step, _ = gpu_step_fn(name, pkg, arrays)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms = elapsed / args.steps * 1e3
+    value = tokens / (elapsed / args.steps)
+
+    t_f, t_b = kernel_times(name, pkg, arrays, max(20, min(args.steps, 100)))
+    fwd_bytes = w["fwd_bytes"](D) * token_heads
+    bwd_bytes = w["bwd_bytes"](D) * token_heads
+    dom = "bwd" if t_b >= t_f else "fwd"
+    dom_bytes, dom_t = (bwd_bytes, t_b) if dom == "bwd" else (fwd_bytes, t_f)
+    flops = w["flop_c"] * D * D * token_heads
+    kernel_s = t_f + t_b
+    result = {
+        "metric": METRIC, "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w["label"], "B": B, "H": H, "T": T, "D": D},
+        "roofline": {"bound": "hbm", "kernel": f"{name} {dom}", "achieved": dom_bytes / dom_t / 1e9,
+                     "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": dom_bytes / dom_t / PEAK_HBM,
+                     "traffic": None},
+        "kernels": {"fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
+                    "fwd_GBps": fwd_bytes / t_f / 1e9, "bwd_GBps": bwd_bytes / t_b / 1e9,
+                    "kernel_only_tokens_per_s": tokens / kernel_s,
+                    "valu_frac_of_157.3TF": flops / kernel_s / PEAK_VALU,
+                    "hbm_frac_of_8TBps": (fwd_bytes + bwd_bytes) / kernel_s / PEAK_HBM,
+                    "step_valu_frac_of_157.3TF": flops / (ms * 1e-3) / PEAK_VALU},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(name, arrays, w, args.cpu_reps)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()
