@@ -10,6 +10,7 @@ using namespace fwp;
 namespace {
 
 bool bad_view(const fwp_view &v) { return v.ptr == nullptr; }
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int check_dims(int N, int H, int L, int E, int M, int chunk) {
     if (N < 1 || H < 1 || L < 1 || E < 1 || M < 1) return FWP_E_SHAPE;
@@ -63,6 +64,10 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
+        aligned16(vdiff) && aligned16(ckpt))
+        return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
+                             (hipStream_t)stream);
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
                              (hipStream_t)stream);
 }
@@ -74,6 +79,10 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         !gq || !gk || !gv || !gbeta)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
+        aligned16(vdiff) && aligned16(ckpt))
+        return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
+                             chunk, (hipStream_t)stream);
     return generic_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
                              chunk, (hipStream_t)stream);
 }

@@ -41,6 +41,15 @@ int generic_rec_bwd(const float *q_act, const float *k_act, const float *beta_ac
 int reduce_rec_param_grads(const float *workspace, float *gRq, float *gRk, float *gRv,
                            float *grb, int N, int H, int D, hipStream_t s);
 
+// Register-state kernels (one wave per sequence): E = M = D in {16, 32}, 16-byte aligned rows.
+bool reg_view_ok(const fwp_view &v);
+bool reg_delta_supported(int E, int M);
+int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                  float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
+                  const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
+                  int L, int D, int chunk, hipStream_t s);
+
 // Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 

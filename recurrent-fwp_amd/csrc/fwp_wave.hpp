@@ -1,0 +1,69 @@
+// Wave-level building blocks of the register-state kernels (gfx950, wave64).
+//
+// A sequence is owned by ONE wave.  The D x D state lives in VGPRs: lane
+// l = i*S + s (i in [0,D), s in [0,S), D*S = 64) holds R = D/S elements of row or
+// column i.  Sums over the S lanes of a group are DPP quad permutes; sums over the
+// D groups are DPP row rotates plus two row swaps.
+#pragma once
+#include <hip/hip_runtime.h>
+
+namespace fwp {
+
+constexpr int kWave = 64;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp(float x) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+
+constexpr int kQuadXor1 = 0xB1;  // quad_perm:[1,0,3,2]
+constexpr int kQuadXor2 = 0x4E;  // quad_perm:[2,3,0,1]
+constexpr int kRowRor4 = 0x124;
+constexpr int kRowRor8 = 0x128;
+
+// Sum over the S adjacent lanes of a group; every lane of the group gets the sum.
+template <int S>
+__device__ __forceinline__ float group_sum(float x) {
+    static_assert(S == 1 || S == 2 || S == 4, "group of 1, 2 or 4 lanes");
+    if constexpr (S >= 2) x += dpp<kQuadXor1>(x);
+    if constexpr (S >= 4) x += dpp<kQuadXor2>(x);
+    return x;
+}
+
+// Exchange between the four 16-lane rows of the wave.  The compiler's builtins
+// for these two gfx950 instructions drop the second result, hence the asm.
+// After swap16: a = {r0,r0,r2,r2}, b = {r1,r1,r3,r3} for a = b = {r0,r1,r2,r3};
+// after swap32: a = {lo,lo}, b = {hi,hi}.
+__device__ __forceinline__ void swap16(float &a, float &b) {
+    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ void swap32(float &a, float &b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+
+struct OpSum {
+    __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
+};
+struct OpMax {
+    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+};
+
+// All-reduce over the D groups of a wave for a value that is already uniform
+// inside each group of S lanes (S*D = 64).  Every lane gets the result.
+template <int S, typename Op>
+__device__ __forceinline__ float across_groups(float x, Op op) {
+    static_assert(S == 1 || S == 2 || S == 4, "group of 1, 2 or 4 lanes");
+    if constexpr (S == 1) x = op(x, dpp<kQuadXor1>(x));
+    if constexpr (S <= 2) x = op(x, dpp<kQuadXor2>(x));
+    x = op(x, dpp<kRowRor4>(x));
+    x = op(x, dpp<kRowRor8>(x));
+    float y = x;
+    swap16(x, y);
+    x = op(x, y);
+    y = x;
+    swap32(x, y);
+    return op(x, y);
+}
+
+}  // namespace fwp
