@@ -1,26 +1,99 @@
 // Register-state kernels of the delta rule for E = M = D in {16, 32}.
 //
-// One wave64 per (n,h) sequence.  Forward keeps W by columns: lane (m, s) holds
-// W[s*R .. s*R+R-1][m], so v_old = W^T k and out = W^T q are R in-lane FMAs plus a
-// DPP sum over the S lanes of the column.  Backward keeps W by rows and G (the
-// gradient of the state) twice, by rows and by columns, so that every mat-vec of
-// the reverse step is in-lane as well; the only cross-lane traffic per step is the
-// S-lane DPP sums, one D-vector exchanged through LDS and one wave-wide sum.
-// q/k/v/beta (and grad_out, vdiff) are streamed through double-buffered LDS tiles
-// of kTile steps, fetched from HBM one tile ahead with 16-byte loads.
+// One wave64 per (n,h) sequence, the D x D state in VGPRs.  Lane l belongs to
+// group g = l / S (S = 64 / D lanes per group) and has sub-index s = l % S; a
+// group owns one column (forward) or one row (backward) of the state and each of
+// its lanes holds R = D / S entries of it.  Which entries is chosen so that the
+// operand vectors never have to be gathered: a D-vector x is held "periodically"
+// (lane l holds x[16*p + l % 16], p < D/16) and the entry a lane needs for its
+// j-th state register is the one that a DPP row rotation by S*j brings to it, so
+// every mat-vec and rank-1 update is a run of v_fmac_f32 with a rotating DPP
+// source operand.  Sums over the S lanes of a group are DPP quad permutes.
+//
+// Forward keeps W by columns.  Backward keeps W by rows and the gradient of the
+// state G twice, by rows and by columns, so that both G^T k and G u are in-lane;
+// per step the only other cross-lane traffic is one D-vector (the gradient of
+// v_old) permuted across groups, and the partial products of grad beta that are
+// summed once per tile.
+//
+// q/k/v/beta (grad_out, vdiff) stream through double-buffered LDS tiles of kTile
+// steps, fetched from HBM two tiles ahead with 16-byte loads; inside a tile the
+// operands of the next steps are read from LDS while the current step computes.
 #include "fwp_common.hpp"
 #include "fwp_wave.hpp"
+
+#include <utility>
 
 namespace fwp {
 namespace {
 
 template <int D>
 struct Geo {
-    static constexpr int S = kWave / D;                // lanes per row/column
-    static constexpr int R = D / S;                    // state elements per lane
+    static constexpr int S = kWave / D;                // lanes per group
+    static constexpr int NP = D / 16;                  // periodic registers per D-vector
+    static constexpr int NR = 16 / S;                  // rotations per periodic register
+    static constexpr int R = NP * NR;                  // state entries per lane (= D / S)
     static constexpr int NV4 = kTile * D / 4 / kWave;  // float4 per lane per tile tensor
-    static_assert(D * S == kWave && R % 4 == 0 && NV4 >= 1, "D must be 16 or 32");
+    static_assert(D * S == kWave && NV4 >= 1, "D must be 16 or 32");
 };
+
+// Index (row in forward, column in backward) of state register jj of lane `lane`.
+template <int D>
+__device__ __forceinline__ int reg_index(int lane, int jj) {
+    using G = Geo<D>;
+    const int pr = jj / G::NR, j = jj % G::NR;
+    const int mm = (lane % 16) / G::S, s = lane % G::S;
+    return 16 * pr + G::S * ((mm - j + G::NR) % G::NR) + s;
+}
+
+constexpr int kRowHalfMirror = 0x141;
+
+// acc + ror(x, ROT) * y, the rotation being inside the 16-lane row.  x must come
+// straight from an LDS/memory load (a DPP source written by a VALU instruction just
+// before would need wait states the compiler cannot see through the asm).
+template <int ROT>
+__device__ __forceinline__ float fmac_ror(float acc, float x, float y) {
+    if constexpr (ROT == 0) {
+        return fmaf(x, y, acc);
+    } else {
+        asm("v_fmac_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+            : "+v"(acc)
+            : "v"(x), "v"(y), "n"(ROT));
+        return acc;
+    }
+}
+
+template <int S, int... J>
+__device__ __forceinline__ float dot_rot1(const float *w, float x, float acc,
+                                          std::integer_sequence<int, J...>) {
+    ((acc = fmac_ror<S * J>(acc, x, w[J])), ...);
+    return acc;
+}
+template <int S, int... J>
+__device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
+                                           std::integer_sequence<int, J...>) {
+    ((w[J] = fmac_ror<S * J>(w[J], x, y)), ...);
+}
+
+// sum_jj w[jj] * x[index(jj)]  for a periodic vector x[NP]
+template <int D>
+__device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
+                                         float acc = 0.f) {
+    using G = Geo<D>;
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        acc = dot_rot1<G::S>(&w[p * G::NR], x[p], acc, std::make_integer_sequence<int, G::NR>{});
+    return acc;
+}
+// w[jj] += x[index(jj)] * y
+template <int D>
+__device__ __forceinline__ void rank1_rot(float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
+                                          float y) {
+    using G = Geo<D>;
+#pragma unroll
+    for (int p = 0; p < G::NP; p++)
+        rank1_rot1<G::S>(&w[p * G::NR], x[p], y, std::make_integer_sequence<int, G::NR>{});
+}
 
 // One tile of one [.,D] tensor on its way from HBM to LDS.
 template <int D>
@@ -48,54 +121,63 @@ struct TileRegs {
     }
 };
 
-template <int R>
-__device__ __forceinline__ void lds_vec(float (&dst)[R], const float *src) {
+// Row-wise dot products of two tiles held in registers: lane gets (a_row . b_row)
+// of row (lane + 64 i) / (D/4) in out[i].
+template <int D>
+__device__ __forceinline__ void tile_row_dots(const TileRegs<D> &a, const TileRegs<D> &b,
+                                              float (&out)[Geo<D>::NV4]) {
 #pragma unroll
-    for (int j = 0; j < R; j += 4) {
-        const float4 x = *reinterpret_cast<const float4 *>(src + j);
-        dst[j] = x.x; dst[j + 1] = x.y; dst[j + 2] = x.z; dst[j + 3] = x.w;
+    for (int i = 0; i < Geo<D>::NV4; i++) {
+        float x = a.r[i].x * b.r[i].x;
+        x = fmaf(a.r[i].y, b.r[i].y, x);
+        x = fmaf(a.r[i].z, b.r[i].z, x);
+        x = fmaf(a.r[i].w, b.r[i].w, x);
+        x = group_sum<4>(x);
+        if constexpr (D == 32) x += dpp<kRowHalfMirror>(x);
+        out[i] = x;
     }
-}
-
-template <int R>
-__device__ __forceinline__ float dot(const float (&a)[R], const float (&b)[R]) {
-    float acc = a[0] * b[0];
-#pragma unroll
-    for (int j = 1; j < R; j++) acc = fmaf(a[j], b[j], acc);
-    return acc;
-}
-
-template <int R>
-__device__ __forceinline__ void axpy(float (&y)[R], float a, const float (&x)[R]) {
-#pragma unroll
-    for (int j = 0; j < R; j++) y[j] = fmaf(a, x[j], y[j]);
 }
 
 // ------------------------------------------------------------------ forward
 
 template <int D>
-__global__ __launch_bounds__(kWave) void k_delta_fwd_reg(fwp_view q, fwp_view k, fwp_view v,
+struct FwdOps {
+    float k[Geo<D>::NP], q[Geo<D>::NP], v, b, kq;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_view k, fwp_view v,
                                                          fwp_view beta, float *__restrict__ W,
                                                          float *__restrict__ out,
                                                          float *__restrict__ vdiff,
                                                          float *__restrict__ ckpt, int H, int L,
-                                                         int chunk, int nchunk) {
+                                                         int chunk, int nchunk, int nseq) {
     using G = Geo<D>;
-    constexpr int S = G::S, R = G::R;
-    __shared__ __align__(16) float sq[2][kTile * D];
-    __shared__ __align__(16) float sk[2][kTile * D];
-    __shared__ __align__(16) float sv[2][kTile * D];
-    __shared__ float sb[2][kTile];
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sq_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sv_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float skq_[WPB][2][kTile];
 
-    const int lane = threadIdx.x, col = lane / S, sl = lane % S;
-    const int64_t seq = blockIdx.x;
-    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sq = sq_[wave];
+    auto &sk = sk_[wave];
+    auto &sv = sv_[wave];
+    auto &sb = sb_[wave];
+    auto &skq = skq_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
                 *bb = row(beta, n, h, 0);
 
-    float Wc[R];  // W[sl*R + j][col]
+    float Wc[R];  // W[reg_index(jj)][col]
 #pragma unroll
-    for (int j = 0; j < R; j++) Wc[j] = W[(seq * D + sl * R + j) * D + col];
+    for (int jj = 0; jj < R; jj++) Wc[jj] = W[(seq * D + reg_index<D>(lane, jj)) * D + col];
 
     TileRegs<D> pq, pk, pv;
     float pb = 0.f;
@@ -110,83 +192,125 @@ __global__ __launch_bounds__(kWave) void k_delta_fwd_reg(fwp_view q, fwp_view k,
         pk.commit(sk[buf], lane);
         pv.commit(sv[buf], lane);
         if (lane < kTile) sb[buf][lane] = pb;
+        float kq[NV4];
+        tile_row_dots<D>(pk, pq, kq);
+#pragma unroll
+        for (int i = 0; i < NV4; i++) skq[buf][(lane + kWave * i) / (D / 4)] = kq[i];
     };
 
     // lanes with odd s store vdiff, the others out (same value from every lane that shares an address)
     const bool store_d = (vdiff != nullptr) && (sl & 1);
     float *dst = (store_d ? vdiff : out) + seq * L * D + col;
 
-    auto step = [&](int buf, int tt, float *o_ptr) {
-        float kk[R], qq[R];
-        lds_vec<R>(kk, &sk[buf][tt * D + sl * R]);
-        lds_vec<R>(qq, &sq[buf][tt * D + sl * R]);
-        const float vm = sv[buf][tt * D + col];
-        const float b = sb[buf][tt];
-        const float d = vm - group_sum<S>(dot<R>(Wc, kk));
-        axpy<R>(Wc, b * d, kk);
-        const float o = group_sum<S>(dot<R>(Wc, qq));
-        *o_ptr = store_d ? d : o;
+    auto load_ops = [&](FwdOps<D> &o, int buf, int tt) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.k[p] = sk[buf][tt * D + 16 * p + per];
+            o.q[p] = sq[buf][tt * D + 16 * p + per];
+        }
+        o.v = sv[buf][tt * D + col];
+        o.b = sb[buf][tt];
+        o.kq = skq[buf][tt];
+    };
+    // out_t = W_t^T q = W_{t-1}^T q + u (k.q): both mat-vecs read the old state
+    auto compute = [&](const FwdOps<D> &o, float *o_ptr) {
+        const float p_old = group_sum<S>(dot_rot<D>(Wc, o.k));
+        const float p_out = group_sum<S>(dot_rot<D>(Wc, o.q));
+        const float d = o.v - p_old;
+        const float u = o.b * d;
+        rank1_rot<D>(Wc, o.k, u);
+        *o_ptr = store_d ? d : fmaf(u, o.kq, p_out);
     };
 
     const int ntile = (L + kTile - 1) / kTile;
     fetch(0);
     commit(0);
-    __syncthreads();
+    if (ntile > 1) fetch(kTile);
+    FwdOps<D> ring[RING];
+#pragma unroll
+    for (int p = 0; p < PF; p++) load_ops(ring[p], 0, p);
+
     for (int it = 0; it < ntile; it++) {
         const int buf = it & 1, t0 = it * kTile;
         const int nst = min(kTile, L - t0);
-        if (it + 1 < ntile) fetch(t0 + kTile);
+        if (it + 1 < ntile) commit(buf ^ 1);
+        if (it + 2 < ntile) fetch(t0 + 2 * kTile);
         float *tile_dst = dst + (int64_t)t0 * D;
         if (nst == kTile) {
 #pragma unroll
-            for (int tt = 0; tt < kTile; tt++) step(buf, tt, tile_dst + tt * D);
-        } else {
-            for (int tt = 0; tt < nst; tt++) step(buf, tt, tile_dst + tt * D);
+            for (int tt = 0; tt < kTile; tt++) {
+                const int nt = tt + PF;
+                if (nt < kTile) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[nt % RING], buf ^ 1, nt - kTile);
+                compute(ring[tt % RING], tile_dst + tt * D);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                FwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tile_dst + tt * D);
+            }
         }
         const int t_end = t0 + nst;
         if (ckpt && (t_end % chunk == 0 || t_end == L)) {
             float *c = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
 #pragma unroll
-            for (int j = 0; j < R; j++) c[(sl * R + j) * D + col] = Wc[j];
+            for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[jj];
         }
-        if (it + 1 < ntile) commit(buf ^ 1);
-        __syncthreads();
     }
 #pragma unroll
-    for (int j = 0; j < R; j++) W[(seq * D + sl * R + j) * D + col] = Wc[j];
+    for (int jj = 0; jj < R; jj++) W[(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[jj];
 }
 
 // ----------------------------------------------------------------- backward
 
 template <int D>
-__global__ __launch_bounds__(kWave) void k_delta_bwd_reg(fwp_view q, fwp_view k, fwp_view beta,
+struct BwdOps {
+    float q[Geo<D>::NP], k[Geo<D>::NP], go[Geo<D>::NP], u[Geo<D>::NP];
+    float q_i, k_i, go_i, d_i, b;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_view k, fwp_view beta,
                                                          const float *__restrict__ vdiff,
                                                          fwp_view go, const float *__restrict__ ckpt,
                                                          float *__restrict__ gq,
                                                          float *__restrict__ gk,
                                                          float *__restrict__ gv,
                                                          float *__restrict__ gbeta, int H, int L,
-                                                         int chunk, int nchunk) {
+                                                         int chunk, int nchunk, int nseq) {
     using G = Geo<D>;
-    constexpr int S = G::S, R = G::R, NV4 = G::NV4;
-    __shared__ __align__(16) float sq[2][kTile * D];
-    __shared__ __align__(16) float sk[2][kTile * D];
-    __shared__ __align__(16) float sgo[2][kTile * D];
-    __shared__ __align__(16) float sd[2][kTile * D];
-    __shared__ __align__(16) float su[2][kTile * D];
-    __shared__ float sb[2][kTile];
-    __shared__ __align__(16) float sa[D];
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sq_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sgo_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sd_[WPB][2][kTile * D];
+    __shared__ __align__(16) float su_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float spd_[WPB][kTile * D];   // r_i * d_i per step, summed per tile
 
-    const int lane = threadIdx.x, i = lane / S, sl = lane % S;
-    const int64_t seq = blockIdx.x;
-    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sq = sq_[wave];
+    auto &sk = sk_[wave];
+    auto &sgo = sgo_[wave];
+    auto &sd = sd_[wave];
+    auto &su = su_[wave];
+    auto &sb = sb_[wave];
+    auto &spd = spd_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
                 *bb = row(beta, n, h, 0);
     const float *db = vdiff + seq * L * D;
 
-    float Wr[R], Gr[R], Gc[R], Wnext[R];  // W[i][sl*R+j], G[i][sl*R+j], G[sl*R+j][i]
+    // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
+    float Wr[R], Gr[R], Gc[R], Wnext[R];
 #pragma unroll
-    for (int j = 0; j < R; j++) Gr[j] = Gc[j] = Wr[j] = 0.f;
+    for (int jj = 0; jj < R; jj++) Gr[jj] = Gc[jj] = Wr[jj] = 0.f;
 
     TileRegs<D> pq, pk, pgo, pd, pu;
     float pb = 0.f;
@@ -214,73 +338,115 @@ __global__ __launch_bounds__(kWave) void k_delta_bwd_reg(fwp_view q, fwp_view k,
         if (lane < kTile) sb[buf][lane] = pb;
     };
     auto fetch_state = [&](int c) {
-        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D + sl * R;
+        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
 #pragma unroll
-        for (int j = 0; j < R; j += 4) {
-            const float4 x = *reinterpret_cast<const float4 *>(src + j);
-            Wnext[j] = x.x; Wnext[j + 1] = x.y; Wnext[j + 2] = x.z; Wnext[j + 3] = x.w;
-        }
+        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
     };
 
-    auto step = [&](int buf, int tt, int64_t row0) {
-        float q4[R], k4[R], go4[R], u4[R], a4[R];
-        const int o = tt * D;
-        lds_vec<R>(q4, &sq[buf][o + sl * R]);
-        lds_vec<R>(k4, &sk[buf][o + sl * R]);
-        lds_vec<R>(go4, &sgo[buf][o + sl * R]);
-        lds_vec<R>(u4, &su[buf][o + sl * R]);
-        const float q_i = sq[buf][o + i], k_i = sk[buf][o + i], go_i = sgo[buf][o + i],
-                    d_i = sd[buf][o + i], b = sb[buf][tt];
-        // G' = G + q (x) go, in both layouts
-        axpy<R>(Gr, q_i, go4);
-        axpy<R>(Gc, go_i, q4);
-        const float gq_i = group_sum<S>(dot<R>(Wr, go4));   // (W_t go)[i]
-        const float r_i = group_sum<S>(dot<R>(Gc, k4));     // (G'^T k)[i]
-        const float gv_i = b * r_i;
-        const float a_i = -gv_i;                            // gradient w.r.t. v_old
-        sa[i] = a_i;
-        const float gb = across_groups<S>(r_i * d_i, OpSum());
-        axpy<R>(Wr, -k_i, u4);                              // W_{t-1}
-        lds_vec<R>(a4, &sa[sl * R]);
-        float gk_i = dot<R>(Gr, u4);
+    // One store per step covers gq, gk and gv: lanes pick their output by s.
+    // S = 4: s=0 -> gq, s=1 -> gk, s=2,3 -> gv.   S = 2: s=0 -> gq, s=1 -> gk, and a second store for gv.
+    float *dst1 = (sl == 0 ? gq : (sl == 1 ? gk : gv)) + seq * L * D + i;
+    float *dst2 = gv + seq * L * D + i;
+    // source lane (as a byte address for ds_bpermute) of the periodic copy of a per-group value
+    int gather[NP];
 #pragma unroll
-        for (int j = 0; j < R; j++) gk_i = fmaf(Wr[j], a4[j], gk_i);
-        gk_i = group_sum<S>(gk_i);
-        axpy<R>(Gr, k_i, a4);
-        axpy<R>(Gc, a_i, k4);
-        if (sl == 0) {
-            (gq + row0 * D + i)[tt * D] = gq_i;
-            (gk + row0 * D + i)[tt * D] = gk_i;
-            (gv + row0 * D + i)[tt * D] = gv_i;
+    for (int p = 0; p < NP; p++) gather[p] = 4 * S * (16 * p + per);
+
+    auto load_ops = [&](BwdOps<D> &o, int buf, int tt) {
+        const int off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.q[p] = sq[buf][off + 16 * p + per];
+            o.k[p] = sk[buf][off + 16 * p + per];
+            o.go[p] = sgo[buf][off + 16 * p + per];
+            o.u[p] = su[buf][off + 16 * p + per];
         }
-        if (lane == 0) (gbeta + row0)[tt] = gb;
+        o.q_i = sq[buf][off + i];
+        o.k_i = sk[buf][off + i];
+        o.go_i = sgo[buf][off + i];
+        o.d_i = sd[buf][off + i];
+        o.b = sb[buf][tt];
+    };
+    auto compute = [&](const BwdOps<D> &o, int tt, int64_t tile_off) {
+        // G' = G + q (x) go (both layouts);  r = G'^T k
+        rank1_rot<D>(Gc, o.q, o.go_i);
+        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        const float gv_i = o.b * r_i;
+        const float a_i = -gv_i;                              // gradient w.r.t. v_old
+        float a[NP];
+#pragma unroll
+        for (int p = 0; p < NP; p++)
+            a[p] = __builtin_bit_cast(
+                float, __builtin_amdgcn_ds_bpermute(gather[p], __builtin_bit_cast(int, a_i)));
+        spd[tt * D + i] = r_i * o.d_i;
+        rank1_rot<D>(Gr, o.go, o.q_i);
+        const float gq_i = group_sum<S>(dot_rot<D>(Wr, o.go));   // (W_t go)[i]
+        rank1_rot<D>(Wr, o.u, -o.k_i);                            // W_{t-1}
+        rank1_rot<D>(Gc, o.k, a_i);
+        float gk_i = dot_rot<D>(Gr, o.u);                         // G' u + W_{t-1} a
+        gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
+        rank1_rot<D>(Gr, a, o.k_i);
+        if constexpr (S == 4) {
+            (dst1 + tile_off)[tt * D] = sl == 0 ? gq_i : (sl == 1 ? gk_i : gv_i);
+        } else {
+            (dst1 + tile_off)[tt * D] = sl == 0 ? gq_i : gk_i;
+            (dst2 + tile_off)[tt * D] = gv_i;
+        }
+    };
+    // gbeta of the tile's steps: sum spd[tt][:] over the D entries, four lanes per step
+    auto flush_gbeta = [&](int t0, int nst) {
+        const int tt = lane / 4, part = lane % 4;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < D / 4; j += 4) {
+            const float4 x = *reinterpret_cast<const float4 *>(&spd[tt * D + part * (D / 4) + j]);
+            acc += (x.x + x.y) + (x.z + x.w);
+        }
+        acc = group_sum<4>(acc);
+        if (tt < nst) gbeta[seq * L + t0 + tt] = acc;
     };
 
     const int ntile = (L + kTile - 1) / kTile;
     fetch((ntile - 1) * kTile);
     commit((ntile - 1) & 1);
     fetch_state(nchunk - 1);
-    __syncthreads();
+    if (ntile > 1) fetch((ntile - 2) * kTile);
+    BwdOps<D> ring[RING];
+    bool primed = false;
+
     for (int it = ntile - 1; it >= 0; it--) {
         const int buf = it & 1, t0 = it * kTile;
         const int nst = min(kTile, L - t0);
         const int t_end = t0 + nst;
         if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
 #pragma unroll
-            for (int j = 0; j < R; j++) Wr[j] = Wnext[j];
+            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
         }
-        if (it > 0) {
-            fetch(t0 - kTile);
-            if (t0 % chunk == 0) fetch_state(t0 / chunk - 1);
-        }
+        if (it >= 1) commit(buf ^ 1);
+        if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
+        if (it >= 2) fetch(t0 - 2 * kTile);
+        const int64_t tile_off = (int64_t)t0 * D;
         if (nst == kTile) {
+            if (!primed) {
 #pragma unroll
-            for (int tt = kTile - 1; tt >= 0; tt--) step(buf, tt, seq * L + t0);
-        } else {
-            for (int tt = nst - 1; tt >= 0; tt--) step(buf, tt, seq * L + t0);
+                for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
+                primed = true;
+            }
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                const int nt = tt - PF;
+                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
+                compute(ring[tt % RING], tt, tile_off);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                BwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt, tile_off);
+            }
         }
-        if (it > 0) commit(buf ^ 1);
-        __syncthreads();
+        flush_gbeta(t0, nst);
     }
 }
 
@@ -297,12 +463,13 @@ bool reg_delta_supported(int E, int M) { return E == M && (E == 16 || E == 32); 
 int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                   float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
+    const int nseq = N * H;
     if (D == 16)
-        hipLaunchKernelGGL(k_delta_fwd_reg<16>, dim3(N * H), dim3(kWave), 0, s, q, k, v, beta, W,
-                           out, vdiff, ckpt, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_fwd_reg<16, 4, 2, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, v, beta, W, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL(k_delta_fwd_reg<32>, dim3(N * H), dim3(kWave), 0, s, q, k, v, beta, W,
-                           out, vdiff, ckpt, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, v, beta, W, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
 
@@ -310,12 +477,13 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                   int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
+    const int nseq = N * H;
     if (D == 16)
-        hipLaunchKernelGGL(k_delta_bwd_reg<16>, dim3(N * H), dim3(kWave), 0, s, q, k, beta, vdiff,
-                           go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, beta, vdiff, go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL(k_delta_bwd_reg<32>, dim3(N * H), dim3(kWave), 0, s, q, k, beta, vdiff,
-                           go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
+                           q, k, beta, vdiff, go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
 
