@@ -59,9 +59,9 @@ def gpu_step_fn(name, pkg, arrays):
         W = W0.clone()
 
         def step():
-            W.copy_(W0)
+            W.zero_()                     # W0 = 0 for every step of the benchmark
             out = pkg.fast_weight_delta(*diff, W)
-            torch.autograd.backward(out, go, inputs=diff)
+            torch.autograd.grad(out, diff, go)
             return out
     elif name == "rnn":
         z, k, v, W0, beta, h0 = dev[:6]
@@ -69,10 +69,10 @@ def gpu_step_fn(name, pkg, arrays):
         W, h = W0.clone(), h0.clone()
 
         def step():
-            W.copy_(W0)
-            h.copy_(h0)
+            W.zero_()
+            h.zero_()
             out = pkg.fast_rnn_v2(diff[0], diff[1], diff[2], W, diff[3], h)
-            torch.autograd.backward(out, go, inputs=diff)
+            torch.autograd.grad(out, diff, go)
             return out
     else:
         diff = [t.requires_grad_(True) for t in dev[:8]]
@@ -80,10 +80,10 @@ def gpu_step_fn(name, pkg, arrays):
         W, h = W0.clone(), h0.clone()
 
         def step():
-            W.copy_(W0)
-            h.copy_(h0)
+            W.zero_()
+            h.zero_()
             out = pkg.rec_update_fwm_tanh(*diff, W, h)
-            torch.autograd.backward(out, go, inputs=diff)
+            torch.autograd.grad(out, diff, go)
             return out
     return step, diff
 
@@ -96,7 +96,7 @@ def kernel_times(name, pkg, arrays, iters):
     lib = L.lib()
     dev = [torch.from_numpy(a).to("cuda:0") for a in arrays]
     go = dev[-1]
-    stream = L.stream_of(go)
+    stream_of = lambda: L.stream_of(go)      # evaluated per launch: the current stream may be a capturing one
     chunk = L.query(L.Q_DEFAULT_CHUNK)
     f32 = dict(device="cuda:0", dtype=torch.float32)
 
@@ -115,11 +115,11 @@ def kernel_times(name, pkg, arrays, iters):
 
         def fwd():
             return lib.fwp_delta_fwd(view(q), view(k), view(v), view(beta), L.ptr(W), L.ptr(out), L.ptr(vdiff),
-                                     L.ptr(ckpt), N, H, T, E, M, chunk, stream)
+                                     L.ptr(ckpt), N, H, T, E, M, chunk, stream_of())
 
         def bwd():
             return lib.fwp_delta_bwd(view(q), view(k), view(beta), L.ptr(vdiff), view(go), L.ptr(ckpt), L.ptr(gq),
-                                     L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, E, M, chunk, stream)
+                                     L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, E, M, chunk, stream_of())
         reset = lambda: W.copy_(W0)
     elif name == "rnn":
         z, k, v, W0, beta, h0 = dev[:6]
@@ -132,11 +132,11 @@ def kernel_times(name, pkg, arrays, iters):
 
         def fwd():
             return lib.fwp_rnn_fwd(view(z), view(k), view(v), view(beta), L.ptr(W), L.ptr(h), L.ptr(out),
-                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream)
+                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream_of())
 
         def bwd():
             return lib.fwp_rnn_bwd(view(k), view(beta), L.ptr(vdiff), L.ptr(out), L.ptr(h0), view(go), L.ptr(ckpt),
-                                   L.ptr(gz), L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, D, chunk, stream)
+                                   L.ptr(gz), L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, D, chunk, stream_of())
 
         def reset():
             W.copy_(W0)
@@ -155,41 +155,45 @@ def kernel_times(name, pkg, arrays, iters):
         def fwd():
             return lib.fwp_rec_fwd(view(qx), view(kx), view(vx), view(bx), L.ptr(Rq), L.ptr(Rk), L.ptr(Rv),
                                    L.ptr(rb), L.ptr(W), L.ptr(h), L.ptr(out), L.ptr(qa), L.ptr(ka), L.ptr(ba),
-                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream)
+                                   L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk, stream_of())
 
         def bwd():
             return lib.fwp_rec_bwd(L.ptr(qa), L.ptr(ka), L.ptr(ba), L.ptr(vdiff), L.ptr(out), L.ptr(h0), view(go),
                                    L.ptr(Rq), L.ptr(Rk), L.ptr(Rv), L.ptr(rb), L.ptr(ckpt), *[L.ptr(t) for t in g],
-                                   L.ptr(ws), N, H, T, D, chunk, stream)
+                                   L.ptr(ws), N, H, T, D, chunk, stream_of())
 
         def reset():
             W.copy_(W0)
             h.copy_(h0)
 
-    def timed(fn, pre=None):
+    def timed(fn):
+        """Average duration of `iters` back-to-back launches between two events on the launch stream."""
         for _ in range(3):
-            if pre:
-                pre()
             L.check(fn(), "warm-up launch")
         torch.cuda.synchronize()
-        total = 0.0
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
         for _ in range(iters):
-            if pre:
-                pre()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
             rc = fn()
-            e1.record()
-            L.check(rc, "timed launch")
-            e1.synchronize()
-            total += e0.elapsed_time(e1) * 1e-3
-        return total / iters
+        e1.record()
+        L.check(rc, "timed launch")
+        e1.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / iters
 
-    t_f = timed(fwd, reset)
+    t_f = timed(fwd)       # the state carries over between launches; the work per launch is the same
     reset()
     L.check(fwd(), "forward before backward timing")
     t_b = timed(bwd)
-    return t_f, t_b
+
+    def abi_step():
+        """state reset + forward + backward, straight through the C ABI on preallocated buffers"""
+        W.zero_()
+        if name != "delta":
+            h.zero_()
+        L.check(fwd(), "forward")
+        L.check(bwd(), "backward")
+
+    return t_f, t_b, abi_step
 
 
 def cpu_baseline(name, arrays, w, reps):
@@ -230,6 +234,8 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS), default="delta")
     ap.add_argument("--cpu-reps", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="time a HIP graph replay of the step recorded through the C ABI instead of eager calls")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sequences are independent; "
@@ -246,19 +252,44 @@ def main():
     tokens = B * T
     token_heads = tokens * H
 
+    # run backward on the calling thread: the hand-over to the autograd engine's device thread costs
+    # more than the kernels of this step take
+    torch.autograd.set_multithreading_enabled(False)
     step, _ = gpu_step_fn(name, pkg, arrays)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms = elapsed / args.steps * 1e3
-    value = tokens / (elapsed / args.steps)
 
-    t_f, t_b = kernel_times(name, pkg, arrays, max(20, min(args.steps, 100)))
+    def timed_steps(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    eager_s = timed_steps(step)
+    t_f, t_b, abi_step = kernel_times(name, pkg, arrays, max(20, min(args.steps, 100)))
+    launch = "eager calls of the autograd Function"
+    step_s = eager_s
+    if args.graph:
+        # The same three launches (state reset, forward, backward) recorded once into a HIP graph
+        # through the C ABI on preallocated buffers and replayed: no Python or autograd-engine time
+        # between the kernels.
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                abi_step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            abi_step()
+        step_s = timed_steps(graph.replay)
+        launch = "hipGraph replay of reset+forward+backward recorded through the C ABI"
+    ms = step_s * 1e3
+    value = tokens / step_s
+
     fwd_bytes = w["fwd_bytes"](D) * token_heads
     bwd_bytes = w["bwd_bytes"](D) * token_heads
     dom = "bwd" if t_b >= t_f else "fwd"
@@ -269,7 +300,7 @@ def main():
         "metric": METRIC, "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": w["label"], "B": B, "H": H, "T": T, "D": D},
+        "config": {"workload": w["label"], "B": B, "H": H, "T": T, "D": D, "launch": launch},
         "roofline": {"bound": "hbm", "kernel": f"{name} {dom}", "achieved": dom_bytes / dom_t / 1e9,
                      "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": dom_bytes / dom_t / PEAK_HBM,
                      "traffic": None},
@@ -278,7 +309,8 @@ def main():
                     "kernel_only_tokens_per_s": tokens / kernel_s,
                     "valu_frac_of_157.3TF": flops / kernel_s / PEAK_VALU,
                     "hbm_frac_of_8TBps": (fwd_bytes + bwd_bytes) / kernel_s / PEAK_HBM,
-                    "step_valu_frac_of_157.3TF": flops / (ms * 1e-3) / PEAK_VALU},
+                    "step_valu_frac_of_157.3TF": flops / (ms * 1e-3) / PEAK_VALU,
+                    "eager_tokens_per_s": tokens / eager_s, "eager_ms_per_step": eager_s * 1e3},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(name, arrays, w, args.cpu_reps)

@@ -61,8 +61,13 @@ def lib():
     return _lib
 
 
+_query_cache = {}
+
+
 def query(what):
-    return int(lib().fwp_query(int(what)))
+    if what not in _query_cache:
+        _query_cache[what] = int(lib().fwp_query(int(what)))
+    return _query_cache[what]
 
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
@@ -79,13 +84,14 @@ def check(code, what):
 
 def require_device(t):
     """The operators exist for fp32 tensors on a gfx950 GPU only."""
-    if t.device.type != "cuda":
-        raise FwpError(f"fast-weight operators need tensors on an MI355X GPU, got device '{t.device}'")
-    idx = t.device.index if t.device.index is not None else torch.cuda.current_device()
-    if idx not in _checked_devices:
-        with torch.cuda.device(idx):
-            check(lib().fwp_check_device(), "device check")
-        _checked_devices.add(idx)
+    dev = t.device
+    if dev in _checked_devices:
+        return
+    if dev.type != "cuda":
+        raise FwpError(f"fast-weight operators need tensors on an MI355X GPU, got device '{dev}'")
+    with torch.cuda.device(dev):
+        check(lib().fwp_check_device(), "device check")
+    _checked_devices.add(dev)
 
 
 def rows(t):
@@ -105,3 +111,19 @@ def ptr(t):
 
 def stream_of(t):
     return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+class on_device:
+    """Make the tensor's GPU current for the launch; free when it already is."""
+
+    def __init__(self, t):
+        idx = (t if isinstance(t, torch.device) else t.device).index
+        self.guard = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
+
+    def __enter__(self):
+        if self.guard is not None:
+            self.guard.__enter__()
+
+    def __exit__(self, *exc):
+        if self.guard is not None:
+            self.guard.__exit__(*exc)

@@ -46,15 +46,18 @@ __device__ __forceinline__ int reg_index(int lane, int jj) {
     return 16 * pr + G::S * ((mm - j + G::NR) % G::NR) + s;
 }
 
-constexpr int kRowHalfMirror = 0x141;
-
 // acc + ror(x, ROT) * y, the rotation being inside the 16-lane row.  x must come
 // straight from an LDS/memory load (a DPP source written by a VALU instruction just
 // before would need wait states the compiler cannot see through the asm).
-template <int ROT>
+template <int ROT, bool NEG = false>
 __device__ __forceinline__ float fmac_ror(float acc, float x, float y) {
     if constexpr (ROT == 0) {
-        return fmaf(x, y, acc);
+        return NEG ? fmaf(x, -y, acc) : fmaf(x, y, acc);
+    } else if constexpr (NEG) {
+        asm("v_fmac_f32_dpp %0, %1, -%2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+            : "+v"(acc)
+            : "v"(x), "v"(y), "n"(ROT));
+        return acc;
     } else {
         asm("v_fmac_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
             : "+v"(acc)
@@ -69,10 +72,10 @@ __device__ __forceinline__ float dot_rot1(const float *w, float x, float acc,
     ((acc = fmac_ror<S * J>(acc, x, w[J])), ...);
     return acc;
 }
-template <int S, int... J>
+template <int S, bool NEG, int... J>
 __device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
                                            std::integer_sequence<int, J...>) {
-    ((w[J] = fmac_ror<S * J>(w[J], x, y)), ...);
+    ((w[J] = fmac_ror<S * J, NEG>(w[J], x, y)), ...);
 }
 
 // sum_jj w[jj] * x[index(jj)]  for a periodic vector x[NP]
@@ -85,26 +88,31 @@ __device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const floa
         acc = dot_rot1<G::S>(&w[p * G::NR], x[p], acc, std::make_integer_sequence<int, G::NR>{});
     return acc;
 }
-// w[jj] += x[index(jj)] * y
-template <int D>
+// w[jj] += x[index(jj)] * y   (NEG: -= )
+template <int D, bool NEG = false>
 __device__ __forceinline__ void rank1_rot(float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
                                           float y) {
     using G = Geo<D>;
 #pragma unroll
     for (int p = 0; p < G::NP; p++)
-        rank1_rot1<G::S>(&w[p * G::NR], x[p], y, std::make_integer_sequence<int, G::NR>{});
+        rank1_rot1<G::S, NEG>(&w[p * G::NR], x[p], y, std::make_integer_sequence<int, G::NR>{});
 }
 
 // One tile of one [.,D] tensor on its way from HBM to LDS.
 template <int D>
 struct TileRegs {
     float4 r[Geo<D>::NV4];
-    __device__ __forceinline__ void fetch(const float *base, int64_t sL, int t0, int L, int lane) {
+    // lane_base points at this lane's first float4 of the sequence: row lane / (D/4), column
+    // 4 * (lane % (D/4)); the i-th float4 of a tile is kWave / (D/4) rows further down.
+    static constexpr int kRowsPerLoad = kWave / (D / 4);
+    template <bool FULL>
+    __device__ __forceinline__ void fetch(const float *lane_base, int64_t sL, int t0, int L, int lane) {
 #pragma unroll
         for (int i = 0; i < Geo<D>::NV4; i++) {
-            const int f = lane + kWave * i, rw = f / (D / 4), c4 = f % (D / 4);
-            r[i] = (t0 + rw < L) ? *reinterpret_cast<const float4 *>(base + (t0 + rw) * sL + 4 * c4)
-                                 : make_float4(0.f, 0.f, 0.f, 0.f);
+            const int rw = t0 + lane / (D / 4) + kRowsPerLoad * i;
+            const float4 *src = reinterpret_cast<const float4 *>(lane_base + (int64_t)(t0 + kRowsPerLoad * i) * sL);
+            if constexpr (FULL) r[i] = *src;
+            else r[i] = rw < L ? *src : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
     __device__ __forceinline__ void commit(float *tile, int lane) const {
@@ -121,8 +129,20 @@ struct TileRegs {
     }
 };
 
+// A tile of outputs staged in LDS goes to HBM with 16-byte stores (rows beyond L are dropped).
+template <int D>
+__device__ __forceinline__ void flush_tile(const float *tile, float *dst_rows, int t0, int L,
+                                           int lane) {
+#pragma unroll
+    for (int i = 0; i < Geo<D>::NV4; i++) {
+        const int f = lane + kWave * i, rw = f / (D / 4), c4 = f % (D / 4);
+        const float4 x = *reinterpret_cast<const float4 *>(tile + 4 * f);
+        if (t0 + rw < L) *reinterpret_cast<float4 *>(dst_rows + (int64_t)(t0 + rw) * D + 4 * c4) = x;
+    }
+}
+
 // Row-wise dot products of two tiles held in registers: lane gets (a_row . b_row)
-// of row (lane + 64 i) / (D/4) in out[i].
+// of the row of its i-th float4 in out[i].
 template <int D>
 __device__ __forceinline__ void tile_row_dots(const TileRegs<D> &a, const TileRegs<D> &b,
                                               float (&out)[Geo<D>::NV4]) {
@@ -133,7 +153,7 @@ __device__ __forceinline__ void tile_row_dots(const TileRegs<D> &a, const TileRe
         x = fmaf(a.r[i].z, b.r[i].z, x);
         x = fmaf(a.r[i].w, b.r[i].w, x);
         x = group_sum<4>(x);
-        if constexpr (D == 32) x += dpp<kRowHalfMirror>(x);
+        if constexpr (D == 32) x += dpp<0x141>(x);   // row_half_mirror: the other quad of the 8-lane row group
         out[i] = x;
     }
 }
@@ -160,6 +180,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     __shared__ __align__(16) float sv_[WPB][2][kTile * D];
     __shared__ __align__(16) float sb_[WPB][2][kTile];
     __shared__ __align__(16) float skq_[WPB][2][kTile];
+    __shared__ __align__(16) float sout_[WPB][2][kTile * D];   // staged out and vdiff tiles
 
     // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
     const int wave = threadIdx.x / kWave;
@@ -172,6 +193,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     auto &sv = sv_[wave];
     auto &sb = sb_[wave];
     auto &skq = skq_[wave];
+    auto &sout = sout_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
                 *bb = row(beta, n, h, 0);
 
@@ -181,26 +203,43 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
 
     TileRegs<D> pq, pk, pv;
     float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *qlane = qb + lrow * q.sL + 4 * lc4, *klane = kb + lrow * k.sL + 4 * lc4,
+                *vlane = vb + lrow * v.sL + 4 * lc4;
     auto fetch = [&](int t0) {
-        pq.fetch(qb, q.sL, t0, L, lane);
-        pk.fetch(kb, k.sL, t0, L, lane);
-        pv.fetch(vb, v.sL, t0, L, lane);
-        if (lane < kTile) pb = (t0 + lane < L) ? bb[(t0 + lane) * beta.sL] : 0.f;
+        if (t0 + kTile <= L) {
+            pq.template fetch<true>(qlane, q.sL, t0, L, lane);
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pv.template fetch<true>(vlane, v.sL, t0, L, lane);
+        } else {
+            pq.template fetch<false>(qlane, q.sL, t0, L, lane);
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pv.template fetch<false>(vlane, v.sL, t0, L, lane);
+        }
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];   // every 16-lane row loads the tile's betas
     };
     auto commit = [&](int buf) {
         pq.commit(sq[buf], lane);
         pk.commit(sk[buf], lane);
         pv.commit(sv[buf], lane);
-        if (lane < kTile) sb[buf][lane] = pb;
+        sb[buf][per] = pb;
         float kq[NV4];
         tile_row_dots<D>(pk, pq, kq);
 #pragma unroll
-        for (int i = 0; i < NV4; i++) skq[buf][(lane + kWave * i) / (D / 4)] = kq[i];
+        for (int i = 0; i < NV4; i++) skq[buf][lrow + TileRegs<D>::kRowsPerLoad * i] = kq[i];
     };
 
-    // lanes with odd s store vdiff, the others out (same value from every lane that shares an address)
-    const bool store_d = (vdiff != nullptr) && (sl & 1);
-    float *dst = (store_d ? vdiff : out) + seq * L * D + col;
+    // Results are staged in LDS (lanes with odd s write vdiff, the others out; lanes that share
+    // an address write the same value) and leave for HBM one tile later, so that the only
+    // memory operations in flight when a tile is committed are at least a tile old.
+    const bool store_d = sl & 1;
+    float *stage = sout[store_d ? 1 : 0] + col;
+    float *out_rows = out + seq * L * D;
+    float *vd_rows = vdiff ? vdiff + seq * L * D : nullptr;
+    auto flush = [&](int t0) {
+        flush_tile<D>(sout[0], out_rows, t0, L, lane);
+        if (vd_rows) flush_tile<D>(sout[1], vd_rows, t0, L, lane);
+    };
 
     auto load_ops = [&](FwdOps<D> &o, int buf, int tt) {
 #pragma unroll
@@ -212,7 +251,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
         o.b = sb[buf][tt];
         o.kq = skq[buf][tt];
     };
-    // out_t = W_t^T q = W_{t-1}^T q + u (k.q): both mat-vecs read the old state
+    // out_t = W_t^T q = W_{t-1}^T q + u (k.q): both mat-vecs read the old state, so their
+    // dependent DPP sums overlap instead of running one after the other
     auto compute = [&](const FwdOps<D> &o, float *o_ptr) {
         const float p_old = group_sum<S>(dot_rot<D>(Wc, o.k));
         const float p_out = group_sum<S>(dot_rot<D>(Wc, o.q));
@@ -234,8 +274,9 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
         const int buf = it & 1, t0 = it * kTile;
         const int nst = min(kTile, L - t0);
         if (it + 1 < ntile) commit(buf ^ 1);
+        if (it > 0) flush(t0 - kTile);
         if (it + 2 < ntile) fetch(t0 + 2 * kTile);
-        float *tile_dst = dst + (int64_t)t0 * D;
+        float *tile_dst = stage;
         if (nst == kTile) {
 #pragma unroll
             for (int tt = 0; tt < kTile; tt++) {
@@ -258,6 +299,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
             for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[jj];
         }
     }
+    flush((ntile - 1) * kTile);
 #pragma unroll
     for (int jj = 0; jj < R; jj++) W[(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[jj];
 }
@@ -289,6 +331,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     __shared__ __align__(16) float su_[WPB][2][kTile * D];
     __shared__ __align__(16) float sb_[WPB][2][kTile];
     __shared__ __align__(16) float spd_[WPB][kTile * D];   // r_i * d_i per step, summed per tile
+    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D];   // staged gq, gk, gv tiles
 
     // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
     const int wave = threadIdx.x / kWave;
@@ -303,6 +346,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     auto &su = su_[wave];
     auto &sb = sb_[wave];
     auto &spd = spd_[wave];
+    auto &sgrad = sgrad_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
                 *bb = row(beta, n, h, 0);
     const float *db = vdiff + seq * L * D;
@@ -314,20 +358,28 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
 
     TileRegs<D> pq, pk, pgo, pd, pu;
     float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *qlane = qb + lrow * q.sL + 4 * lc4, *klane = kb + lrow * k.sL + 4 * lc4,
+                *golane = gob + lrow * go.sL + 4 * lc4, *dlane = db + lrow * D + 4 * lc4;
     auto fetch = [&](int t0) {
-        pq.fetch(qb, q.sL, t0, L, lane);
-        pk.fetch(kb, k.sL, t0, L, lane);
-        pgo.fetch(gob, go.sL, t0, L, lane);
-        pd.fetch(db, D, t0, L, lane);
+        if (t0 + kTile <= L) {
+            pq.template fetch<true>(qlane, q.sL, t0, L, lane);
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+            pd.template fetch<true>(dlane, D, t0, L, lane);
+        } else {
+            pq.template fetch<false>(qlane, q.sL, t0, L, lane);
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+            pd.template fetch<false>(dlane, D, t0, L, lane);
+        }
         float bs[NV4];
 #pragma unroll
-        for (int x = 0; x < NV4; x++) {
-            const int rw = (lane + kWave * x) / (D / 4);
-            bs[x] = (t0 + rw < L) ? bb[(t0 + rw) * beta.sL] : 0.f;
-        }
+        for (int x = 0; x < NV4; x++)
+            bs[x] = bb[(int64_t)min(t0 + lrow + TileRegs<D>::kRowsPerLoad * x, L - 1) * beta.sL];
         pu = pd;
         pu.scale_rows(bs);
-        if (lane < kTile) pb = (t0 + lane < L) ? bb[(t0 + lane) * beta.sL] : 0.f;
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
     };
     auto commit = [&](int buf) {
         pq.commit(sq[buf], lane);
@@ -335,7 +387,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         pgo.commit(sgo[buf], lane);
         pd.commit(sd[buf], lane);
         pu.commit(su[buf], lane);
-        if (lane < kTile) sb[buf][lane] = pb;
+        sb[buf][per] = pb;
     };
     auto fetch_state = [&](int c) {
         const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
@@ -343,10 +395,12 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
     };
 
-    // One store per step covers gq, gk and gv: lanes pick their output by s.
-    // S = 4: s=0 -> gq, s=1 -> gk, s=2,3 -> gv.   S = 2: s=0 -> gq, s=1 -> gk, and a second store for gv.
-    float *dst1 = (sl == 0 ? gq : (sl == 1 ? gk : gv)) + seq * L * D + i;
-    float *dst2 = gv + seq * L * D + i;
+    // Gradients are staged in LDS and leave for HBM one tile later (see the forward kernel).
+    // One LDS write per step covers gq, gk and gv: lanes pick their output by s.
+    // S = 4: s=0 -> gq, s=1 -> gk, s=2,3 -> gv.   S = 2: s=0 -> gq, s=1 -> gk, and a second write for gv.
+    float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
+    float *dst2 = sgrad[2] + i;
+    float *gq_rows = gq + seq * L * D, *gk_rows = gk + seq * L * D, *gv_rows = gv + seq * L * D;
     // source lane (as a byte address for ds_bpermute) of the periodic copy of a per-group value
     int gather[NP];
 #pragma unroll
@@ -367,7 +421,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         o.d_i = sd[buf][off + i];
         o.b = sb[buf][tt];
     };
-    auto compute = [&](const BwdOps<D> &o, int tt, int64_t tile_off) {
+    auto compute = [&](const BwdOps<D> &o, int tt) {
         // G' = G + q (x) go (both layouts);  r = G'^T k
         rank1_rot<D>(Gc, o.q, o.go_i);
         const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
@@ -381,20 +435,24 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         spd[tt * D + i] = r_i * o.d_i;
         rank1_rot<D>(Gr, o.go, o.q_i);
         const float gq_i = group_sum<S>(dot_rot<D>(Wr, o.go));   // (W_t go)[i]
-        rank1_rot<D>(Wr, o.u, -o.k_i);                            // W_{t-1}
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                       // W_{t-1}
         rank1_rot<D>(Gc, o.k, a_i);
         float gk_i = dot_rot<D>(Gr, o.u);                         // G' u + W_{t-1} a
         gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
         rank1_rot<D>(Gr, a, o.k_i);
         if constexpr (S == 4) {
-            (dst1 + tile_off)[tt * D] = sl == 0 ? gq_i : (sl == 1 ? gk_i : gv_i);
+            dst1[tt * D] = sl == 0 ? gq_i : (sl == 1 ? gk_i : gv_i);
         } else {
-            (dst1 + tile_off)[tt * D] = sl == 0 ? gq_i : gk_i;
-            (dst2 + tile_off)[tt * D] = gv_i;
+            dst1[tt * D] = sl == 0 ? gq_i : gk_i;
+            dst2[tt * D] = gv_i;
         }
     };
-    // gbeta of the tile's steps: sum spd[tt][:] over the D entries, four lanes per step
-    auto flush_gbeta = [&](int t0, int nst) {
+    // a finished tile of gradients goes to HBM; gbeta of its steps is the sum of spd[tt][:]
+    // over the D entries, four lanes per step
+    auto flush = [&](int t0, int nst) {
+        flush_tile<D>(sgrad[0], gq_rows, t0, L, lane);
+        flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
+        flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
         const int tt = lane / 4, part = lane % 4;
         float acc = 0.f;
 #pragma unroll
@@ -423,9 +481,9 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
             for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
         }
         if (it >= 1) commit(buf ^ 1);
+        if (it + 1 < ntile) flush(t0 + kTile, min(kTile, L - t0 - kTile));
         if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
         if (it >= 2) fetch(t0 - 2 * kTile);
-        const int64_t tile_off = (int64_t)t0 * D;
         if (nst == kTile) {
             if (!primed) {
 #pragma unroll
@@ -437,17 +495,17 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
                 const int nt = tt - PF;
                 if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
                 else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
-                compute(ring[tt % RING], tt, tile_off);
+                compute(ring[tt % RING], tt);
             }
         } else {  // ragged last tile (first in reverse): not pipelined
             for (int tt = nst - 1; tt >= 0; tt--) {
                 BwdOps<D> o;
                 load_ops(o, buf, tt);
-                compute(o, tt, tile_off);
+                compute(o, tt);
             }
         }
-        flush_gbeta(t0, nst);
     }
+    flush(0, min(kTile, L));
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }

@@ -29,10 +29,10 @@ class DeltaFastWeight(torch.autograd.Function):
                                 f"V{tuple(V.shape)} beta{tuple(beta.shape)}")
         if W.shape != (N, H, E, M) or not W.is_contiguous() or W.dtype != torch.float32:
             raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
-        Q, qv = _lib.rows(Q.detach())
-        K, kv = _lib.rows(K.detach())
-        V, vv = _lib.rows(V.detach())
-        beta, bv = _lib.rows(beta.detach())
+        Q, qv = _lib.rows(Q)
+        K, kv = _lib.rows(K)
+        V, vv = _lib.rows(V)
+        beta, bv = _lib.rows(beta)
         need_grad = any(ctx.needs_input_grad[:4])
         chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
         out = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
@@ -40,7 +40,7 @@ class DeltaFastWeight(torch.autograd.Function):
         if need_grad:
             vdiff = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
             ckpt = torch.empty((N, H, _nchunk(L, chunk), E, M), device=Q.device, dtype=torch.float32)
-        with torch.cuda.device(Q.device):
+        with _lib.on_device(Q):
             rc = _lib.lib().fwp_delta_fwd(
                 qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out),
                 _lib.ptr(vdiff) if need_grad else None, _lib.ptr(ckpt) if need_grad else None,
@@ -66,7 +66,7 @@ class DeltaFastWeight(torch.autograd.Function):
         grad_K = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
         grad_V = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
         grad_beta = torch.empty((N, H, L, 1), device=Q.device, dtype=torch.float32)
-        with torch.cuda.device(Q.device):
+        with _lib.on_device(Q):
             rc = _lib.lib().fwp_delta_bwd(
                 qv, kv, bv, _lib.ptr(vdiff), gv_, _lib.ptr(ckpt), _lib.ptr(grad_Q),
                 _lib.ptr(grad_K), _lib.ptr(grad_V), _lib.ptr(grad_beta), N, H, L, E, M, chunk,

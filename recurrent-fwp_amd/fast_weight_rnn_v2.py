@@ -30,10 +30,10 @@ class FastRNNv2(torch.autograd.Function):
         for name, t in (("W", W), ("h0", h0)):
             if not t.is_contiguous() or t.dtype != torch.float32:
                 raise _lib.FwpError(f"{name} must be a contiguous fp32 tensor")
-        Z, zv = _lib.rows(Z.detach())
-        K, kv = _lib.rows(K.detach())
-        V, vv = _lib.rows(V.detach())
-        beta, bv = _lib.rows(beta.detach())
+        Z, zv = _lib.rows(Z)
+        K, kv = _lib.rows(K)
+        V, vv = _lib.rows(V)
+        beta, bv = _lib.rows(beta)
         need_grad = any(ctx.needs_input_grad)
         chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
         dev = Z.device
@@ -43,7 +43,7 @@ class FastRNNv2(torch.autograd.Function):
             h_init = h0.detach().clone()
             vdiff = torch.empty((N, H, L, D), device=dev, dtype=torch.float32)
             ckpt = torch.empty((N, H, _nchunk(L, chunk), D, D), device=dev, dtype=torch.float32)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             rc = _lib.lib().fwp_rnn_fwd(
                 zv, kv, vv, bv, _lib.ptr(W), _lib.ptr(h0), _lib.ptr(out),
                 _lib.ptr(vdiff) if need_grad else None, _lib.ptr(ckpt) if need_grad else None,
@@ -68,7 +68,7 @@ class FastRNNv2(torch.autograd.Function):
         grad_Z, grad_K, grad_V = (torch.empty((N, H, L, D), device=dev, dtype=torch.float32)
                                   for _ in range(3))
         grad_beta = torch.empty((N, H, L, 1), device=dev, dtype=torch.float32)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             rc = _lib.lib().fwp_rnn_bwd(
                 kv, bv, _lib.ptr(vdiff), _lib.ptr(out), _lib.ptr(h_init), gv_, _lib.ptr(ckpt),
                 _lib.ptr(grad_Z), _lib.ptr(grad_K), _lib.ptr(grad_V), _lib.ptr(grad_beta),

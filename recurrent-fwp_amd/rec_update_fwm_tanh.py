@@ -33,10 +33,10 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
             if not t.is_contiguous() or t.dtype != torch.float32:
                 raise _lib.FwpError(f"{name} must be a contiguous fp32 tensor")
         D = M
-        qx, qv = _lib.rows(qx.detach())
-        kx, kv = _lib.rows(kx.detach())
-        vx, vv = _lib.rows(vx.detach())
-        bx, bv = _lib.rows(bx.detach())
+        qx, qv = _lib.rows(qx)
+        kx, kv = _lib.rows(kx)
+        vx, vv = _lib.rows(vx)
+        bx, bv = _lib.rows(bx)
         Rq, Rk, Rv, rb = (t.detach().contiguous().float() for t in (R_q, R_k, R_v, r_b))
         need_grad = any(ctx.needs_input_grad)
         chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
@@ -51,7 +51,7 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
                      torch.empty((N, H, L), device=dev, dtype=torch.float32),      # beta after sigmoid
                      torch.empty((N, H, L, D), device=dev, dtype=torch.float32),   # v - v_old
                      torch.empty((N, H, _nchunk(L, chunk), D, D), device=dev, dtype=torch.float32)]
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             rc = _lib.lib().fwp_rec_fwd(
                 qv, kv, vv, bv, _lib.ptr(Rq), _lib.ptr(Rk), _lib.ptr(Rv), _lib.ptr(rb),
                 _lib.ptr(W), _lib.ptr(h0), _lib.ptr(out),
@@ -79,7 +79,7 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
                                         for _ in range(3))
         grad_r_b = torch.empty((1, H, 1, D), device=dev, dtype=torch.float32)
         workspace = torch.empty((N, H, 3 * D * D + D), device=dev, dtype=torch.float32)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             rc = _lib.lib().fwp_rec_bwd(
                 _lib.ptr(q_act), _lib.ptr(k_act), _lib.ptr(beta_act), _lib.ptr(vdiff),
                 _lib.ptr(out), _lib.ptr(h_init), gv_, _lib.ptr(Rq), _lib.ptr(Rk), _lib.ptr(Rv),
