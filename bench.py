@@ -236,7 +236,19 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true",
                     help="time a HIP graph replay of the step recorded through the C ABI instead of eager calls")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run ten device-to-device copies of 256 MiB (a kernel of known traffic for "
+                         "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
+    if args.copy_calibration:
+        import torch
+        src = torch.ones(64 * 1024 * 1024, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
+        return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sequences are independent; "
                  "more GPUs would just split the batch). Use --gpus 1.")

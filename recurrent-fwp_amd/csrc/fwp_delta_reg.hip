@@ -180,7 +180,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     __shared__ __align__(16) float sv_[WPB][2][kTile * D];
     __shared__ __align__(16) float sb_[WPB][2][kTile];
     __shared__ __align__(16) float skq_[WPB][2][kTile];
-    __shared__ __align__(16) float sout_[WPB][2][kTile * D];   // staged out and vdiff tiles
+    __shared__ __align__(16) float sout_[WPB][2][kTile * D + 16];   // staged out and vdiff tiles (+16: the two land in different banks)
 
     // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
     const int wave = threadIdx.x / kWave;
@@ -331,7 +331,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     __shared__ __align__(16) float su_[WPB][2][kTile * D];
     __shared__ __align__(16) float sb_[WPB][2][kTile];
     __shared__ __align__(16) float spd_[WPB][kTile * D];   // r_i * d_i per step, summed per tile
-    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D];   // staged gq, gk, gv tiles
+    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gq, gk, gv tiles (+16: different banks)
 
     // every wave of the block owns one sequence and its own LDS tiles; waves never synchronise
     const int wave = threadIdx.x / kWave;
