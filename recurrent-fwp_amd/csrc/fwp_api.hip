@@ -2,6 +2,7 @@
 // the register-state kernels (E = M in {16, 32}, 16-byte aligned rows) and the
 // LDS-state kernels (everything else).
 #include "fwp_common.hpp"
+#include <stdint.h>
 
 #include <string.h>
 
@@ -65,7 +66,7 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
-        aligned16(vdiff) && aligned16(ckpt))
+        aligned16(vdiff) && aligned16(ckpt) && aligned16(out))
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                              (hipStream_t)stream);
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
@@ -80,7 +81,7 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
-        aligned16(vdiff) && aligned16(ckpt))
+        aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv))
         return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
                              chunk, (hipStream_t)stream);
     return generic_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
@@ -93,6 +94,10 @@ int fwp_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, flo
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    if (reg_rnn_supported(D) && reg_view_ok(z) && reg_view_ok(k) && reg_view_ok(v) &&
+        aligned16(vdiff) && aligned16(ckpt) && aligned16(out))
+        return reg_rnn_fwd(z, k, v, beta, W, h, out, vdiff, ckpt, N, H, L, D, chunk,
+                           (hipStream_t)stream);
     return generic_rnn_fwd(z, k, v, beta, W, h, out, vdiff, ckpt, N, H, L, D, chunk,
                            (hipStream_t)stream);
 }
@@ -104,6 +109,11 @@ int fwp_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
         !ckpt || !gz || !gk || !gv || !gbeta)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    if (reg_rnn_supported(D) && reg_view_ok(k) && reg_view_ok(grad_out) && aligned16(vdiff) &&
+        aligned16(ckpt) && aligned16(out) && aligned16(h_init) && aligned16(gz) && aligned16(gk) &&
+        aligned16(gv))
+        return reg_rnn_bwd(k, beta, vdiff, out, h_init, grad_out, ckpt, gz, gk, gv, gbeta, N, H, L, D,
+                           chunk, (hipStream_t)stream);
     return generic_rnn_bwd(k, beta, vdiff, out, h_init, grad_out, ckpt, gz, gk, gv, gbeta, N, H, L,
                            D, chunk, (hipStream_t)stream);
 }

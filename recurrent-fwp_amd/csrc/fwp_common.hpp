@@ -50,6 +50,13 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                   int L, int D, int chunk, hipStream_t s);
 
+bool reg_rnn_supported(int D);
+int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
+                float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
+                const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
+                float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s);
+
 // Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 

@@ -19,127 +19,10 @@
 // q/k/v/beta (grad_out, vdiff) stream through double-buffered LDS tiles of kTile
 // steps, fetched from HBM two tiles ahead with 16-byte loads; inside a tile the
 // operands of the next steps are read from LDS while the current step computes.
-#include "fwp_common.hpp"
-#include "fwp_wave.hpp"
-
-#include <utility>
+#include "fwp_reg.hpp"
 
 namespace fwp {
 namespace {
-
-template <int D>
-struct Geo {
-    static constexpr int S = kWave / D;                // lanes per group
-    static constexpr int NP = D / 16;                  // periodic registers per D-vector
-    static constexpr int NR = 16 / S;                  // rotations per periodic register
-    static constexpr int R = NP * NR;                  // state entries per lane (= D / S)
-    static constexpr int NV4 = kTile * D / 4 / kWave;  // float4 per lane per tile tensor
-    static_assert(D * S == kWave && NV4 >= 1, "D must be 16 or 32");
-};
-
-// Index (row in forward, column in backward) of state register jj of lane `lane`.
-template <int D>
-__device__ __forceinline__ int reg_index(int lane, int jj) {
-    using G = Geo<D>;
-    const int pr = jj / G::NR, j = jj % G::NR;
-    const int mm = (lane % 16) / G::S, s = lane % G::S;
-    return 16 * pr + G::S * ((mm - j + G::NR) % G::NR) + s;
-}
-
-// acc + ror(x, ROT) * y, the rotation being inside the 16-lane row.  x must come
-// straight from an LDS/memory load (a DPP source written by a VALU instruction just
-// before would need wait states the compiler cannot see through the asm).
-template <int ROT, bool NEG = false>
-__device__ __forceinline__ float fmac_ror(float acc, float x, float y) {
-    if constexpr (ROT == 0) {
-        return NEG ? fmaf(x, -y, acc) : fmaf(x, y, acc);
-    } else if constexpr (NEG) {
-        asm("v_fmac_f32_dpp %0, %1, -%2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
-            : "+v"(acc)
-            : "v"(x), "v"(y), "n"(ROT));
-        return acc;
-    } else {
-        asm("v_fmac_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
-            : "+v"(acc)
-            : "v"(x), "v"(y), "n"(ROT));
-        return acc;
-    }
-}
-
-template <int S, int... J>
-__device__ __forceinline__ float dot_rot1(const float *w, float x, float acc,
-                                          std::integer_sequence<int, J...>) {
-    ((acc = fmac_ror<S * J>(acc, x, w[J])), ...);
-    return acc;
-}
-template <int S, bool NEG, int... J>
-__device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
-                                           std::integer_sequence<int, J...>) {
-    ((w[J] = fmac_ror<S * J, NEG>(w[J], x, y)), ...);
-}
-
-// sum_jj w[jj] * x[index(jj)]  for a periodic vector x[NP]
-template <int D>
-__device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
-                                         float acc = 0.f) {
-    using G = Geo<D>;
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        acc = dot_rot1<G::S>(&w[p * G::NR], x[p], acc, std::make_integer_sequence<int, G::NR>{});
-    return acc;
-}
-// w[jj] += x[index(jj)] * y   (NEG: -= )
-template <int D, bool NEG = false>
-__device__ __forceinline__ void rank1_rot(float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
-                                          float y) {
-    using G = Geo<D>;
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        rank1_rot1<G::S, NEG>(&w[p * G::NR], x[p], y, std::make_integer_sequence<int, G::NR>{});
-}
-
-// One tile of one [.,D] tensor on its way from HBM to LDS.
-template <int D>
-struct TileRegs {
-    float4 r[Geo<D>::NV4];
-    // lane_base points at this lane's first float4 of the sequence: row lane / (D/4), column
-    // 4 * (lane % (D/4)); the i-th float4 of a tile is kWave / (D/4) rows further down.
-    static constexpr int kRowsPerLoad = kWave / (D / 4);
-    template <bool FULL>
-    __device__ __forceinline__ void fetch(const float *lane_base, int64_t sL, int t0, int L, int lane) {
-#pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++) {
-            const int rw = t0 + lane / (D / 4) + kRowsPerLoad * i;
-            const float4 *src = reinterpret_cast<const float4 *>(lane_base + (int64_t)(t0 + kRowsPerLoad * i) * sL);
-            if constexpr (FULL) r[i] = *src;
-            else r[i] = rw < L ? *src : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-    }
-    __device__ __forceinline__ void commit(float *tile, int lane) const {
-#pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++)
-            *reinterpret_cast<float4 *>(tile + 4 * (lane + kWave * i)) = r[i];
-    }
-    __device__ __forceinline__ void scale_rows(const float *rowscale) {
-#pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++) {
-            const float b = rowscale[i];
-            r[i].x *= b; r[i].y *= b; r[i].z *= b; r[i].w *= b;
-        }
-    }
-};
-
-// A tile of outputs staged in LDS goes to HBM with 16-byte stores (rows beyond L are dropped).
-template <int D>
-__device__ __forceinline__ void flush_tile(const float *tile, float *dst_rows, int t0, int L,
-                                           int lane) {
-#pragma unroll
-    for (int i = 0; i < Geo<D>::NV4; i++) {
-        const int f = lane + kWave * i, rw = f / (D / 4), c4 = f % (D / 4);
-        const float4 x = *reinterpret_cast<const float4 *>(tile + 4 * f);
-        if (t0 + rw < L) *reinterpret_cast<float4 *>(dst_rows + (int64_t)(t0 + rw) * D + 4 * c4) = x;
-    }
-}
 
 // Row-wise dot products of two tiles held in registers: lane gets (a_row . b_row)
 // of the row of its i-th float4 in out[i].
@@ -152,9 +35,7 @@ __device__ __forceinline__ void tile_row_dots(const TileRegs<D> &a, const TileRe
         x = fmaf(a.r[i].y, b.r[i].y, x);
         x = fmaf(a.r[i].z, b.r[i].z, x);
         x = fmaf(a.r[i].w, b.r[i].w, x);
-        x = group_sum<4>(x);
-        if constexpr (D == 32) x += dpp<0x141>(x);   // row_half_mirror: the other quad of the 8-lane row group
-        out[i] = x;
+        out[i] = row_reduce<D>(x, OpSum());
     }
 }
 
@@ -401,10 +282,6 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
     float *dst2 = sgrad[2] + i;
     float *gq_rows = gq + seq * L * D, *gk_rows = gk + seq * L * D, *gv_rows = gv + seq * L * D;
-    // source lane (as a byte address for ds_bpermute) of the periodic copy of a per-group value
-    int gather[NP];
-#pragma unroll
-    for (int p = 0; p < NP; p++) gather[p] = 4 * S * (16 * p + per);
 
     auto load_ops = [&](BwdOps<D> &o, int buf, int tt) {
         const int off = tt * D;
@@ -428,10 +305,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         const float gv_i = o.b * r_i;
         const float a_i = -gv_i;                              // gradient w.r.t. v_old
         float a[NP];
-#pragma unroll
-        for (int p = 0; p < NP; p++)
-            a[p] = __builtin_bit_cast(
-                float, __builtin_amdgcn_ds_bpermute(gather[p], __builtin_bit_cast(int, a_i)));
+        to_periodic<D>(a_i, a, lane);
         spd[tt * D + i] = r_i * o.d_i;
         rank1_rot<D>(Gr, o.go, o.q_i);
         const float gq_i = group_sum<S>(dot_rot<D>(Wr, o.go));   // (W_t go)[i]
@@ -507,8 +381,6 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     }
     flush(0, min(kTile, L));
 }
-
-bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 }  // namespace
 

@@ -1,0 +1,386 @@
+// Register-state kernels of the Delta RNN v2 op for D in {16, 32}: the delta-rule kernels of
+// fwp_delta_reg.hip plus the recurrent read h_t = W_t^T softmax(h_{t-1}) + z_t.
+//
+// The recurrent vector lives "grouped" (every lane of group m holds h[m]); its softmax needs a max
+// and a sum over the whole wave (DPP row rotates + two row swaps each) and then becomes a periodic
+// operand with one ds_bpermute per 16 entries.  In backward the softmax of the delayed output does
+// not sit on the sequential path: it is recomputed for a whole tile when the tile is committed.
+#include "fwp_reg.hpp"
+
+namespace fwp {
+namespace {
+
+// ------------------------------------------------------------------ forward
+
+template <int D>
+struct RnnFwdOps {
+    float k[Geo<D>::NP], v, z, b;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_view k, fwp_view v,
+                                                             fwp_view beta, float *__restrict__ W,
+                                                             float *__restrict__ hstate,
+                                                             float *__restrict__ out,
+                                                             float *__restrict__ vdiff,
+                                                             float *__restrict__ ckpt, int H, int L,
+                                                             int chunk, int nchunk, int nseq) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sz_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sv_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float sout_[WPB][2][kTile * D + 16];
+
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sz = sz_[wave];
+    auto &sk = sk_[wave];
+    auto &sv = sv_[wave];
+    auto &sb = sb_[wave];
+    auto &sout = sout_[wave];
+    const float *zb = row(z, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
+                *bb = row(beta, n, h, 0);
+
+    float Wc[R];  // W[reg_index(jj)][col]
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Wc[jj] = W[(seq * D + reg_index<D>(lane, jj)) * D + col];
+    float hcur = hstate[seq * D + col];
+
+    TileRegs<D> pz, pk, pv;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *zlane = zb + lrow * z.sL + 4 * lc4, *klane = kb + lrow * k.sL + 4 * lc4,
+                *vlane = vb + lrow * v.sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pz.template fetch<true>(zlane, z.sL, t0, L, lane);
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pv.template fetch<true>(vlane, v.sL, t0, L, lane);
+        } else {
+            pz.template fetch<false>(zlane, z.sL, t0, L, lane);
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pv.template fetch<false>(vlane, v.sL, t0, L, lane);
+        }
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+    };
+    auto commit = [&](int buf) {
+        pz.commit(sz[buf], lane);
+        pk.commit(sk[buf], lane);
+        pv.commit(sv[buf], lane);
+        sb[buf][per] = pb;
+    };
+
+    const bool store_d = sl & 1;
+    float *stage = sout[store_d ? 1 : 0] + col;
+    float *out_rows = out + seq * L * D;
+    float *vd_rows = vdiff ? vdiff + seq * L * D : nullptr;
+    auto flush = [&](int t0) {
+        flush_tile<D>(sout[0], out_rows, t0, L, lane);
+        if (vd_rows) flush_tile<D>(sout[1], vd_rows, t0, L, lane);
+    };
+
+    auto load_ops = [&](RnnFwdOps<D> &o, int buf, int tt) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) o.k[p] = sk[buf][tt * D + 16 * p + per];
+        o.v = sv[buf][tt * D + col];
+        o.z = sz[buf][tt * D + col];
+        o.b = sb[buf][tt];
+    };
+    auto compute = [&](const RnnFwdOps<D> &o, float *o_ptr) {
+        // s = softmax(h_{t-1}); independent of the delta write below, which overlaps its latency
+        const float mx = across_groups<S>(hcur, OpMax());
+        const float e = __expf(hcur - mx);
+        const float s_m = __fdividef(e, across_groups<S>(e, OpSum()));
+        float s[NP];
+        to_periodic<D>(s_m, s, lane);
+        const float d = o.v - group_sum<S>(dot_rot<D>(Wc, o.k));
+        rank1_rot<D>(Wc, o.k, o.b * d);
+        hcur = group_sum<S>(dot_rot<D>(Wc, s)) + o.z;
+        *o_ptr = store_d ? d : hcur;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch(0);
+    commit(0);
+    if (ntile > 1) fetch(kTile);
+    RnnFwdOps<D> ring[RING];
+#pragma unroll
+    for (int p = 0; p < PF; p++) load_ops(ring[p], 0, p);
+
+    for (int it = 0; it < ntile; it++) {
+        const int buf = it & 1, t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        if (it + 1 < ntile) commit(buf ^ 1);
+        if (it > 0) flush(t0 - kTile);
+        if (it + 2 < ntile) fetch(t0 + 2 * kTile);
+        if (nst == kTile) {
+#pragma unroll
+            for (int tt = 0; tt < kTile; tt++) {
+                const int nt = tt + PF;
+                if (nt < kTile) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[nt % RING], buf ^ 1, nt - kTile);
+                compute(ring[tt % RING], stage + tt * D);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                RnnFwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, stage + tt * D);
+            }
+        }
+        const int t_end = t0 + nst;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *c = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[jj];
+        }
+    }
+    flush((ntile - 1) * kTile);
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) W[(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[jj];
+    if (sl == 0) hstate[seq * D + col] = hcur;
+}
+
+// ----------------------------------------------------------------- backward
+
+template <int D>
+struct RnnBwdOps {
+    float k[Geo<D>::NP], u[Geo<D>::NP], s[Geo<D>::NP];
+    float go_i, s_i, k_i, d_i, b;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_rnn_bwd_reg(
+    fwp_view k, fwp_view beta, const float *__restrict__ vdiff, const float *__restrict__ out,
+    const float *__restrict__ h_init, fwp_view go, const float *__restrict__ ckpt,
+    float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv,
+    float *__restrict__ gbeta, int H, int L, int chunk, int nchunk, int nseq) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sgo_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sd_[WPB][2][kTile * D];
+    __shared__ __align__(16) float su_[WPB][2][kTile * D];
+    __shared__ __align__(16) float ss_[WPB][2][kTile * D];   // softmax of the delayed output
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float spd_[WPB][kTile * D];
+    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gz, gk, gv tiles
+
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sk = sk_[wave];
+    auto &sgo = sgo_[wave];
+    auto &sd = sd_[wave];
+    auto &su = su_[wave];
+    auto &ss = ss_[wave];
+    auto &sb = sb_[wave];
+    auto &spd = spd_[wave];
+    auto &sgrad = sgrad_[wave];
+    const float *kb = row(k, n, h, 0), *gob = row(go, n, h, 0), *bb = row(beta, n, h, 0);
+    const float *db = vdiff + seq * L * D, *ob = out + seq * L * D, *hib = h_init + seq * D;
+
+    // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
+    float Wr[R], Gr[R], Gc[R], Wnext[R];
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Gr[jj] = Gc[jj] = Wr[jj] = 0.f;
+    float dh_i = 0.f;   // gradient carried to the previous output, entry i
+
+    TileRegs<D> pk, pgo, pd, pu, ps;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane = kb + lrow * k.sL + 4 * lc4, *golane = gob + lrow * go.sL + 4 * lc4,
+                *dlane = db + lrow * D + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+            pd.template fetch<true>(dlane, D, t0, L, lane);
+        } else {
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+            pd.template fetch<false>(dlane, D, t0, L, lane);
+        }
+        float bs[NV4];
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            const int t = t0 + lrow + TileRegs<D>::kRowsPerLoad * x;
+            bs[x] = bb[(int64_t)min(t, L - 1) * beta.sL];
+            // row t of the delayed output is out[t-1], or the initial state for t = 0
+            const float *src = t == 0 ? hib + 4 * lc4 : ob + (int64_t)(min(t, L) - 1) * D + 4 * lc4;
+            ps.r[x] = *reinterpret_cast<const float4 *>(src);
+        }
+        pu = pd;
+        pu.scale_rows(bs);
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+    };
+    auto commit = [&](int buf) {
+        pk.commit(sk[buf], lane);
+        pgo.commit(sgo[buf], lane);
+        pd.commit(sd[buf], lane);
+        pu.commit(su[buf], lane);
+        sb[buf][per] = pb;
+        // softmax of each row of the delayed output, off the sequential path
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            float4 &r = ps.r[x];
+            const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
+            r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
+            const float inv = 1.f / row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum());
+            r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
+        }
+        ps.commit(ss[buf], lane);
+    };
+    auto fetch_state = [&](int c) {
+        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
+    };
+
+    // S = 4: s=0 -> gz, s=1 -> gk, s=2,3 -> gv.   S = 2: s=0 -> gz, s=1 -> gk, and a second write for gv.
+    float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
+    float *dst2 = sgrad[2] + i;
+    float *gz_rows = gz + seq * L * D, *gk_rows = gk + seq * L * D, *gv_rows = gv + seq * L * D;
+
+    auto load_ops = [&](RnnBwdOps<D> &o, int buf, int tt) {
+        const int off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.k[p] = sk[buf][off + 16 * p + per];
+            o.u[p] = su[buf][off + 16 * p + per];
+            o.s[p] = ss[buf][off + 16 * p + per];
+        }
+        o.go_i = sgo[buf][off + i];
+        o.s_i = ss[buf][off + i];
+        o.k_i = sk[buf][off + i];
+        o.d_i = sd[buf][off + i];
+        o.b = sb[buf][tt];
+    };
+    auto compute = [&](const RnnBwdOps<D> &o, int tt) {
+        const float g_i = dh_i + o.go_i;                      // gradient of h_t = grad_z
+        float g[NP], a[NP];
+        to_periodic<D>(g_i, g, lane);
+        // G' = G + s (x) g (both layouts);  r = G'^T k
+        rank1_rot<D>(Gc, o.s, g_i);
+        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        const float gv_i = o.b * r_i;
+        const float a_i = -gv_i;                              // gradient w.r.t. v_old
+        to_periodic<D>(a_i, a, lane);
+        spd[tt * D + i] = r_i * o.d_i;
+        rank1_rot<D>(Gr, g, o.s_i);
+        // gradient of s_t = W_t g, through the softmax to h_{t-1}
+        const float ds_i = group_sum<S>(dot_rot<D>(Wr, g));
+        const float dot = across_groups<S>(ds_i * o.s_i, OpSum());
+        dh_i = o.s_i * (ds_i - dot);
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                   // W_{t-1}
+        rank1_rot<D>(Gc, o.k, a_i);
+        float gk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
+        gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
+        rank1_rot<D>(Gr, a, o.k_i);
+        if constexpr (S == 4) {
+            dst1[tt * D] = sl == 0 ? g_i : (sl == 1 ? gk_i : gv_i);
+        } else {
+            dst1[tt * D] = sl == 0 ? g_i : gk_i;
+            dst2[tt * D] = gv_i;
+        }
+    };
+    auto flush = [&](int t0, int nst) {
+        flush_tile<D>(sgrad[0], gz_rows, t0, L, lane);
+        flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
+        flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
+        const int tt = lane / 4, part = lane % 4;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < D / 4; j += 4) {
+            const float4 x = *reinterpret_cast<const float4 *>(&spd[tt * D + part * (D / 4) + j]);
+            acc += (x.x + x.y) + (x.z + x.w);
+        }
+        acc = group_sum<4>(acc);
+        if (tt < nst) gbeta[seq * L + t0 + tt] = acc;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch((ntile - 1) * kTile);
+    commit((ntile - 1) & 1);
+    fetch_state(nchunk - 1);
+    if (ntile > 1) fetch((ntile - 2) * kTile);
+    RnnBwdOps<D> ring[RING];
+    bool primed = false;
+
+    for (int it = ntile - 1; it >= 0; it--) {
+        const int buf = it & 1, t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
+        }
+        if (it >= 1) commit(buf ^ 1);
+        if (it + 1 < ntile) flush(t0 + kTile, min(kTile, L - t0 - kTile));
+        if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
+        if (it >= 2) fetch(t0 - 2 * kTile);
+        if (nst == kTile) {
+            if (!primed) {
+#pragma unroll
+                for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
+                primed = true;
+            }
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                const int nt = tt - PF;
+                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
+                compute(ring[tt % RING], tt);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                RnnBwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt);
+            }
+        }
+    }
+    flush(0, min(kTile, L));
+}
+
+}  // namespace
+
+bool reg_rnn_supported(int D) { return D == 16 || D == 32; }
+
+int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
+                float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_rnn_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
+                           k, v, beta, W, h, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_rnn_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
+                           k, v, beta, W, h, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
+                const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
+                float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_rnn_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, k,
+                           beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
+                           nseq);
+    else
+        hipLaunchKernelGGL((k_rnn_bwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, k,
+                           beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
+                           nseq);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fwp
