@@ -129,6 +129,10 @@ int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float 
                       (vdiff != nullptr) + (ckpt != nullptr);
     if (saved != 0 && saved != 5) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    if (reg_rec_supported(D) && reg_view_ok(qx) && reg_view_ok(kx) && reg_view_ok(vx) &&
+        aligned16(out) && aligned16(vdiff) && aligned16(q_act) && aligned16(k_act) && aligned16(ckpt))
+        return reg_rec_fwd(qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
+                           ckpt, N, H, L, D, chunk, (hipStream_t)stream);
     return generic_rec_fwd(qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act,
                            vdiff, ckpt, N, H, L, D, chunk, (hipStream_t)stream);
 }
@@ -144,7 +148,14 @@ int fwp_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
         !grb || !workspace)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
-    int rc = generic_rec_bwd(q_act, k_act, beta_act, vdiff, out, h_init, grad_out, Rq, Rk, Rv, rb,
+    int rc;
+    if (reg_rec_supported(D) && reg_view_ok(grad_out) && aligned16(q_act) && aligned16(k_act) &&
+        aligned16(vdiff) && aligned16(out) && aligned16(h_init) && aligned16(gqx) && aligned16(gkx) &&
+        aligned16(gvx))
+        rc = reg_rec_bwd(q_act, k_act, beta_act, vdiff, out, h_init, grad_out, Rq, Rk, Rv, rb, ckpt,
+                         gqx, gkx, gvx, gbx, workspace, N, H, L, D, chunk, (hipStream_t)stream);
+    else
+        rc = generic_rec_bwd(q_act, k_act, beta_act, vdiff, out, h_init, grad_out, Rq, Rk, Rv, rb,
                              ckpt, gqx, gkx, gvx, gbx, workspace, N, H, L, D, chunk,
                              (hipStream_t)stream);
     if (rc) return rc;

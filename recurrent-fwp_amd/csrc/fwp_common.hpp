@@ -57,6 +57,17 @@ int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                 const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
                 float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s);
 
+bool reg_rec_supported(int D);
+int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,
+                float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,
+                int H, int L, int D, int chunk, hipStream_t s);
+int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, const float *vdiff,
+                const float *out, const float *h_init, fwp_view go, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, const float *ckpt, float *gqx,
+                float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
+                int chunk, hipStream_t s);
+
 // Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 

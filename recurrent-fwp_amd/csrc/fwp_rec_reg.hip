@@ -1,0 +1,461 @@
+// Register-state kernels of the Recurrent Delta Net op (rec_update_fwm_tanh) for D in {16, 32}.
+//
+// On top of the delta-rule state, the slow recurrent matrices R_q, R_k, R_v of the head are held
+// in VGPRs in the same layout as the state (by columns in forward, by rows in backward, where the
+// three gradient accumulators of R_* live in VGPRs too and are written out once per sequence).
+// Per step the fed-back vector tanh(out_{t-1}) and the activated q and k are "grouped" vectors
+// (every lane of group m holds entry m) that become periodic operands through ds_bpermute; the
+// softmax maxima/sums, the beta logit and the softmax-Jacobian dot products are wave-wide
+// reductions (DPP row rotates + two row swaps).
+#include "fwp_reg.hpp"
+
+namespace fwp {
+namespace {
+
+__device__ __forceinline__ float fast_tanh(float x) {
+    return 1.f - __fdividef(2.f, 1.f + __expf(2.f * x));
+}
+__device__ __forceinline__ float fast_sigmoid(float x) {
+    return __fdividef(1.f, 1.f + __expf(-x));
+}
+
+// ------------------------------------------------------------------ forward
+
+template <int D>
+struct RecFwdOps {
+    float qx, kx, vx, bx;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
+    fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *__restrict__ Rq,
+    const float *__restrict__ Rk, const float *__restrict__ Rv, const float *__restrict__ rb,
+    float *__restrict__ W, float *__restrict__ hstate, float *__restrict__ out,
+    float *__restrict__ q_act, float *__restrict__ k_act, float *__restrict__ beta_act,
+    float *__restrict__ vdiff, float *__restrict__ ckpt, int H, int L, int chunk, int nchunk,
+    int nseq) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sq_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sv_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float sout_[WPB][4][kTile * D + 16];   // staged out, vdiff, q, k tiles
+    __shared__ __align__(16) float sba_[WPB][kTile];                // staged beta after the sigmoid
+
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sq = sq_[wave];
+    auto &sk = sk_[wave];
+    auto &sv = sv_[wave];
+    auto &sb = sb_[wave];
+    auto &sout = sout_[wave];
+    auto &sba = sba_[wave];
+    const float *qb = row(qx, n, h, 0), *kb = row(kx, n, h, 0), *vb = row(vx, n, h, 0),
+                *bb = row(bx, n, h, 0);
+
+    // column `col` of the state and of the head's three recurrent matrices
+    float Wc[R], Rqc[R], Rkc[R], Rvc[R];
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) {
+        const int e = reg_index<D>(lane, jj);
+        Wc[jj] = W[(seq * D + e) * D + col];
+        Rqc[jj] = Rq[((int64_t)h * D + e) * D + col];
+        Rkc[jj] = Rk[((int64_t)h * D + e) * D + col];
+        Rvc[jj] = Rv[((int64_t)h * D + e) * D + col];
+    }
+    const float rb_m = rb[(int64_t)h * D + col];
+    float hcur = hstate[seq * D + col];
+
+    TileRegs<D> pq, pk, pv;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *qlane = qb + lrow * qx.sL + 4 * lc4, *klane = kb + lrow * kx.sL + 4 * lc4,
+                *vlane = vb + lrow * vx.sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pq.template fetch<true>(qlane, qx.sL, t0, L, lane);
+            pk.template fetch<true>(klane, kx.sL, t0, L, lane);
+            pv.template fetch<true>(vlane, vx.sL, t0, L, lane);
+        } else {
+            pq.template fetch<false>(qlane, qx.sL, t0, L, lane);
+            pk.template fetch<false>(klane, kx.sL, t0, L, lane);
+            pv.template fetch<false>(vlane, vx.sL, t0, L, lane);
+        }
+        pb = bb[(int64_t)min(t0 + per, L - 1) * bx.sL];
+    };
+    auto commit = [&](int buf) {
+        pq.commit(sq[buf], lane);
+        pk.commit(sk[buf], lane);
+        pv.commit(sv[buf], lane);
+        sb[buf][per] = pb;
+    };
+
+    // S = 4: one LDS write per step, s = 0..3 -> out, vdiff, q, k.  S = 2: two writes.
+    float *stage1 = sout[sl] + col;                      // s=0 -> out, s=1 -> vdiff (S=4: s=2 -> q, s=3 -> k)
+    float *stage2 = sout[2 + (sl & 1)] + col;            // S=2 only: s=0 -> q, s=1 -> k
+    const bool save = vdiff != nullptr;
+    float *out_rows = out + seq * L * D;
+    auto flush = [&](int t0) {
+        flush_tile<D>(sout[0], out_rows, t0, L, lane);
+        if (save) {
+            flush_tile<D>(sout[1], vdiff + seq * L * D, t0, L, lane);
+            flush_tile<D>(sout[2], q_act + seq * L * D, t0, L, lane);
+            flush_tile<D>(sout[3], k_act + seq * L * D, t0, L, lane);
+            const float b = sba[per];
+            if (lane < kTile && t0 + lane < L) beta_act[seq * L + t0 + lane] = b;
+        }
+    };
+
+    auto load_ops = [&](RecFwdOps<D> &o, int buf, int tt) {
+        o.qx = sq[buf][tt * D + col];
+        o.kx = sk[buf][tt * D + col];
+        o.vx = sv[buf][tt * D + col];
+        o.bx = sb[buf][tt];
+    };
+    auto compute = [&](const RecFwdOps<D> &o, int tt) {
+        const float y_m = fast_tanh(hcur);
+        float y[NP], kp[NP], qp[NP];
+        to_periodic<D>(y_m, y, lane);
+        const float qa = o.qx + group_sum<S>(dot_rot<D>(Rqc, y));
+        const float ka = o.kx + group_sum<S>(dot_rot<D>(Rkc, y));
+        const float va = o.vx + group_sum<S>(dot_rot<D>(Rvc, y));
+        const float b = fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum()));
+        const float eq = __expf(qa - across_groups<S>(qa, OpMax()));
+        const float ek = __expf(ka - across_groups<S>(ka, OpMax()));
+        const float q_m = __fdividef(eq, across_groups<S>(eq, OpSum()));
+        const float k_m = __fdividef(ek, across_groups<S>(ek, OpSum()));
+        to_periodic<D>(k_m, kp, lane);
+        to_periodic<D>(q_m, qp, lane);
+        const float d = va - group_sum<S>(dot_rot<D>(Wc, kp));
+        rank1_rot<D>(Wc, kp, b * d);
+        hcur = group_sum<S>(dot_rot<D>(Wc, qp));
+        if constexpr (S == 4) {
+            stage1[tt * D] = sl == 0 ? hcur : (sl == 1 ? d : (sl == 2 ? q_m : k_m));
+        } else {
+            stage1[tt * D] = sl == 0 ? hcur : d;
+            stage2[tt * D] = sl == 0 ? q_m : k_m;
+        }
+        sba[tt] = b;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch(0);
+    commit(0);
+    if (ntile > 1) fetch(kTile);
+    RecFwdOps<D> ring[RING];
+#pragma unroll
+    for (int p = 0; p < PF; p++) load_ops(ring[p], 0, p);
+
+    for (int it = 0; it < ntile; it++) {
+        const int buf = it & 1, t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        if (it + 1 < ntile) commit(buf ^ 1);
+        if (it > 0) flush(t0 - kTile);
+        if (it + 2 < ntile) fetch(t0 + 2 * kTile);
+        if (nst == kTile) {
+#pragma unroll
+            for (int tt = 0; tt < kTile; tt++) {
+                const int nt = tt + PF;
+                if (nt < kTile) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[nt % RING], buf ^ 1, nt - kTile);
+                compute(ring[tt % RING], tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                RecFwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt);
+            }
+        }
+        const int t_end = t0 + nst;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *c = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[jj];
+        }
+    }
+    flush((ntile - 1) * kTile);
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) W[(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[jj];
+    if (sl == 0) hstate[seq * D + col] = hcur;
+}
+
+// ----------------------------------------------------------------- backward
+
+template <int D>
+struct RecBwdOps {
+    float q[Geo<D>::NP], k[Geo<D>::NP], u[Geo<D>::NP];
+    float q_i, k_i, go_i, d_i, y_i, b;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
+    const float *__restrict__ q_act, const float *__restrict__ k_act,
+    const float *__restrict__ beta_act, const float *__restrict__ vdiff,
+    const float *__restrict__ out, const float *__restrict__ h_init, fwp_view go,
+    const float *__restrict__ Rq, const float *__restrict__ Rk, const float *__restrict__ Rv,
+    const float *__restrict__ rb, const float *__restrict__ ckpt, float *__restrict__ gqx,
+    float *__restrict__ gkx, float *__restrict__ gvx, float *__restrict__ gbx,
+    float *__restrict__ workspace, int H, int L, int chunk, int nchunk, int nseq) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sq_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sgo_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sd_[WPB][2][kTile * D];
+    __shared__ __align__(16) float su_[WPB][2][kTile * D];
+    __shared__ __align__(16) float sy_[WPB][2][kTile * D];   // tanh of the delayed output
+    __shared__ __align__(16) float sb_[WPB][2][kTile];
+    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gqx, gkx, gvx tiles
+    __shared__ __align__(16) float sgb_[WPB][kTile];                 // staged gbx
+
+    const int wave = threadIdx.x / kWave;
+    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int h = (int)(seq % H), n = (int)(seq / H);
+    auto &sq = sq_[wave];
+    auto &sk = sk_[wave];
+    auto &sgo = sgo_[wave];
+    auto &sd = sd_[wave];
+    auto &su = su_[wave];
+    auto &sy = sy_[wave];
+    auto &sb = sb_[wave];
+    auto &sgrad = sgrad_[wave];
+    auto &sgb = sgb_[wave];
+    const float *gob = row(go, n, h, 0);
+    const float *qb = q_act + seq * L * D, *kb = k_act + seq * L * D, *db = vdiff + seq * L * D,
+                *ob = out + seq * L * D, *hib = h_init + seq * D, *bb = beta_act + seq * L;
+
+    // row i of: the state, its gradient (also column i of it), the recurrent matrices and their gradients
+    float Wr[R], Gr[R], Gc[R], Wnext[R], Rqr[R], Rkr[R], Rvr[R], gRq[R], gRk[R], gRv[R];
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) {
+        const int m = reg_index<D>(lane, jj);
+        Gr[jj] = Gc[jj] = Wr[jj] = gRq[jj] = gRk[jj] = gRv[jj] = 0.f;
+        Rqr[jj] = Rq[((int64_t)h * D + i) * D + m];
+        Rkr[jj] = Rk[((int64_t)h * D + i) * D + m];
+        Rvr[jj] = Rv[((int64_t)h * D + i) * D + m];
+    }
+    const float rb_i = rb[(int64_t)h * D + i];
+    float grb_i = 0.f, dh_i = 0.f;
+
+    TileRegs<D> pq, pk, pgo, pd, pu, py;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *qlane = qb + lrow * D + 4 * lc4, *klane = kb + lrow * D + 4 * lc4,
+                *dlane = db + lrow * D + 4 * lc4, *golane = gob + lrow * go.sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pq.template fetch<true>(qlane, D, t0, L, lane);
+            pk.template fetch<true>(klane, D, t0, L, lane);
+            pd.template fetch<true>(dlane, D, t0, L, lane);
+            pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+        } else {
+            pq.template fetch<false>(qlane, D, t0, L, lane);
+            pk.template fetch<false>(klane, D, t0, L, lane);
+            pd.template fetch<false>(dlane, D, t0, L, lane);
+            pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+        }
+        float bs[NV4];
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            const int t = t0 + lrow + TileRegs<D>::kRowsPerLoad * x;
+            bs[x] = bb[min(t, L - 1)];
+            // row t of the delayed output is out[t-1], or the initial state for t = 0
+            const float *src = t == 0 ? hib + 4 * lc4 : ob + (int64_t)(min(t, L) - 1) * D + 4 * lc4;
+            py.r[x] = *reinterpret_cast<const float4 *>(src);
+        }
+        pu = pd;
+        pu.scale_rows(bs);
+        pb = bb[min(t0 + per, L - 1)];
+    };
+    auto commit = [&](int buf) {
+        pq.commit(sq[buf], lane);
+        pk.commit(sk[buf], lane);
+        pgo.commit(sgo[buf], lane);
+        pd.commit(sd[buf], lane);
+        pu.commit(su[buf], lane);
+        sb[buf][per] = pb;
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            float4 &r = py.r[x];
+            r.x = fast_tanh(r.x); r.y = fast_tanh(r.y); r.z = fast_tanh(r.z); r.w = fast_tanh(r.w);
+        }
+        py.commit(sy[buf], lane);
+    };
+    auto fetch_state = [&](int c) {
+        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
+    };
+
+    // S = 4: s=0 -> gqx, s=1 -> gkx, s=2,3 -> gvx.   S = 2: s=0 -> gqx, s=1 -> gkx, second write gvx.
+    float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
+    float *dst2 = sgrad[2] + i;
+    float *gq_rows = gqx + seq * L * D, *gk_rows = gkx + seq * L * D, *gv_rows = gvx + seq * L * D;
+
+    auto load_ops = [&](RecBwdOps<D> &o, int buf, int tt) {
+        const int off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.q[p] = sq[buf][off + 16 * p + per];
+            o.k[p] = sk[buf][off + 16 * p + per];
+            o.u[p] = su[buf][off + 16 * p + per];
+        }
+        o.q_i = sq[buf][off + i];
+        o.k_i = sk[buf][off + i];
+        o.go_i = sgo[buf][off + i];
+        o.d_i = sd[buf][off + i];
+        o.y_i = sy[buf][off + i];
+        o.b = sb[buf][tt];
+    };
+    auto compute = [&](const RecBwdOps<D> &o, int tt) {
+        const float g_i = dh_i + o.go_i;                      // gradient of out_t
+        float g[NP], a[NP], gqp[NP], gkp[NP], gvp[NP];
+        to_periodic<D>(g_i, g, lane);
+        // gradient of q (after softmax) = W_t g, then through the softmax
+        const float dq_i = group_sum<S>(dot_rot<D>(Wr, g));
+        // G' = G + q (x) g (both layouts);  r = G'^T k
+        rank1_rot<D>(Gc, o.q, g_i);
+        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        const float gqx_i = o.q_i * (dq_i - across_groups<S>(dq_i * o.q_i, OpSum()));
+        const float gvx_i = o.b * r_i;
+        const float a_i = -gvx_i;                             // gradient w.r.t. v_old
+        to_periodic<D>(a_i, a, lane);
+        const float gb = across_groups<S>(r_i * o.d_i, OpSum());
+        const float gbx_t = gb * o.b * (1.f - o.b);           // through the sigmoid
+        rank1_rot<D>(Gr, g, o.q_i);
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                   // W_{t-1}
+        rank1_rot<D>(Gc, o.k, a_i);
+        float dk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
+        dk_i = group_sum<S>(dot_rot<D>(Wr, a, dk_i));
+        rank1_rot<D>(Gr, a, o.k_i);
+        const float gkx_i = o.k_i * (dk_i - across_groups<S>(dk_i * o.k_i, OpSum()));
+        // back through the slow recurrent weights to tanh(out_{t-1}) and to out_{t-1}
+        to_periodic<D>(gqx_i, gqp, lane);
+        to_periodic<D>(gkx_i, gkp, lane);
+        to_periodic<D>(gvx_i, gvp, lane);
+        float acc = dot_rot<D>(Rqr, gqp);
+        acc = dot_rot<D>(Rkr, gkp, acc);
+        acc = group_sum<S>(dot_rot<D>(Rvr, gvp, acc));
+        acc = fmaf(rb_i, gbx_t, acc);
+        dh_i = (1.f - o.y_i * o.y_i) * acc;
+        rank1_rot<D>(gRq, gqp, o.y_i);
+        rank1_rot<D>(gRk, gkp, o.y_i);
+        rank1_rot<D>(gRv, gvp, o.y_i);
+        grb_i = fmaf(o.y_i, gbx_t, grb_i);
+        if constexpr (S == 4) {
+            dst1[tt * D] = sl == 0 ? gqx_i : (sl == 1 ? gkx_i : gvx_i);
+        } else {
+            dst1[tt * D] = sl == 0 ? gqx_i : gkx_i;
+            dst2[tt * D] = gvx_i;
+        }
+        sgb[tt] = gbx_t;
+    };
+    auto flush = [&](int t0) {
+        flush_tile<D>(sgrad[0], gq_rows, t0, L, lane);
+        flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
+        flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
+        const float x = sgb[per];
+        if (lane < kTile && t0 + lane < L) gbx[seq * L + t0 + lane] = x;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch((ntile - 1) * kTile);
+    commit((ntile - 1) & 1);
+    fetch_state(nchunk - 1);
+    if (ntile > 1) fetch((ntile - 2) * kTile);
+    RecBwdOps<D> ring[RING];
+    bool primed = false;
+
+    for (int it = ntile - 1; it >= 0; it--) {
+        const int buf = it & 1, t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
+        }
+        if (it >= 1) commit(buf ^ 1);
+        if (it + 1 < ntile) flush(t0 + kTile);
+        if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
+        if (it >= 2) fetch(t0 - 2 * kTile);
+        if (nst == kTile) {
+            if (!primed) {
+#pragma unroll
+                for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
+                primed = true;
+            }
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                const int nt = tt - PF;
+                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
+                compute(ring[tt % RING], tt);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                RecBwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt);
+            }
+        }
+    }
+    flush(0);
+    // this sequence's share of the parameter gradients: [gRq | gRk | gRv | grb], rows e, columns m
+    float *ws = workspace + seq * (3 * D * D + D);
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) {
+        const int m = reg_index<D>(lane, jj);
+        ws[i * D + m] = gRq[jj];
+        ws[D * D + i * D + m] = gRk[jj];
+        ws[2 * D * D + i * D + m] = gRv[jj];
+    }
+    if (sl == 0) ws[3 * D * D + i] = grb_i;
+}
+
+}  // namespace
+
+bool reg_rec_supported(int D) { return D == 16 || D == 32; }
+
+int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,
+                float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,
+                int H, int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_rec_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
+                           ckpt, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
+                           ckpt, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, const float *vdiff,
+                const float *out, const float *h_init, fwp_view go, const float *Rq,
+                const float *Rk, const float *Rv, const float *rb, const float *ckpt, float *gqx,
+                float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
+                int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_rec_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
+                           gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_rec_bwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
+                           gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fwp
