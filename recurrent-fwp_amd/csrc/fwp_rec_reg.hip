@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
     __shared__ __align__(16) float sout_[WPB][4][kTile * D + 16];   // staged out, vdiff, q, k tiles
     __shared__ __align__(16) float sba_[WPB][kTile];                // staged beta after the sigmoid
 
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
     const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
     const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
     if (seq >= nseq) return;
@@ -134,11 +134,13 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
         const float d = va - group_sum<S>(dot_rot<D>(Wc, kp));
         rank1_rot<D>(Wc, kp, b * d);
         hcur = group_sum<S>(dot_rot<D>(Wc, qp));
+        hcur = pinned(hcur);
+        const float o_d = pinned(d), o_q = pinned(q_m), o_k = pinned(k_m);
         if constexpr (S == 4) {
-            stage1[tt * D] = sl == 0 ? hcur : (sl == 1 ? d : (sl == 2 ? q_m : k_m));
+            stage1[tt * D] = sl == 0 ? hcur : (sl == 1 ? o_d : (sl == 2 ? o_q : o_k));
         } else {
-            stage1[tt * D] = sl == 0 ? hcur : d;
-            stage2[tt * D] = sl == 0 ? q_m : k_m;
+            stage1[tt * D] = sl == 0 ? hcur : o_d;
+            stage2[tt * D] = sl == 0 ? o_q : o_k;
         }
         sba[tt] = b;
     };
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
     __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gqx, gkx, gvx tiles
     __shared__ __align__(16) float sgb_[WPB][kTile];                 // staged gbx
 
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
     const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
     const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
     if (seq >= nseq) return;
@@ -351,11 +353,12 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
         rank1_rot<D>(gRk, gkp, o.y_i);
         rank1_rot<D>(gRv, gvp, o.y_i);
         grb_i = fmaf(o.y_i, gbx_t, grb_i);
+        const float o_q = pinned(gqx_i), o_k = pinned(gkx_i), o_v = pinned(gvx_i);
         if constexpr (S == 4) {
-            dst1[tt * D] = sl == 0 ? gqx_i : (sl == 1 ? gkx_i : gvx_i);
+            dst1[tt * D] = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
         } else {
-            dst1[tt * D] = sl == 0 ? gqx_i : gkx_i;
-            dst2[tt * D] = gvx_i;
+            dst1[tt * D] = sl == 0 ? o_q : o_k;
+            dst2[tt * D] = o_v;
         }
         sgb[tt] = gbx_t;
     };

@@ -131,6 +131,25 @@ __device__ __forceinline__ void flush_tile(const float *tile, float *dst_rows, i
 }
 
 
+// Value held by the lane with sub-index sp of the caller's own group (a DPP quad broadcast that
+// the compiler folds into the consuming instruction).  A register loaded as "lane (g,s) holds the
+// value of step S*j + s" thus serves S consecutive steps.
+template <int S>
+__device__ __forceinline__ float group_pick(float x, int sp) {
+    if constexpr (S == 2) {
+        return sp == 0 ? dpp<0xA0>(x) : dpp<0xF5>(x);          // quad_perm:[0,0,2,2] / [1,1,3,3]
+    } else if constexpr (S == 4) {
+        switch (sp) {
+            case 0: return dpp<0x00>(x);
+            case 1: return dpp<0x55>(x);
+            case 2: return dpp<0xAA>(x);
+            default: return dpp<0xFF>(x);
+        }
+    } else {
+        return x;
+    }
+}
+
 // Periodic copy of a grouped vector: lane l gets y[16*p + l % 16] in out[p].
 template <int D>
 __device__ __forceinline__ void to_periodic(float y, float (&out)[Geo<D>::NP], int lane) {

@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
     __shared__ __align__(16) float sb_[WPB][2][kTile];
     __shared__ __align__(16) float sout_[WPB][2][kTile * D + 16];
 
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
     const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
     const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
     if (seq >= nseq) return;
@@ -102,7 +102,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
         const float d = o.v - group_sum<S>(dot_rot<D>(Wc, o.k));
         rank1_rot<D>(Wc, o.k, o.b * d);
         hcur = group_sum<S>(dot_rot<D>(Wc, s)) + o.z;
-        *o_ptr = store_d ? d : hcur;
+        hcur = pinned(hcur);
+        *o_ptr = store_d ? pinned(d) : hcur;
     };
 
     const int ntile = (L + kTile - 1) / kTile;
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_bwd_reg(
     __shared__ __align__(16) float spd_[WPB][kTile * D];
     __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gz, gk, gv tiles
 
-    const int wave = threadIdx.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
     const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
     const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
     if (seq >= nseq) return;
@@ -286,11 +287,12 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_bwd_reg(
         float gk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
         gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
         rank1_rot<D>(Gr, a, o.k_i);
+        const float o_z = pinned(g_i), o_k = pinned(gk_i), o_v = pinned(gv_i);
         if constexpr (S == 4) {
-            dst1[tt * D] = sl == 0 ? g_i : (sl == 1 ? gk_i : gv_i);
+            dst1[tt * D] = sl == 0 ? o_z : (sl == 1 ? o_k : o_v);
         } else {
-            dst1[tt * D] = sl == 0 ? g_i : gk_i;
-            dst2[tt * D] = gv_i;
+            dst1[tt * D] = sl == 0 ? o_z : o_k;
+            dst2[tt * D] = o_v;
         }
     };
     auto flush = [&](int t0, int nst) {

@@ -42,6 +42,14 @@ __device__ __forceinline__ void swap32(float &a, float &b) {
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
 
+// Forces x to be computed by every lane at this point.  Values that come out of cross-lane
+// operations must not be left for the compiler to compute lazily inside a lane-dependent select:
+// it may then run the cross-lane operation with part of the wave masked off.
+__device__ __forceinline__ float pinned(float x) {
+    asm volatile("" : "+v"(x));
+    return x;
+}
+
 struct OpSum {
     __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
