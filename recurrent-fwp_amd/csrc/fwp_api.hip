@@ -15,7 +15,7 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 int check_dims(int N, int H, int L, int E, int M, int chunk) {
     if (N < 1 || H < 1 || L < 1 || E < 1 || M < 1) return FWP_E_SHAPE;
-    if (chunk < kTile || chunk % kTile != 0) return FWP_E_CHUNK;
+    if (chunk < kChunkQuantum || chunk % kChunkQuantum != 0) return FWP_E_CHUNK;
     if ((int64_t)E * M > fwp_query(FWP_Q_MAX_STATE_FLOATS)) return FWP_E_TOO_LARGE;
     return 0;
 }
@@ -41,7 +41,7 @@ const char *fwp_strerror(int code) {
 int fwp_query(int what) {
     switch (what) {
         case FWP_Q_VERSION: return 1;
-        case FWP_Q_CHUNK_QUANTUM: return kTile;
+        case FWP_Q_CHUNK_QUANTUM: return kChunkQuantum;
         case FWP_Q_DEFAULT_CHUNK: return kDefaultChunk;
         case FWP_Q_MAX_STATE_FLOATS: return 16384;
         default: return -1;

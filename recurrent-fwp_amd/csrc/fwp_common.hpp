@@ -9,6 +9,8 @@ namespace fwp {
 // Length of the LDS input tiles of the register-state kernels.  The state
 // checkpoint interval (`chunk` of the C ABI) must be a multiple of it.
 constexpr int kTile = 16;
+// The state checkpoint interval (`chunk` of the C ABI) must be a multiple of this (the longest tile).
+constexpr int kChunkQuantum = 32;
 constexpr int kDefaultChunk = 64;
 
 __device__ __forceinline__ const float *row(const fwp_view &v, int n, int h, int t) {

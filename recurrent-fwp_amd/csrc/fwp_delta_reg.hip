@@ -42,11 +42,8 @@ __device__ __forceinline__ void tile_row_dots(const TileRegs<D> &a, const TileRe
 // ------------------------------------------------------------------ forward
 
 template <int D>
-struct FwdOps {      // per step: the periodic operands
-    float k[Geo<D>::NP], q[Geo<D>::NP];
-};
-struct FwdGroupOps { // per S steps: lane (g,s) holds v[col], beta and k.q of step S*j + s
-    float v, b, kq;
+struct FwdOps {
+    float k[Geo<D>::NP], q[Geo<D>::NP], v, b, kq;
 };
 
 template <int D, int RING, int PF, int WPB>
@@ -131,22 +128,19 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
             o.k[p] = sk[buf][tt * D + 16 * p + per];
             o.q[p] = sq[buf][tt * D + 16 * p + per];
         }
-    };
-    auto load_group = [&](FwdGroupOps &o, int buf, int grp) {
-        const int t = grp * S + sl;
-        o.v = sv[buf][t * D + col];
-        o.b = sb[buf][t];
-        o.kq = skq[buf][t];
+        o.v = sv[buf][tt * D + col];
+        o.b = sb[buf][tt];
+        o.kq = skq[buf][tt];
     };
     // out_t = W_t^T q = W_{t-1}^T q + u (k.q): both mat-vecs read the old state, so their
     // dependent DPP sums overlap instead of running one after the other
-    auto compute = [&](const FwdOps<D> &o, const FwdGroupOps &go, int sp, float *o_ptr) {
+    auto compute = [&](const FwdOps<D> &o, float *o_ptr) {
         const float p_old = group_sum<S>(dot_rot<D>(Wc, o.k));
         const float p_out = group_sum<S>(dot_rot<D>(Wc, o.q));
-        const float d = group_pick<S>(go.v, sp) - p_old;
-        const float u = group_pick<S>(go.b, sp) * d;
+        const float d = o.v - p_old;
+        const float u = o.b * d;
         rank1_rot<D>(Wc, o.k, u);
-        const float res = pinned(fmaf(group_pick<S>(go.kq, sp), u, p_out));
+        const float res = pinned(fmaf(u, o.kq, p_out));
         *o_ptr = store_d ? d : res;
     };
 
@@ -155,10 +149,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     commit(0);
     if (ntile > 1) fetch(kTile);
     FwdOps<D> ring[RING];
-    FwdGroupOps gring[2];
 #pragma unroll
     for (int p = 0; p < PF; p++) load_ops(ring[p], 0, p);
-    load_group(gring[0], 0, 0);
 
     for (int it = 0; it < ntile; it++) {
         const int buf = it & 1, t0 = it * kTile;
@@ -173,20 +165,13 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
                 const int nt = tt + PF;
                 if (nt < kTile) load_ops(ring[nt % RING], buf, nt);
                 else load_ops(ring[nt % RING], buf ^ 1, nt - kTile);
-                if (tt % S == 0) {   // the next group of S steps, possibly the first of the next tile
-                    const int ng = tt / S + 1;
-                    if (ng < kTile / S) load_group(gring[ng % 2], buf, ng);
-                    else load_group(gring[ng % 2], buf ^ 1, 0);
-                }
-                compute(ring[tt % RING], gring[(tt / S) % 2], tt % S, tile_dst + tt * D);
+                compute(ring[tt % RING], tile_dst + tt * D);
             }
         } else {  // ragged last tile: not pipelined
             for (int tt = 0; tt < nst; tt++) {
                 FwdOps<D> o;
-                FwdGroupOps go;
                 load_ops(o, buf, tt);
-                load_group(go, buf, tt / S);
-                compute(o, go, tt % S, tile_dst + tt * D);
+                compute(o, tile_dst + tt * D);
             }
         }
         const int t_end = t0 + nst;
@@ -204,10 +189,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
 // ----------------------------------------------------------------- backward
 
 template <int D>
-struct BwdOps {      // per step: the periodic operands
+struct BwdOps {
     float q[Geo<D>::NP], k[Geo<D>::NP], go[Geo<D>::NP], u[Geo<D>::NP];
-};
-struct BwdGroupOps { // per S steps: lane (g,s) holds entry g of q, k, grad_out, vdiff and beta of step S*j + s
     float q_i, k_i, go_i, d_i, b;
 };
 
@@ -310,35 +293,28 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
             o.go[p] = sgo[buf][off + 16 * p + per];
             o.u[p] = su[buf][off + 16 * p + per];
         }
-    };
-    auto load_group = [&](BwdGroupOps &o, int buf, int grp) {
-        const int t = grp * S + sl, off = t * D;
         o.q_i = sq[buf][off + i];
         o.k_i = sk[buf][off + i];
         o.go_i = sgo[buf][off + i];
         o.d_i = sd[buf][off + i];
-        o.b = sb[buf][t];
+        o.b = sb[buf][tt];
     };
-    auto compute = [&](const BwdOps<D> &o, const BwdGroupOps &gp, int tt) {
-        const int sp = tt % S;
-        const float q_i = group_pick<S>(gp.q_i, sp), k_i = group_pick<S>(gp.k_i, sp),
-                    go_i = group_pick<S>(gp.go_i, sp), d_i = group_pick<S>(gp.d_i, sp),
-                    b = group_pick<S>(gp.b, sp);
+    auto compute = [&](const BwdOps<D> &o, int tt) {
         // G' = G + q (x) go (both layouts);  r = G'^T k
-        rank1_rot<D>(Gc, o.q, go_i);
+        rank1_rot<D>(Gc, o.q, o.go_i);
         const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
-        const float gv_i = b * r_i;
+        const float gv_i = o.b * r_i;
         const float a_i = -gv_i;                              // gradient w.r.t. v_old
         float a[NP];
         to_periodic<D>(a_i, a, lane);
-        spd[tt * D + i] = r_i * d_i;
-        rank1_rot<D>(Gr, o.go, q_i);
+        spd[tt * D + i] = r_i * o.d_i;
+        rank1_rot<D>(Gr, o.go, o.q_i);
         const float gq_i = group_sum<S>(dot_rot<D>(Wr, o.go));   // (W_t go)[i]
-        rank1_rot<D, true>(Wr, o.u, k_i);                         // W_{t-1}
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                       // W_{t-1}
         rank1_rot<D>(Gc, o.k, a_i);
         float gk_i = dot_rot<D>(Gr, o.u);                         // G' u + W_{t-1} a
         gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
-        rank1_rot<D>(Gr, a, k_i);
+        rank1_rot<D>(Gr, a, o.k_i);
         const float o_q = pinned(gq_i), o_k = pinned(gk_i), o_v = pinned(gv_i);
         if constexpr (S == 4) {
             dst1[tt * D] = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
@@ -370,7 +346,6 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     fetch_state(nchunk - 1);
     if (ntile > 1) fetch((ntile - 2) * kTile);
     BwdOps<D> ring[RING];
-    BwdGroupOps gring[2];
     bool primed = false;
 
     for (int it = ntile - 1; it >= 0; it--) {
@@ -389,7 +364,6 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
             if (!primed) {
 #pragma unroll
                 for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
-                load_group(gring[(kTile / S - 1) % 2], buf, kTile / S - 1);
                 primed = true;
             }
 #pragma unroll
@@ -397,20 +371,13 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
                 const int nt = tt - PF;
                 if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
                 else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
-                if (tt % S == S - 1) {   // the next (earlier) group of S steps, possibly of the next tile
-                    const int ng = tt / S - 1;
-                    if (ng >= 0) load_group(gring[ng % 2], buf, ng);
-                    else load_group(gring[(kTile / S - 1) % 2], buf ^ 1, kTile / S - 1);
-                }
-                compute(ring[tt % RING], gring[(tt / S) % 2], tt);
+                compute(ring[tt % RING], tt);
             }
         } else {  // ragged last tile (first in reverse): not pipelined
             for (int tt = nst - 1; tt >= 0; tt--) {
                 BwdOps<D> o;
-                BwdGroupOps gp;
                 load_ops(o, buf, tt);
-                load_group(gp, buf, tt / S);
-                compute(o, gp, tt);
+                compute(o, tt);
             }
         }
     }

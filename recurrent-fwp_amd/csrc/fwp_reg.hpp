@@ -16,13 +16,13 @@
 
 namespace fwp {
 
-template <int D>
+template <int D, int TL = kTile>
 struct Geo {
     static constexpr int S = kWave / D;                // lanes per group
     static constexpr int NP = D / 16;                  // periodic registers per D-vector
     static constexpr int NR = 16 / S;                  // rotations per periodic register
     static constexpr int R = NP * NR;                  // state entries per lane (= D / S)
-    static constexpr int NV4 = kTile * D / 4 / kWave;  // float4 per lane per tile tensor
+    static constexpr int NV4 = TL * D / 4 / kWave;     // float4 per lane per tile tensor (tile of TL steps)
     static_assert(D * S == kWave && NV4 >= 1, "D must be 16 or 32");
 };
 
@@ -88,16 +88,17 @@ __device__ __forceinline__ void rank1_rot(float (&w)[Geo<D>::R], const float (&x
 }
 
 // One tile of one [.,D] tensor on its way from HBM to LDS.
-template <int D>
+template <int D, int TL = kTile>
 struct TileRegs {
-    float4 r[Geo<D>::NV4];
+    static constexpr int NV4 = Geo<D, TL>::NV4;
+    float4 r[NV4];
     // lane_base points at this lane's first float4 of the sequence: row lane / (D/4), column
     // 4 * (lane % (D/4)); the i-th float4 of a tile is kWave / (D/4) rows further down.
     static constexpr int kRowsPerLoad = kWave / (D / 4);
     template <bool FULL>
     __device__ __forceinline__ void fetch(const float *lane_base, int64_t sL, int t0, int L, int lane) {
 #pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++) {
+        for (int i = 0; i < NV4; i++) {
             const int rw = t0 + lane / (D / 4) + kRowsPerLoad * i;
             const float4 *src = reinterpret_cast<const float4 *>(lane_base + (int64_t)(t0 + kRowsPerLoad * i) * sL);
             if constexpr (FULL) r[i] = *src;
@@ -106,12 +107,12 @@ struct TileRegs {
     }
     __device__ __forceinline__ void commit(float *tile, int lane) const {
 #pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++)
+        for (int i = 0; i < NV4; i++)
             *reinterpret_cast<float4 *>(tile + 4 * (lane + kWave * i)) = r[i];
     }
     __device__ __forceinline__ void scale_rows(const float *rowscale) {
 #pragma unroll
-        for (int i = 0; i < Geo<D>::NV4; i++) {
+        for (int i = 0; i < NV4; i++) {
             const float b = rowscale[i];
             r[i].x *= b; r[i].y *= b; r[i].z *= b; r[i].w *= b;
         }
@@ -148,6 +149,56 @@ __device__ __forceinline__ float group_pick(float x, int sp) {
     } else {
         return x;
     }
+}
+
+// NT tiles held in registers go to LDS interleaved: entry (row, col) of tensor n lands at
+// dst[(row * D + col) * NT + n], so that ONE NT-dword LDS read fetches that entry of every tensor
+// (a lone wave pays per LDS instruction, not per byte).  Same number of 16-byte writes as NT
+// separate commits.
+template <int D, int TL>
+__device__ __forceinline__ void commit_interleaved(float *dst, const TileRegs<D, TL> &a,
+                                                   const TileRegs<D, TL> &b, int lane) {
+#pragma unroll
+    for (int i = 0; i < Geo<D, TL>::NV4; i++) {
+        float4 *o = reinterpret_cast<float4 *>(dst + 8 * (lane + kWave * i));
+        o[0] = make_float4(a.r[i].x, b.r[i].x, a.r[i].y, b.r[i].y);
+        o[1] = make_float4(a.r[i].z, b.r[i].z, a.r[i].w, b.r[i].w);
+    }
+}
+template <int D, int TL>
+__device__ __forceinline__ void commit_interleaved(float *dst, const TileRegs<D, TL> &a,
+                                                   const TileRegs<D, TL> &b,
+                                                   const TileRegs<D, TL> &c,
+                                                   const TileRegs<D, TL> &d, int lane) {
+#pragma unroll
+    for (int i = 0; i < Geo<D, TL>::NV4; i++) {
+        float4 *o = reinterpret_cast<float4 *>(dst + 16 * (lane + kWave * i));
+        o[0] = make_float4(a.r[i].x, b.r[i].x, c.r[i].x, d.r[i].x);
+        o[1] = make_float4(a.r[i].y, b.r[i].y, c.r[i].y, d.r[i].y);
+        o[2] = make_float4(a.r[i].z, b.r[i].z, c.r[i].z, d.r[i].z);
+        o[3] = make_float4(a.r[i].w, b.r[i].w, c.r[i].w, d.r[i].w);
+    }
+}
+
+// NT staged tiles go to HBM together: all LDS reads first, then all 16-byte stores.
+template <int D, int TL, int NT, bool FULL>
+__device__ __forceinline__ void flush_tiles(const float *const (&tile)[NT], float *const (&rows)[NT],
+                                            int t0, int L, int lane) {
+    constexpr int NV4 = Geo<D, TL>::NV4;
+    float4 x[NT][NV4];
+#pragma unroll
+    for (int n = 0; n < NT; n++)
+#pragma unroll
+        for (int i = 0; i < NV4; i++)
+            x[n][i] = *reinterpret_cast<const float4 *>(tile[n] + 4 * (lane + kWave * i));
+#pragma unroll
+    for (int n = 0; n < NT; n++)
+#pragma unroll
+        for (int i = 0; i < NV4; i++) {
+            const int f = lane + kWave * i, rw = f / (D / 4), c4 = f % (D / 4);
+            if (FULL || t0 + rw < L)
+                *reinterpret_cast<float4 *>(rows[n] + (int64_t)(t0 + rw) * D + 4 * c4) = x[n][i];
+        }
 }
 
 // Periodic copy of a grouped vector: lane l gets y[16*p + l % 16] in out[p].
