@@ -23,6 +23,11 @@ METRIC = "fast-weight update tokens/s (fwd+bwd), % of FP32-VALU roofline, 1 GPU"
 PEAK_VALU = 157.3e12     # MI355X fp32 vector peak (packed), FLOP/s
 PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
 
+# HBM bytes per launch of the forward / backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch; FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by what the same counters read
+# for a 2 GiB device-to-device copy, `--copy-calibration`).
+MEASURED_TRAFFIC = {'delta': {'fwd': 68600000.0, 'bwd': 93000000.0}, 'rnn': {'fwd': 97500000.0, 'bwd': 127400000.0}, 'rec': {'fwd': 132100000.0, 'bwd': 150800000.0}}
+
 # name -> (B, H, T, D, algorithmic flops per token-head = c*D^2, fwd bytes, bwd bytes per token-head)
 WORKLOADS = {
     "delta": dict(B=96, H=8, T=256, D=16, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
@@ -237,14 +242,14 @@ def main():
     ap.add_argument("--graph", action="store_true",
                     help="time a HIP graph replay of the step recorded through the C ABI instead of eager calls")
     ap.add_argument("--copy-calibration", action="store_true",
-                    help="only run ten device-to-device copies of 256 MiB (a kernel of known traffic for "
+                    help="only run five device-to-device copies of 2 GiB (a kernel of known traffic for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
     if args.copy_calibration:
         import torch
-        src = torch.ones(64 * 1024 * 1024, device="cuda:0")
+        src = torch.ones(512 * 1024 * 1024, device="cuda:0")      # 2 GiB: far beyond every cache level
         dst = torch.empty_like(src)
-        for _ in range(10):
+        for _ in range(5):
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
@@ -315,7 +320,7 @@ def main():
         "config": {"workload": w["label"], "B": B, "H": H, "T": T, "D": D, "launch": launch},
         "roofline": {"bound": "hbm", "kernel": f"{name} {dom}", "achieved": dom_bytes / dom_t / 1e9,
                      "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": dom_bytes / dom_t / PEAK_HBM,
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom)},
         "kernels": {"fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
                     "fwd_GBps": fwd_bytes / t_f / 1e9, "bwd_GBps": bwd_bytes / t_b / 1e9,
                     "kernel_only_tokens_per_s": tokens / kernel_s,

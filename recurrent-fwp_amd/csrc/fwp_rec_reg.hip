@@ -438,7 +438,7 @@ int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float 
                            qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
                            ckpt, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+        hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
                            qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
                            ckpt, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
@@ -455,7 +455,7 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
                            q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
                            gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL((k_rec_bwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+        hipLaunchKernelGGL((k_rec_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
                            q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
                            gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();

@@ -365,7 +365,7 @@ int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, flo
         hipLaunchKernelGGL((k_rnn_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
                            k, v, beta, W, h, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL((k_rnn_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
+        hipLaunchKernelGGL((k_rnn_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, z,
                            k, v, beta, W, h, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
@@ -379,7 +379,7 @@ int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                            beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
                            nseq);
     else
-        hipLaunchKernelGGL((k_rnn_bwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, k,
+        hipLaunchKernelGGL((k_rnn_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, k,
                            beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
                            nseq);
     return (int)hipGetLastError();
