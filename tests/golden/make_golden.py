@@ -27,7 +27,7 @@ def f64(arrays):
 
 
 def main():
-    # BASELINE config 1: B=2,H=2,T=64,D=16, W0=0, seed 0
+    # the CPU-runnable benchmark configuration: B=2,H=2,T=64,D=16, W0=0, seed 0
     q, k, v, beta, W0, go = f32(delta_inputs(0, 2, 2, 64, 16, 16))
     out, W = oracle.delta_fwd(*f64([q, k, v, beta, W0]))
     gq, gk, gv, gb, _ = oracle.delta_bwd(*f64([q, k, v, beta, W0, go]))

@@ -1,0 +1,97 @@
+"""Benchmark-size checks through properties that do not need an oracle run of that size:
+carried-state segment splits, linearity in the values, batch/head permutation, determinism."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import delta_inputs, rec_inputs, rnn_inputs
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.asarray(a, np.float32)).cuda()
+
+
+def grads_of(fn, inputs, go):
+    ts = [t.clone().requires_grad_(True) for t in inputs]
+    out = fn(ts)
+    return out.detach(), torch.autograd.grad(out, ts, go)
+
+
+def test_delta_full_size_properties(fwp):
+    # LM-small shape of the benchmark: B=96,H=8,T=256,D=16
+    q, k, v, beta, W0, go = (dev(a) for a in delta_inputs(0, 96, 8, 256, 16, 16, dtype=np.float32))
+
+    def run(qq, kk, vv, bb, w0):
+        W = w0.clone()
+        return fwp.fast_weight_delta(qq, kk, vv, bb, W), W
+
+    out, W = run(q, k, v, beta, W0)
+    assert torch.isfinite(out).all()
+    # a split at a position that is not a tile boundary, state carried over
+    a, b = slice(0, 100), slice(100, 256)
+    o1, W1 = run(q[:, :, a], k[:, :, a], v[:, :, a], beta[:, :, a], W0)
+    o2, W2 = run(q[:, :, b], k[:, :, b], v[:, :, b], beta[:, :, b], W1)
+    assert torch.equal(torch.cat([o1, o2], 2), out) and torch.equal(W2, W)
+    # linear in (v, W0)
+    v2 = torch.randn_like(v)
+    o_b, _ = run(q, k, v2, beta, W0)
+    o_c, _ = run(q, k, 2 * v - 3 * v2, beta, W0)
+    assert torch.allclose(o_c, 2 * out - 3 * o_b, atol=2e-4, rtol=1e-3)
+    # batch permutation
+    perm = torch.randperm(96, device="cuda")
+    o_p, W_p = run(q[perm], k[perm], v[perm], beta[perm], W0[perm])
+    assert torch.equal(o_p, out[perm]) and torch.equal(W_p, W[perm])
+    # gradients: deterministic, and the gradient of sum(out * go) w.r.t. v is linear in go
+    _, g1 = grads_of(lambda t: fwp.fast_weight_delta(*t, W0.clone()), [q, k, v, beta], go)
+    _, g2 = grads_of(lambda t: fwp.fast_weight_delta(*t, W0.clone()), [q, k, v, beta], go)
+    for x, y in zip(g1, g2):
+        assert torch.isfinite(x).all() and torch.equal(x, y)
+    _, g3 = grads_of(lambda t: fwp.fast_weight_delta(*t, W0.clone()), [q, k, v, beta], 2 * go)
+    assert torch.allclose(g3[2], 2 * g1[2], atol=1e-5, rtol=1e-5)
+
+
+def test_rnn_full_size_properties(fwp):
+    z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(1, 64, 8, 256, 32, dtype=np.float32))
+
+    def run(sl, w0, hh):
+        W, h = w0.clone(), hh.clone()
+        out = fwp.fast_rnn_v2(z[:, :, sl], k[:, :, sl], v[:, :, sl], W, beta[:, :, sl], h)
+        return out, W, h
+
+    out, W, h = run(slice(0, 256), W0, h0)
+    assert torch.isfinite(out).all() and torch.equal(h[:, :, 0], out[:, :, -1])
+    o1, W1, h1 = run(slice(0, 70), W0, h0)
+    o2, W2, h2 = run(slice(70, 256), W1, h1)
+    assert torch.equal(torch.cat([o1, o2], 2), out) and torch.equal(W2, W) and torch.equal(h2, h)
+    _, g1 = grads_of(lambda t: fwp.fast_rnn_v2(t[0], t[1], t[2], W0.clone(), t[3], h0.clone()), [z, k, v, beta], go)
+    _, g2 = grads_of(lambda t: fwp.fast_rnn_v2(t[0], t[1], t[2], W0.clone(), t[3], h0.clone()), [z, k, v, beta], go)
+    for x, y in zip(g1, g2):
+        assert torch.isfinite(x).all() and torch.equal(x, y)
+    assert torch.equal(g1[0][:, :, -1], go[:, :, -1])      # grad_z of the last step is the upstream gradient
+
+
+def test_rec_full_size_properties(fwp):
+    *x, go = (dev(a) for a in rec_inputs(2, 64, 8, 256, 32, dtype=np.float32))
+    qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0 = x
+
+    def run(sl, w0, hh):
+        W, h = w0.clone(), hh.clone()
+        out = fwp.rec_update_fwm_tanh(qx[:, :, sl], kx[:, :, sl], vx[:, :, sl], bx[:, :, sl], R_q, R_k, R_v, r_b, W, h)
+        return out, W, h
+
+    out, W, h = run(slice(0, 256), W0, h0)
+    assert torch.isfinite(out).all()
+    o1, W1, h1 = run(slice(0, 130), W0, h0)
+    o2, W2, h2 = run(slice(130, 256), W1, h1)
+    assert torch.equal(torch.cat([o1, o2], 2), out) and torch.equal(W2, W) and torch.equal(h2, h)
+    fn = lambda t: fwp.rec_update_fwm_tanh(*t, W0.clone(), h0.clone())
+    _, g1 = grads_of(fn, x[:8], go)
+    _, g2 = grads_of(fn, x[:8], go)
+    for a, b in zip(g1, g2):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+    # the softmax Jacobian annihilates constants: grad_qx and grad_kx sum to zero over D
+    scale = g1[0].abs().max().item()
+    assert g1[0].sum(-1).abs().max().item() <= 1e-4 * max(scale, 1.0)
+    assert g1[1].sum(-1).abs().max().item() <= 1e-4 * max(g1[1].abs().max().item(), 1.0)

@@ -88,6 +88,7 @@ def test_delta_no_grad_path(fwp):
 
 
 RNN_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 64, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
+              (3, 5, 40, 32, True), (1, 3, 100, 16, True),
               (2, 3, 77, 8, True), (1, 1, 19, 5, True)]
 
 
@@ -107,6 +108,7 @@ def test_rnn(fwp, N, H, L, D, w0):
 
 
 REC_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 32, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
+              (1, 3, 100, 16, True),
               (2, 3, 77, 8, True), (1, 1, 19, 5, True), (1, 2, 30, 64, False)]
 
 
@@ -124,6 +126,26 @@ def test_rec(fwp, N, H, L, D, w0):
     names = "qx kx vx bx R_q R_k R_v r_b".split()
     for name, t, r in zip(names, ts, oracle.rec_bwd(*x, go)):
         check("grad_" + name, t.grad, r)
+
+
+def test_rnn_and_rec_take_strided_views(fwp):
+    # inputs as the layers pass them: [L,N,H,*] storage permuted to [N,H,L,*]
+    def lnh(x):
+        return dev(np.ascontiguousarray(x.transpose(2, 0, 1, 3))).permute(1, 2, 0, 3)
+    z, k, v, W0, beta, h0, go = rnn_inputs(11, 2, 3, 40, 32, w0=True)
+    ts = [lnh(a).requires_grad_(True) for a in (z, k, v, beta)]
+    out = fwp.fast_rnn_v2(ts[0], ts[1], ts[2], dev(W0), ts[3], dev(h0))
+    out.backward(lnh(go))
+    check("rnn out", out, oracle.rnn_fwd(z, k, v, W0, beta, h0)[0])
+    for t, r in zip(ts, oracle.rnn_bwd(z, k, v, W0, beta, h0, go)):
+        check("rnn grad", t.grad, r)
+    *x, go = rec_inputs(12, 2, 3, 40, 32, w0=True)
+    ts = [lnh(a).requires_grad_(True) for a in x[:4]] + [dev(a, True) for a in x[4:8]]
+    out = fwp.rec_update_fwm_tanh(*ts, dev(x[8]), dev(x[9]))
+    out.backward(lnh(go))
+    check("rec out", out, oracle.rec_fwd(*x)[0])
+    for t, r in zip(ts, oracle.rec_bwd(*x, go)):
+        check("rec grad", t.grad, r)
 
 
 def test_deterministic(fwp):
