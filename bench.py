@@ -33,6 +33,10 @@ WORKLOADS = {
     "delta": dict(B=96, H=8, T=256, D=16, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
                   bwd_bytes=lambda D: (7 * D + 2) * 4,
                   label="delta-rule fast_weight fwd+bwd, B=96 H=8 T=256 D=16, fp32"),
+    "delta_lm": dict(B=32, H=8, T=1024, D=32, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
+                     bwd_bytes=lambda D: (7 * D + 2) * 4,
+                     label="delta-rule fast_weight fwd+bwd at the shape one layer of the 16-layer LM gives it, "
+                           "B=32 H=8 T=1024 D=32, fp32"),
     "rnn": dict(B=64, H=8, T=256, D=32, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
                 bwd_bytes=lambda D: (8 * D + 2) * 4,
                 label="Delta RNN fast_rnn_v2 fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
@@ -46,7 +50,7 @@ def make_inputs(name, w):
     import numpy as np
     from helpers import delta_inputs, rec_inputs, rnn_inputs
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
-    if name == "delta":
+    if name.startswith("delta"):
         return delta_inputs(0, B, H, T, D, D, dtype=np.float32)
     if name == "rnn":
         return rnn_inputs(0, B, H, T, D, dtype=np.float32)
@@ -58,7 +62,7 @@ def gpu_step_fn(name, pkg, arrays):
     import torch
     dev = [torch.from_numpy(a).to("cuda:0") for a in arrays]
     go = dev[-1]
-    if name == "delta":
+    if name.startswith("delta"):
         q, k, v, beta, W0 = dev[:5]
         diff = [t.requires_grad_(True) for t in (q, k, v, beta)]
         W = W0.clone()
@@ -108,7 +112,7 @@ def kernel_times(name, pkg, arrays, iters):
     def view(t):
         return L.View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 
-    if name == "delta":
+    if name.startswith("delta"):
         q, k, v, beta, W0 = dev[:5]
         N, H, T, E = q.shape
         M = v.shape[-1]
@@ -193,7 +197,7 @@ def kernel_times(name, pkg, arrays, iters):
     def abi_step():
         """state reset + forward + backward, straight through the C ABI on preallocated buffers"""
         W.zero_()
-        if name != "delta":
+        if not name.startswith("delta"):
             h.zero_()
         L.check(fwd(), "forward")
         L.check(bwd(), "backward")
@@ -212,7 +216,7 @@ def cpu_baseline(name, arrays, w, reps):
     torch.set_num_threads(cores)
     ts = [torch.from_numpy(a) for a in arrays]
     go = ts[-1]
-    if name == "delta":
+    if name.startswith("delta"):
         loop, inputs, idx = torch_loop.delta_loop, ts[:5], [0, 1, 2, 3]
     elif name == "rnn":
         loop, inputs, idx = torch_loop.rnn_v2_loop, ts[:6], [0, 1, 2, 4]
@@ -231,12 +235,108 @@ def cpu_baseline(name, arrays, w, reps):
                       f"({med * 1e3:.0f} ms each)"}
 
 
+LM_CONFIG = dict(n_token=32768, n_layer=16, n_head=8, d_model=256, d_head=32, d_inner=1024)
+LM_BATCH, LM_LEN = 32, 1024
+
+
+def zipf_tokens(n_token, shape, s=1.1, seed=0):
+    """i.i.d. draws from Zipf(s) truncated to the vocabulary: P(rank r) ~ r^-s."""
+    import numpy as np
+    p = np.arange(1, n_token + 1, dtype=np.float64) ** -s
+    cdf = np.cumsum(p / p.sum())
+    u = np.random.default_rng(seed).random(shape)
+    return np.minimum(np.searchsorted(cdf, u), n_token - 1).astype(np.int64)
+
+
+def run_lm(args, pkg):
+    """Forward + backward of the 16-layer Delta-Net language model (random init, Zipf tokens): the
+    operator measured where the reference uses it.  Reports whole-model tokens/s and the share of the
+    step spent in the fast-weight kernels (timed on their own at the shape the layers give them)."""
+    import torch
+    torch.manual_seed(0)
+    model = pkg.DeltaNetLM(**LM_CONFIG).to("cuda:0")
+    toks = torch.from_numpy(zipf_tokens(LM_CONFIG["n_token"], (LM_LEN + 1, LM_BATCH))).to("cuda:0")
+    data, target = toks[:-1], toks[1:]
+    params = [p for p in model.parameters()]
+    torch.autograd.set_multithreading_enabled(False)
+
+    def step():
+        (loss,) = model(data, target)
+        grads = torch.autograd.grad(loss.mean(), params)
+        return loss, grads
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        loss, _ = step()
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+    tokens = LM_BATCH * LM_LEN
+
+    w = WORKLOADS["delta_lm"]
+    t_f, t_b, _ = kernel_times("delta_lm", pkg, make_inputs("delta_lm", w), 20)
+    D, th = w["D"], w["B"] * w["H"] * w["T"]
+    op_s = LM_CONFIG["n_layer"] * (t_f + t_b)
+    dom_t, dom_bytes = (t_b, w["bwd_bytes"](D) * th) if t_b >= t_f else (t_f, w["fwd_bytes"](D) * th)
+    result = {
+        "metric": "Delta-Net LM training tokens/s (fwd+bwd), 1 GPU", "value": tokens / step_s, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_s * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic (Zipf(1.1) tokens, random-init weights)",
+        "config": {"workload": "16-layer Delta-Net LM fwd+bwd, d_model=256 H=8 D=32 FFN=1024 vocab=32768, "
+                               "B=32 T=1024, fp32", **LM_CONFIG, "B": LM_BATCH, "T": LM_LEN},
+        "loss": float(loss.mean()),
+        "roofline": {"bound": "hbm", "kernel": "delta bwd at B=32 H=8 T=1024 D=32",
+                     "achieved": dom_bytes / dom_t / 1e9, "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": dom_bytes / dom_t / PEAK_HBM, "traffic": None},
+        "fast_weight_op": {"fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6, "per_step_ms": op_s * 1e3,
+                           "share_of_step": op_s / step_s},
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = lm_cpu_baseline(pkg)
+    return result
+
+
+def lm_cpu_baseline(pkg):
+    """The same model with the PyTorch step loop as operator on the host cores, on a slice of the batch."""
+    import torch
+    from oracle.torch_loop import delta_loop
+    cores = os.cpu_count() or 1
+    env = os.environ.get("OMP_NUM_THREADS")
+    if env and env.isdigit():
+        cores = min(cores, int(env))
+    torch.set_num_threads(cores)
+
+    def loop_op(q, k, v, beta, W):
+        out, W_end = delta_loop(q, k, v, beta, W.clone())
+        W.copy_(W_end.detach())
+        return out
+
+    torch.manual_seed(0)
+    model = pkg.DeltaNetLM(fast_weight_op=loop_op, **LM_CONFIG)
+    B, T = 4, 128
+    toks = torch.from_numpy(zipf_tokens(LM_CONFIG["n_token"], (T + 1, B)))
+    params = list(model.parameters())
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        (loss,) = model(toks[:-1], toks[1:])
+        torch.autograd.grad(loss.mean(), params)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times[1:])
+    return {"value": B * T / med, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"the same 16-layer model, B={B} T={T} slice, PyTorch step loop as operator, fwd+bwd, "
+                      f"median of 2 runs after a warm-up ({med:.1f} s each)"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS), default="delta")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["lm"], default="delta")
     ap.add_argument("--cpu-reps", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--graph", action="store_true",
@@ -263,6 +363,9 @@ def main():
     pkg = package()
     pkg._lib.lib()                       # fails loudly if the HIP library is not built
     name = args.workload
+    if name == "lm":
+        print(json.dumps(run_lm(args, pkg)))
+        return
     w = WORKLOADS[name]
     arrays = make_inputs(name, w)
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]

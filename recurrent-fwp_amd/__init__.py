@@ -9,6 +9,9 @@ from . import _lib
 from .fast_weight import DeltaFastWeight, fast_weight_delta
 from .fast_weight_rnn_v2 import FastRNNv2, fast_rnn_v2
 from .rec_update_fwm_tanh import FastWeightRecUpdateTanh, rec_update_fwm_tanh
+from .layers import DeltaNetDecoderLayer, DeltaNetLayer, PositionalEmbedding, PositionwiseFF
+from .lm import DeltaNetLM
 
 __all__ = ["DeltaFastWeight", "fast_weight_delta", "FastRNNv2", "fast_rnn_v2",
-           "FastWeightRecUpdateTanh", "rec_update_fwm_tanh"]
+           "FastWeightRecUpdateTanh", "rec_update_fwm_tanh", "DeltaNetLayer",
+           "DeltaNetDecoderLayer", "PositionwiseFF", "PositionalEmbedding", "DeltaNetLM"]

@@ -95,12 +95,21 @@ def require_device(t):
 
 
 def rows(t):
-    """A view argument for a 4-D fp32 tensor; copies only if the last axis is strided."""
+    """A view argument for a 4-D fp32 tensor.
+
+    Permuted views are passed as they are.  A copy is made when the last axis is strided,
+    and when rows of a multiple of 4 floats are not 16-byte aligned (a slice of a wider
+    buffer, such as v inside a fused q|k|v|beta projection): one elementwise pass costs far
+    less than giving up the kernels that read rows with 16-byte loads.
+    """
     if t.dtype != torch.float32:
         raise FwpError(f"fast-weight operators are fp32 only, got {t.dtype}")
     if t.dim() != 4:
         raise FwpError(f"expected a 4-D [N,H,L,D] tensor, got {t.dim()}-D")
-    if t.shape[-1] != 1 and t.stride(-1) != 1:
+    d = t.shape[-1]
+    if d != 1 and t.stride(-1) != 1:
+        t = t.contiguous()
+    elif d % 4 == 0 and (t.data_ptr() % 16 or any(s % 4 for s in t.stride()[:3])):
         t = t.contiguous()
     return t, View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 

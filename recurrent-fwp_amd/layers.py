@@ -1,0 +1,131 @@
+"""The caller of ``fast_weight_delta`` in language modelling: the Delta-Net layer and the
+feed-forward block that follows it, with the module and parameter names of the reference
+(language_modeling/src/utils/cuda_fast_weight_layer.py:57-188, utils/model_utils.py:15-67)
+so a reference state_dict loads unchanged.  Everything except the fast-weight operator is
+stock PyTorch; the operator is the HIP one unless a caller passes another (tests do, to
+compare against a step-by-step loop).
+"""
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .fast_weight import fast_weight_delta
+
+
+class PositionalEmbedding(nn.Module):
+    """Sinusoidal embedding of a position sequence: ``[sin | cos]`` halves, shape
+    ``[len, 1, demb]`` (or ``[len, bsz, demb]``).  utils/model_utils.py:15-31."""
+
+    def __init__(self, demb):
+        super().__init__()
+        self.demb = demb
+        self.register_buffer("inv_freq", 10000.0 ** (-torch.arange(0.0, demb, 2.0) / demb))
+
+    def forward(self, pos_seq, bsz=None):
+        phase = pos_seq[:, None] * self.inv_freq[None, :]
+        emb = torch.cat((phase.sin(), phase.cos()), dim=-1).unsqueeze(1)
+        return emb if bsz is None else emb.expand(-1, bsz, -1)
+
+
+class PositionwiseFF(nn.Module):
+    """Linear-ReLU-Linear with residual and LayerNorm (after, or before when
+    ``pre_lnorm``).  utils/model_utils.py:34-67."""
+
+    def __init__(self, d_model, d_inner, dropout, pre_lnorm=False):
+        super().__init__()
+        self.d_model, self.d_inner, self.dropout, self.pre_lnorm = d_model, d_inner, dropout, pre_lnorm
+        self.CoreNet = nn.Sequential(
+            nn.Linear(d_model, d_inner), nn.ReLU(inplace=True), nn.Dropout(dropout),
+            nn.Linear(d_inner, d_model), nn.Dropout(dropout))
+        self.layer_norm = nn.LayerNorm(d_model)
+
+    def forward(self, inp):
+        if self.pre_lnorm:
+            return inp + self.CoreNet(self.layer_norm(inp))
+        return self.layer_norm(inp + self.CoreNet(inp))
+
+
+def sum_normalised_elu(x):
+    """``phi(x) = (elu(x) + 1) / sum_D(elu(x) + 1)``: positive features that sum to one
+    (cuda_fast_weight_layer.py:118-123)."""
+    x = F.elu(x) + 1.0
+    return x / x.sum(-1, keepdim=True)
+
+
+class DeltaNetLayer(nn.Module):
+    """Delta-rule linear-Transformer layer (the reference's
+    ``CudaFastWeightLinearTransformerLayer`` with its default
+    ``skip_attn_normalization=True``).
+
+    ``h`` is ``[len, bsz, d_model]``.  One projection gives q, k, v and a scalar
+    write strength per head; q and k go through :func:`sum_normalised_elu`, beta
+    through a sigmoid, and the fast weight memory ``W[bsz, n_head, D, D]`` (zero, or
+    ``mems[0]`` when a segment's state is carried over) is updated step by step by
+    ``fast_weight_delta``.  The read-out is scaled by ``1/sqrt(D)``, projected, and
+    added to the input with LayerNorm.  With ``carry_over_fast_weight`` the call
+    returns ``(output, (W_final, None))``.
+    """
+
+    def __init__(self, n_head, d_model, d_head, dropout=0.0, dropatt=0.0, pre_lnorm=False,
+                 layer_id=None, num_layer=None, fast_weight_op=None):
+        super().__init__()
+        self.n_head, self.d_model, self.d_head, self.dropout = n_head, d_model, d_head, dropout
+        self.layer_id, self.num_layer = layer_id, num_layer
+        self.qkvb_net = nn.Linear(d_model, n_head * (3 * d_head + 1), bias=False)
+        self.drop = nn.Dropout(dropout)
+        self.dropatt = nn.Dropout(dropatt)
+        self.o_net = nn.Linear(n_head * d_head, d_model, bias=False)
+        self.layer_norm = nn.LayerNorm(d_model)
+        self.scale = 1.0 / d_head ** 0.5
+        self.pre_lnorm = pre_lnorm
+        self.fast_weight_op = fast_weight_op or fast_weight_delta
+
+    def forward(self, h, attn_mask=None, mems=None, carry_over_fast_weight=False):
+        slen, bsz, _ = h.shape
+        H, D = self.n_head, self.d_head
+        x = self.layer_norm(h) if self.pre_lnorm else h
+        # The reference's pre-LN branch adds the normalised input back (it rebinds h, :100-104).
+        residual = x
+
+        qkvb = self.qkvb_net(x).view(slen, bsz, H, 3 * D + 1)
+        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in qkvb.split((D, D, D, 1), dim=-1))
+        q, k, beta = sum_normalised_elu(q), sum_normalised_elu(k), torch.sigmoid(beta)
+
+        if mems is None:
+            W = torch.zeros(bsz, H, D, D, device=h.device, dtype=h.dtype)
+        else:
+            if not carry_over_fast_weight:
+                raise ValueError("mems are only meaningful with carry_over_fast_weight=True")
+            # The last batch of an epoch may be smaller than the carried state.  The
+            # operator overwrites its state argument, so it gets storage of its own.
+            W = mems[0][:bsz].clone()
+
+        out = self.fast_weight_op(q, k, v, beta, W)                  # [bsz, H, slen, D]
+        out = (self.scale * out).permute(2, 0, 1, 3).reshape(slen, bsz, H * D)
+        out = residual + self.drop(self.o_net(out))
+        if not self.pre_lnorm:
+            out = self.layer_norm(out)
+        if carry_over_fast_weight:
+            return out, (W.detach(), None)
+        return out
+
+
+class DeltaNetDecoderLayer(nn.Module):
+    """Delta-Net layer followed by the feed-forward block (``DecoderLayer`` with
+    ``attn_type=24``, model_main.py:703-775); sub-module names ``dec_attn`` and
+    ``pos_ff`` as there."""
+
+    def __init__(self, n_head, d_model, d_head, d_inner, dropout=0.0, dropatt=0.0, pre_lnorm=False,
+                 layer_id=None, num_layer=None, fast_weight_op=None):
+        super().__init__()
+        self.dec_attn = DeltaNetLayer(n_head, d_model, d_head, dropout, dropatt, pre_lnorm,
+                                      layer_id, num_layer, fast_weight_op)
+        self.pos_ff = PositionwiseFF(d_model, d_inner, dropout, pre_lnorm)
+
+    def forward(self, dec_inp, dec_attn_mask=None, mems=None, carry_over_fast_weight=False):
+        out = self.dec_attn(dec_inp, attn_mask=dec_attn_mask, mems=mems,
+                            carry_over_fast_weight=carry_over_fast_weight)
+        if carry_over_fast_weight:
+            out, new_mem = out
+            return self.pos_ff(out), new_mem
+        return self.pos_ff(out)
