@@ -37,6 +37,9 @@ WORKLOADS = {
                      bwd_bytes=lambda D: (7 * D + 2) * 4,
                      label="delta-rule fast_weight fwd+bwd at the shape one layer of the 16-layer LM gives it, "
                            "B=32 H=8 T=1024 D=32, fp32"),
+    "sum": dict(B=96, H=8, T=256, D=16, flop_c=12, fwd_bytes=lambda D: 4 * D * 4,
+                bwd_bytes=lambda D: 7 * D * 4,
+                label="sum-rule fast_weight_sum (causal linear attention) fwd+bwd, B=96 H=8 T=256 D=16, fp32"),
     "rnn": dict(B=64, H=8, T=256, D=32, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
                 bwd_bytes=lambda D: (8 * D + 2) * 4,
                 label="Delta RNN fast_rnn_v2 fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
@@ -50,7 +53,7 @@ def make_inputs(name, w):
     import numpy as np
     from helpers import delta_inputs, rec_inputs, rnn_inputs
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
-    if name.startswith("delta"):
+    if name.startswith("delta") or name == "sum":
         return delta_inputs(0, B, H, T, D, D, dtype=np.float32)
     if name == "rnn":
         return rnn_inputs(0, B, H, T, D, dtype=np.float32)
@@ -70,6 +73,16 @@ def gpu_step_fn(name, pkg, arrays):
         def step():
             W.zero_()                     # W0 = 0 for every step of the benchmark
             out = pkg.fast_weight_delta(*diff, W)
+            torch.autograd.grad(out, diff, go)
+            return out
+    elif name == "sum":
+        q, k, v, _, W0 = dev[:5]
+        diff = [t.requires_grad_(True) for t in (q, k, v)]
+        W = W0.clone()
+
+        def step():
+            W.zero_()
+            out = pkg.fast_weight_sum(*diff, W)
             torch.autograd.grad(out, diff, go)
             return out
     elif name == "rnn":
@@ -129,6 +142,24 @@ def kernel_times(name, pkg, arrays, iters):
         def bwd():
             return lib.fwp_delta_bwd(view(q), view(k), view(beta), L.ptr(vdiff), view(go), L.ptr(ckpt), L.ptr(gq),
                                      L.ptr(gk), L.ptr(gv), L.ptr(gb), N, H, T, E, M, chunk, stream_of())
+        reset = lambda: W.copy_(W0)
+    elif name == "sum":
+        q, k, v, _, W0 = dev[:5]
+        N, H, T, E = q.shape
+        M = v.shape[-1]
+        nch = (T + chunk - 1) // chunk
+        W = W0.clone()
+        out = torch.empty_like(v)
+        ckpt = torch.empty((N, H, nch, E, M), **f32)
+        gq, gk, gv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+
+        def fwd():
+            return lib.fwp_sum_fwd(view(q), view(k), view(v), L.ptr(W), L.ptr(out), L.ptr(ckpt), N, H, T, E, M,
+                                   chunk, stream_of())
+
+        def bwd():
+            return lib.fwp_sum_bwd(view(q), view(k), view(v), view(go), L.ptr(ckpt), None, L.ptr(gq), L.ptr(gk),
+                                   L.ptr(gv), N, H, T, E, M, chunk, stream_of())
         reset = lambda: W.copy_(W0)
     elif name == "rnn":
         z, k, v, W0, beta, h0 = dev[:6]
@@ -197,7 +228,7 @@ def kernel_times(name, pkg, arrays, iters):
     def abi_step():
         """state reset + forward + backward, straight through the C ABI on preallocated buffers"""
         W.zero_()
-        if not name.startswith("delta"):
+        if name in ("rnn", "rec"):
             h.zero_()
         L.check(fwd(), "forward")
         L.check(bwd(), "backward")
@@ -218,6 +249,8 @@ def cpu_baseline(name, arrays, w, reps):
     go = ts[-1]
     if name.startswith("delta"):
         loop, inputs, idx = torch_loop.delta_loop, ts[:5], [0, 1, 2, 3]
+    elif name == "sum":
+        loop, inputs, idx = torch_loop.sum_loop, [ts[0], ts[1], ts[2], ts[4]], [0, 1, 2]
     elif name == "rnn":
         loop, inputs, idx = torch_loop.rnn_v2_loop, ts[:6], [0, 1, 2, 4]
     else:

@@ -82,6 +82,33 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff,
                   int chunk, void *stream);
 
 /*
+ * Sum update rule (causal linear attention) forward.  Replaces causal_dot_product
+ * (algorithmic/fast_transformers/causal_product_cuda.cu:99-141, kernel :15-96).
+ *   W += k (x) v ; out = W^T q per step.  q,k [N,H,L,E]  v [N,H,L,M]
+ *   W [N,H,E,M] in/out (the reference's carried-in `kv`)
+ *   out [N,H,L,M]; ckpt [N,H,nchunk,E,M] may be NULL if no backward follows.
+ */
+int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out,
+                float *ckpt, int N, int H, int L, int E, int M, int chunk,
+                void *stream);
+
+/*
+ * Sum update rule backward.  Replaces causal_dot_backward
+ * (algorithmic/fast_transformers/causal_product_cuda.cu:369-445, kernels :157-366)
+ * with one reverse pass.
+ *   W_init [N,H,E,M] or NULL: when given (the state W held before forward), it is
+ *   taken out of the state that grad_q is read from.  The reference's backward
+ *   starts that state at zero (:385), i.e. its grad_q never sees the carried-in
+ *   memory: pass the saved initial state to reproduce it, NULL for the gradient of
+ *   the recurrence as written.  With a zero initial state the two agree.
+ *   gq,gk [N,H,L,E]  gv [N,H,L,M]
+ */
+int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out,
+                const float *ckpt, const float *W_init, float *gq, float *gk,
+                float *gv, int N, int H, int L, int E, int M, int chunk,
+                void *stream);
+
+/*
  * Delta RNN v2 forward.  Replaces fast_rnn_v2_forward
  * (algorithmic/fast_weight_rnn_v2/fast_rnn_cuda.cu:233-293, kernel :25-229).
  *   z,k,v [N,H,L,D]  beta [N,H,L,1]  W [N,H,D,D] in/out  h [N,H,D] in/out

@@ -108,6 +108,34 @@ def delta_bwd(q, k, v, beta, W0, go):
     return gq, gk, gv, gb, gW0
 
 
+# ------------------------------------------------------------------ sum rule
+
+def sum_fwd(q, k, v, W0):
+    """out[N,H,L,M], W_L of the sum update rule W += k (x) v, out = W^T q."""
+    dt = np.asarray(q).dtype
+    q, k, v = _c(q, dt), _c(k, dt), _c(v, dt)
+    N, H, L, E = q.shape
+    M = v.shape[-1]
+    assert k.shape == (N, H, L, E) and v.shape == (N, H, L, M) and np.shape(W0) == (N, H, E, M)
+    W = _c(W0, dt).copy()
+    out = np.empty((N, H, L, M), dt)
+    _call("fwp_oracle_sum_fwd", dt, [q, k, v, W, out], [N, H, L, E, M])
+    return out, W
+
+
+def sum_bwd(q, k, v, W0, go, through_state=False):
+    """(gq, gk, gv).  ``through_state=False`` is what the reference computes: its grad_Q
+    leaves out the carried-in state W0; ``True`` is the gradient of the loop as written."""
+    dt = np.asarray(q).dtype
+    q, k, v, W0, go = (_c(x, dt) for x in (q, k, v, W0, go))
+    N, H, L, E = q.shape
+    M = v.shape[-1]
+    gq, gk, gv = np.empty_like(q), np.empty_like(k), np.empty_like(v)
+    _call("fwp_oracle_sum_bwd", dt, [q, k, v, W0, go, gq, gk, gv],
+          [N, H, L, E, M, int(bool(through_state))])
+    return gq, gk, gv
+
+
 # -------------------------------------------------------------- Delta RNN v2
 
 def rnn_fwd(z, k, v, W0, beta, h0):

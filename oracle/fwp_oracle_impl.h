@@ -9,6 +9,7 @@
  *                       (single step: language_modeling/src/utils/fast_weight.py:73-93)
  *   Delta RNN v2        algorithmic/fast_weight_rnn_v2/__init__.py:205-217
  *   Recurrent Delta Net algorithmic/rec_update_fwm_tanh/__init__.py:263-302
+ *   sum rule            algorithmic/fast_transformers/__init__.py:145-152
  *
  * The backward functions are the plain reverse-mode adjoint of those loops with
  * every intermediate state W_t kept in memory (what autograd does for the
@@ -147,6 +148,55 @@ void FN(fwp_oracle_delta_bwd)(const REAL *q, const REAL *k, const REAL *v,
         }
         if (gW0) memcpy(gW0 + (size_t)s * EM, gW, sizeof(REAL) * EM);
         free(Wall); free(dall); free(gW); free(tmp);
+    }
+}
+
+/* ---------------------------------------------------------------- sum rule */
+
+/* W += k (x) v ; out = W^T q  (the loop of the reference's self test,
+ * algorithmic/fast_transformers/__init__.py:149-152).  W in/out. */
+void FN(fwp_oracle_sum_fwd)(const REAL *q, const REAL *k, const REAL *v, REAL *W,
+                            REAL *out, int N, int H, int L, int E, int M) {
+#pragma omp parallel for schedule(static)
+    for (int s = 0; s < N * H; s++) {
+        REAL *Ws = W + (size_t)s * E * M;
+        for (int t = 0; t < L; t++) {
+            size_t r = (size_t)s * L + t;
+            for (int e = 0; e < E; e++)
+                for (int m = 0; m < M; m++) Ws[e * M + m] += k[r * E + e] * v[r * M + m];
+            FN(matTvec)(Ws, q + r * E, out + r * M, E, M);
+        }
+    }
+}
+
+/* Reverse-mode adjoint of the loop above.  gq_t = S_t go_t with S_t = B + sum_{s<=t} k_s (x) v_s,
+ * where the base B is W0 when through_state != 0 (the gradient of the loop as written) and 0
+ * otherwise: the reference's backward starts its forward-direction accumulator at zero
+ * (causal_product_cuda.cu:385) and so leaves the carried-in state out of grad_Q.
+ * gk_t = G_t v_t, gv_t = G_t^T k_t with G_t = sum_{s>=t} q_s (x) go_s. */
+void FN(fwp_oracle_sum_bwd)(const REAL *q, const REAL *k, const REAL *v, const REAL *W0,
+                            const REAL *go, REAL *gq, REAL *gk, REAL *gv, int N, int H,
+                            int L, int E, int M, int through_state) {
+#pragma omp parallel for schedule(static)
+    for (int s = 0; s < N * H; s++) {
+        size_t EM = (size_t)E * M;
+        REAL *S = (REAL *)calloc(EM, sizeof(REAL));
+        REAL *G = (REAL *)calloc(EM, sizeof(REAL));
+        if (through_state) memcpy(S, W0 + (size_t)s * EM, sizeof(REAL) * EM);
+        for (int t = 0; t < L; t++) {
+            size_t r = (size_t)s * L + t;
+            for (int e = 0; e < E; e++)
+                for (int m = 0; m < M; m++) S[e * M + m] += k[r * E + e] * v[r * M + m];
+            FN(matvec)(S, go + r * M, gq + r * E, E, M);
+        }
+        for (int t = L - 1; t >= 0; t--) {
+            size_t r = (size_t)s * L + t;
+            for (int e = 0; e < E; e++)
+                for (int m = 0; m < M; m++) G[e * M + m] += q[r * E + e] * go[r * M + m];
+            FN(matvec)(G, v + r * M, gk + r * E, E, M);
+            FN(matTvec)(G, k + r * E, gv + r * M, E, M);
+        }
+        free(S); free(G);
     }
 }
 

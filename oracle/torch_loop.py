@@ -37,6 +37,16 @@ def delta_loop(q, k, v, beta, W0):
     return torch.stack(outs, dim=2), W
 
 
+def sum_loop(q, k, v, W0):
+    """Sum update rule (algorithmic/fast_transformers/__init__.py:149-152). -> (out, W_L)."""
+    W = W0
+    outs = []
+    for t in range(q.shape[2]):
+        W = W + k[:, :, t].unsqueeze(-1) * v[:, :, t].unsqueeze(-2)
+        outs.append(_read(W, q[:, :, t]))
+    return torch.stack(outs, dim=2), W
+
+
 def rnn_v2_loop(z, k, v, W0, beta, h0):
     """Argument order of the reference op. -> (out[N,H,L,D], W_L, h_L[N,H,1,D])."""
     W = W0

@@ -28,6 +28,8 @@ _P, _I, _V = ctypes.c_void_p, ctypes.c_int, View
 _SIGNATURES = {
     "fwp_delta_fwd": [_V] * 4 + [_P] * 4 + [_I] * 6 + [_P],
     "fwp_delta_bwd": [_V] * 3 + [_P, _V, _P] + [_P] * 4 + [_I] * 6 + [_P],
+    "fwp_sum_fwd": [_V] * 3 + [_P] * 3 + [_I] * 6 + [_P],
+    "fwp_sum_bwd": [_V] * 4 + [_P] * 5 + [_I] * 6 + [_P],
     "fwp_rnn_fwd": [_V] * 4 + [_P] * 5 + [_I] * 5 + [_P],
     "fwp_rnn_bwd": [_V, _V, _P, _P, _P, _V, _P] + [_P] * 4 + [_I] * 5 + [_P],
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],

@@ -88,6 +88,31 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
                              chunk, (hipStream_t)stream);
 }
 
+int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+                int L, int E, int M, int chunk, void *stream) {
+    if (bad_view(q) || bad_view(k) || bad_view(v) || !W || !out) return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
+        aligned16(ckpt) && aligned16(out))
+        return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+    return generic_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
+}
+
+int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const float *ckpt,
+                const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E,
+                int M, int chunk, void *stream) {
+    if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(grad_out) || !ckpt || !gq || !gk || !gv)
+        return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
+        reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
+        aligned16(gk) && aligned16(gv))
+        return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
+                           (hipStream_t)stream);
+    return generic_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
+                           (hipStream_t)stream);
+}
+
 int fwp_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, void *stream) {
     if (bad_view(z) || bad_view(k) || bad_view(v) || bad_view(beta) || !W || !h || !out)

@@ -24,6 +24,11 @@ int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *
 int generic_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                       const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N,
                       int H, int L, int E, int M, int chunk, hipStream_t s);
+int generic_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N,
+                    int H, int L, int E, int M, int chunk, hipStream_t s);
+int generic_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+                    const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L,
+                    int E, int M, int chunk, hipStream_t s);
 int generic_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h,
                     float *out, float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
                     hipStream_t s);
@@ -51,6 +56,13 @@ int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
 int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                   int L, int D, int chunk, hipStream_t s);
+
+// Sum rule on the same kernels (no v_old, beta = 1).
+int reg_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+                int L, int D, int chunk, hipStream_t s);
+int reg_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+                const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int D,
+                int chunk, hipStream_t s);
 
 bool reg_rnn_supported(int D);
 int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,

@@ -16,6 +16,9 @@
 // v_old) permuted across groups, and the partial products of grad beta that are
 // summed once per tile.
 //
+// The sum rule (W += k (x) v, no v_old, no beta) runs on the same kernels with SUM = true: the
+// delta rule with beta = 1 and the v_old terms taken out.
+//
 // q/k/v/beta (grad_out, vdiff) stream through double-buffered LDS tiles of kTile
 // steps, fetched from HBM two tiles ahead with 16-byte loads; inside a tile the
 // operands of the next steps are read from LDS while the current step computes.
@@ -46,7 +49,7 @@ struct FwdOps {
     float k[Geo<D>::NP], q[Geo<D>::NP], v, b, kq;
 };
 
-template <int D, int RING, int PF, int WPB>
+template <int D, int RING, int PF, int WPB, bool SUM = false>
 __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_view k, fwp_view v,
                                                          fwp_view beta, float *__restrict__ W,
                                                          float *__restrict__ out,
@@ -76,7 +79,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     auto &skq = skq_[wave];
     auto &sout = sout_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
-                *bb = row(beta, n, h, 0);
+                *bb = SUM ? nullptr : row(beta, n, h, 0);
 
     float Wc[R];  // W[reg_index(jj)][col]
 #pragma unroll
@@ -97,13 +100,13 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
             pk.template fetch<false>(klane, k.sL, t0, L, lane);
             pv.template fetch<false>(vlane, v.sL, t0, L, lane);
         }
-        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];   // every 16-lane row loads the tile's betas
+        if constexpr (!SUM) pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];   // every 16-lane row loads the tile's betas
     };
     auto commit = [&](int buf) {
         pq.commit(sq[buf], lane);
         pk.commit(sk[buf], lane);
         pv.commit(sv[buf], lane);
-        sb[buf][per] = pb;
+        if constexpr (!SUM) sb[buf][per] = pb;
         float kq[NV4];
         tile_row_dots<D>(pk, pq, kq);
 #pragma unroll
@@ -113,7 +116,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     // Results are staged in LDS (lanes with odd s write vdiff, the others out; lanes that share
     // an address write the same value) and leave for HBM one tile later, so that the only
     // memory operations in flight when a tile is committed are at least a tile old.
-    const bool store_d = sl & 1;
+    const bool store_d = !SUM && (sl & 1);
     float *stage = sout[store_d ? 1 : 0] + col;
     float *out_rows = out + seq * L * D;
     float *vd_rows = vdiff ? vdiff + seq * L * D : nullptr;
@@ -129,12 +132,18 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
             o.q[p] = sq[buf][tt * D + 16 * p + per];
         }
         o.v = sv[buf][tt * D + col];
-        o.b = sb[buf][tt];
+        o.b = SUM ? 1.f : sb[buf][tt];
         o.kq = skq[buf][tt];
     };
     // out_t = W_t^T q = W_{t-1}^T q + u (k.q): both mat-vecs read the old state, so their
     // dependent DPP sums overlap instead of running one after the other
     auto compute = [&](const FwdOps<D> &o, float *o_ptr) {
+        if constexpr (SUM) {
+            const float p_out = group_sum<S>(dot_rot<D>(Wc, o.q));
+            rank1_rot<D>(Wc, o.k, o.v);
+            *o_ptr = pinned(fmaf(o.v, o.kq, p_out));
+            return;
+        }
         const float p_old = group_sum<S>(dot_rot<D>(Wc, o.k));
         const float p_out = group_sum<S>(dot_rot<D>(Wc, o.q));
         const float d = o.v - p_old;
@@ -194,10 +203,13 @@ struct BwdOps {
     float q_i, k_i, go_i, d_i, b;
 };
 
-template <int D, int RING, int PF, int WPB>
+// dv: vdiff of the delta rule (contiguous rows), v itself for the sum rule.  W_init (sum rule only,
+// may be null) is subtracted from the re-anchored state, which takes the carried-in state out of gq.
+template <int D, int RING, int PF, int WPB, bool SUM = false>
 __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_view k, fwp_view beta,
-                                                         const float *__restrict__ vdiff,
+                                                         fwp_view dv,
                                                          fwp_view go, const float *__restrict__ ckpt,
+                                                         const float *__restrict__ W_init,
                                                          float *__restrict__ gq,
                                                          float *__restrict__ gk,
                                                          float *__restrict__ gv,
@@ -230,8 +242,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     auto &spd = spd_[wave];
     auto &sgrad = sgrad_[wave];
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
-                *bb = row(beta, n, h, 0);
-    const float *db = vdiff + seq * L * D;
+                *bb = SUM ? nullptr : row(beta, n, h, 0);
+    const float *db = row(dv, n, h, 0);
 
     // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
     float Wr[R], Gr[R], Gc[R], Wnext[R];
@@ -242,39 +254,50 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
     float pb = 0.f;
     const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
     const float *qlane = qb + lrow * q.sL + 4 * lc4, *klane = kb + lrow * k.sL + 4 * lc4,
-                *golane = gob + lrow * go.sL + 4 * lc4, *dlane = db + lrow * D + 4 * lc4;
+                *golane = gob + lrow * go.sL + 4 * lc4, *dlane = db + lrow * dv.sL + 4 * lc4;
     auto fetch = [&](int t0) {
         if (t0 + kTile <= L) {
             pq.template fetch<true>(qlane, q.sL, t0, L, lane);
             pk.template fetch<true>(klane, k.sL, t0, L, lane);
             pgo.template fetch<true>(golane, go.sL, t0, L, lane);
-            pd.template fetch<true>(dlane, D, t0, L, lane);
+            pd.template fetch<true>(dlane, dv.sL, t0, L, lane);
         } else {
             pq.template fetch<false>(qlane, q.sL, t0, L, lane);
             pk.template fetch<false>(klane, k.sL, t0, L, lane);
             pgo.template fetch<false>(golane, go.sL, t0, L, lane);
-            pd.template fetch<false>(dlane, D, t0, L, lane);
+            pd.template fetch<false>(dlane, dv.sL, t0, L, lane);
         }
-        float bs[NV4];
+        if constexpr (!SUM) {
+            float bs[NV4];
 #pragma unroll
-        for (int x = 0; x < NV4; x++)
-            bs[x] = bb[(int64_t)min(t0 + lrow + TileRegs<D>::kRowsPerLoad * x, L - 1) * beta.sL];
-        pu = pd;
-        pu.scale_rows(bs);
-        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+            for (int x = 0; x < NV4; x++)
+                bs[x] = bb[(int64_t)min(t0 + lrow + TileRegs<D>::kRowsPerLoad * x, L - 1) * beta.sL];
+            pu = pd;
+            pu.scale_rows(bs);
+            pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+        }
     };
     auto commit = [&](int buf) {
         pq.commit(sq[buf], lane);
         pk.commit(sk[buf], lane);
         pgo.commit(sgo[buf], lane);
         pd.commit(sd[buf], lane);
-        pu.commit(su[buf], lane);
-        sb[buf][per] = pb;
+        if constexpr (!SUM) {
+            pu.commit(su[buf], lane);
+            sb[buf][per] = pb;
+        }
     };
     auto fetch_state = [&](int c) {
         const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
 #pragma unroll
         for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
+        if constexpr (SUM) {
+            if (W_init) {
+                const float *w0 = W_init + (seq * D + i) * D;
+#pragma unroll
+                for (int jj = 0; jj < R; jj++) Wnext[jj] -= w0[reg_index<D>(lane, jj)];
+            }
+        }
     };
 
     // Gradients are staged in LDS and leave for HBM one tile later (see the forward kernel).
@@ -291,18 +314,37 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
             o.q[p] = sq[buf][off + 16 * p + per];
             o.k[p] = sk[buf][off + 16 * p + per];
             o.go[p] = sgo[buf][off + 16 * p + per];
-            o.u[p] = su[buf][off + 16 * p + per];
+            o.u[p] = (SUM ? sd : su)[buf][off + 16 * p + per];
         }
         o.q_i = sq[buf][off + i];
         o.k_i = sk[buf][off + i];
         o.go_i = sgo[buf][off + i];
-        o.d_i = sd[buf][off + i];
-        o.b = sb[buf][tt];
+        if constexpr (!SUM) {
+            o.d_i = sd[buf][off + i];
+            o.b = sb[buf][tt];
+        }
+    };
+    auto stage_grads = [&](float gq_i, float gk_i, float gv_i, int tt) {
+        const float o_q = pinned(gq_i), o_k = pinned(gk_i), o_v = pinned(gv_i);
+        if constexpr (S == 4) {
+            dst1[tt * D] = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
+        } else {
+            dst1[tt * D] = sl == 0 ? o_q : o_k;
+            dst2[tt * D] = o_v;
+        }
     };
     auto compute = [&](const BwdOps<D> &o, int tt) {
         // G' = G + q (x) go (both layouts);  r = G'^T k
         rank1_rot<D>(Gc, o.q, o.go_i);
         const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        if constexpr (SUM) {   // gv = r, gk = G' v, and the write has no adjoint into the state
+            rank1_rot<D>(Gr, o.go, o.q_i);
+            const float gq_i = group_sum<S>(dot_rot<D>(Wr, o.go));
+            rank1_rot<D, true>(Wr, o.u, o.k_i);
+            const float gk_i = group_sum<S>(dot_rot<D>(Gr, o.u));
+            stage_grads(gq_i, gk_i, r_i, tt);
+            return;
+        }
         const float gv_i = o.b * r_i;
         const float a_i = -gv_i;                              // gradient w.r.t. v_old
         float a[NP];
@@ -315,13 +357,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         float gk_i = dot_rot<D>(Gr, o.u);                         // G' u + W_{t-1} a
         gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
         rank1_rot<D>(Gr, a, o.k_i);
-        const float o_q = pinned(gq_i), o_k = pinned(gk_i), o_v = pinned(gv_i);
-        if constexpr (S == 4) {
-            dst1[tt * D] = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
-        } else {
-            dst1[tt * D] = sl == 0 ? o_q : o_k;
-            dst2[tt * D] = o_v;
-        }
+        stage_grads(gq_i, gk_i, gv_i, tt);
     };
     // a finished tile of gradients goes to HBM; gbeta of its steps is the sum of spd[tt][:]
     // over the D entries, four lanes per step
@@ -329,6 +365,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_bwd_reg(fwp_view q, fwp_v
         flush_tile<D>(sgrad[0], gq_rows, t0, L, lane);
         flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
         flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
+        if constexpr (SUM) return;
         const int tt = lane / 4, part = lane % 4;
         float acc = 0.f;
 #pragma unroll
@@ -410,12 +447,42 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
                   int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     const int nseq = N * H;
+    const fwp_view dv = {vdiff, (int64_t)H * L * D, (int64_t)L * D, (int64_t)D};
     if (D == 16)
         hipLaunchKernelGGL((k_delta_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                           q, k, beta, vdiff, go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
+                           q, k, beta, dv, go, ckpt, nullptr, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
     else
         hipLaunchKernelGGL((k_delta_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
-                           q, k, beta, vdiff, go, ckpt, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
+                           q, k, beta, dv, go, ckpt, nullptr, gq, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+int reg_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+                int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    const int nseq = N * H;
+    const fwp_view none = {nullptr, 0, 0, 0};
+    if (D == 16)
+        hipLaunchKernelGGL((k_delta_fwd_reg<16, 4, 2, 4, true>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, v, none, W, out, nullptr, ckpt, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_delta_fwd_reg<32, 2, 1, 4, true>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, v, none, W, out, nullptr, ckpt, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+int reg_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+                const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int D,
+                int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    const int nseq = N * H;
+    const fwp_view none = {nullptr, 0, 0, 0};
+    if (D == 16)
+        hipLaunchKernelGGL((k_delta_bwd_reg<16, 2, 1, 4, true>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                           q, k, none, v, go, ckpt, W_init, gq, gk, gv, nullptr, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_delta_bwd_reg<32, 2, 1, 2, true>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
+                           q, k, none, v, go, ckpt, W_init, gq, gk, gv, nullptr, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
 

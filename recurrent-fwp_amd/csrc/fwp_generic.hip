@@ -174,6 +174,76 @@ __global__ __launch_bounds__(NT) void k_delta_bwd(fwp_view q, fwp_view k, fwp_vi
     }
 }
 
+// ------------------------------------------------------------------ sum rule
+
+__global__ __launch_bounds__(NT) void k_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W,
+                                                float *out, float *ckpt, int H, int L, int E, int M,
+                                                int chunk, int nchunk) {
+    extern __shared__ float lds[];
+    const int lda = pitch(M);
+    float *sW = lds, *sk = sW + E * lda, *sq = sk + E, *sv = sq + E;
+    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    const int64_t seq = blockIdx.x;
+    load_state(sW, lda, W + seq * E * M, E, M);
+    for (int t = 0; t < L; t++) {
+        __syncthreads();
+        load_vec(sk, row(k, n, h, t), E);
+        load_vec(sq, row(q, n, h, t), E);
+        load_vec(sv, row(v, n, h, t), M);
+        __syncthreads();
+        rank1(sW, lda, sk, sv, E, M, 1.f);
+        __syncthreads();
+        for (int m = threadIdx.x; m < M; m += NT)
+            out[(seq * L + t) * M + m] = col_dot(sW, lda, sq, E, m);
+        if (ckpt && ((t + 1) % chunk == 0 || t == L - 1))
+            store_state(ckpt + (seq * nchunk + t / chunk) * E * M, sW, lda, E, M);
+    }
+    __syncthreads();
+    store_state(W + seq * E * M, sW, lda, E, M);
+}
+
+// One reverse sweep: G_t = sum_{s>=t} q_s (x) go_s gives gk = G v and gv = G^T k; the forward
+// sums S_t that gq = S_t go needs are re-anchored from the checkpoints and rewound step by step.
+// With W_init the carried-in state is taken out of S (then gq holds only what the sequence wrote).
+__global__ __launch_bounds__(NT) void k_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go,
+                                                const float *ckpt, const float *W_init, float *gq,
+                                                float *gk, float *gv, int H, int L, int E, int M,
+                                                int chunk, int nchunk) {
+    extern __shared__ float lds[];
+    const int lda = pitch(M);
+    float *sW = lds, *sG = sW + E * lda, *sk = sG + E * lda, *sq = sk + E, *sgo = sq + E,
+          *sv = sgo + M;
+    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    const int64_t seq = blockIdx.x;
+    for (int i = threadIdx.x; i < E * lda; i += NT) sG[i] = 0.f;
+    for (int j = nchunk - 1; j >= 0; j--) {
+        __syncthreads();
+        load_state(sW, lda, ckpt + (seq * nchunk + j) * E * M, E, M);
+        if (W_init) {
+            const float *w0 = W_init + seq * E * M;
+            for (int i = threadIdx.x; i < E * M; i += NT) sW[(i / M) * lda + i % M] -= w0[i];
+        }
+        const int t_hi = min((j + 1) * chunk, L) - 1;
+        for (int t = t_hi; t >= j * chunk; t--) {
+            __syncthreads();
+            load_vec(sk, row(k, n, h, t), E);
+            load_vec(sq, row(q, n, h, t), E);
+            load_vec(sgo, row(go, n, h, t), M);
+            load_vec(sv, row(v, n, h, t), M);
+            __syncthreads();
+            rank1(sG, lda, sq, sgo, E, M, 1.f);
+            for (int e = threadIdx.x; e < E; e += NT)
+                gq[(seq * L + t) * E + e] = row_dot(sW, lda, sgo, M, e);
+            __syncthreads();
+            for (int m = threadIdx.x; m < M; m += NT)
+                gv[(seq * L + t) * M + m] = col_dot(sG, lda, sk, E, m);
+            for (int e = threadIdx.x; e < E; e += NT)
+                gk[(seq * L + t) * E + e] = row_dot(sG, lda, sv, M, e);
+            rank1(sW, lda, sk, sv, E, M, -1.f);
+        }
+    }
+}
+
 // -------------------------------------------------------------- Delta RNN v2
 
 __global__ __launch_bounds__(NT) void k_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta,
@@ -459,6 +529,27 @@ int generic_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff,
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_delta_bwd, dim3(N * H), dim3(NT), bytes, s, q, k, beta, vdiff, go, ckpt,
                        gq, gk, gv, gbeta, H, L, E, M, chunk, nchunk);
+    return launched();
+}
+
+int generic_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N,
+                    int H, int L, int E, int M, int chunk, hipStream_t s) {
+    size_t bytes = sizeof(float) * ((size_t)E * pitch(M) + 2 * E + M);
+    if (int rc = prepare(k_sum_fwd, bytes)) return rc;
+    int nchunk = (L + chunk - 1) / chunk;
+    hipLaunchKernelGGL(k_sum_fwd, dim3(N * H), dim3(NT), bytes, s, q, k, v, W, out, ckpt, H, L, E,
+                       M, chunk, nchunk);
+    return launched();
+}
+
+int generic_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+                    const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L,
+                    int E, int M, int chunk, hipStream_t s) {
+    size_t bytes = sizeof(float) * ((size_t)2 * E * pitch(M) + 2 * E + 2 * M);
+    if (int rc = prepare(k_sum_bwd, bytes)) return rc;
+    int nchunk = (L + chunk - 1) / chunk;
+    hipLaunchKernelGGL(k_sum_bwd, dim3(N * H), dim3(NT), bytes, s, q, k, v, go, ckpt, W_init, gq,
+                       gk, gv, H, L, E, M, chunk, nchunk);
     return launched();
 }
 
