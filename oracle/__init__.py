@@ -164,6 +164,39 @@ def rnn_bwd(z, k, v, W0, beta, h0, go):
     return gz, gk, gv, gb
 
 
+# ------------------------------------------------------------- Delta LSTM v4
+
+def _stack3(gates, dt):
+    return np.ascontiguousarray(np.stack([np.asarray(g, dt) for g in gates]))
+
+
+def lstm_fwd(Zs, Ks, Vs, Bs, Ws, h0, c0):
+    """Delta LSTM v4.  ``Zs, Ks, Vs, Bs, Ws`` are triples in gate order (i, u, o):
+    z, k, v ``[N,H,L,D]``, beta ``[N,H,L,1]``, W ``[N,H,D,D]``; h0, c0 ``[N,H,1,D]``.
+    Returns (out, cell_out, [W_i, W_u, W_o] after L steps, h_L, c_L)."""
+    dt = np.asarray(Zs[0]).dtype
+    Z, K, V, B, W = (_stack3(x, dt) for x in (Zs, Ks, Vs, Bs, Ws))
+    _, N, H, L, D = Z.shape
+    assert K.shape == V.shape == Z.shape and B.shape == (3, N, H, L, 1) and W.shape == (3, N, H, D, D)
+    assert np.shape(h0) == np.shape(c0) == (N, H, 1, D)
+    h, c = _c(h0, dt).copy(), _c(c0, dt).copy()
+    out, cell = np.empty((N, H, L, D), dt), np.empty((N, H, L, D), dt)
+    _call("fwp_oracle_lstm_fwd", dt, [Z, K, V, B, W, h, c, out, cell], [N, H, L, D])
+    return out, cell, [W[0], W[1], W[2]], h, c
+
+
+def lstm_bwd(Zs, Ks, Vs, Bs, Ws, h0, c0, go):
+    """Gradients for an upstream gradient on ``out`` only (the reference ignores the one on
+    the cell output): (gZ, gK, gV, gB), each a list in gate order (i, u, o)."""
+    dt = np.asarray(Zs[0]).dtype
+    Z, K, V, B, W = (_stack3(x, dt) for x in (Zs, Ks, Vs, Bs, Ws))
+    _, N, H, L, D = Z.shape
+    h0, c0, go = _c(h0, dt), _c(c0, dt), _c(go, dt)
+    gZ, gK, gV, gB = np.empty_like(Z), np.empty_like(K), np.empty_like(V), np.empty_like(B)
+    _call("fwp_oracle_lstm_bwd", dt, [Z, K, V, B, W, h0, c0, go, gZ, gK, gV, gB], [N, H, L, D])
+    return tuple([g[0], g[1], g[2]] for g in (gZ, gK, gV, gB))
+
+
 # ------------------------------------------------------- Recurrent Delta Net
 
 def rec_fwd(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0):

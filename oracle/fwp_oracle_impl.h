@@ -10,6 +10,7 @@
  *   Delta RNN v2        algorithmic/fast_weight_rnn_v2/__init__.py:205-217
  *   Recurrent Delta Net algorithmic/rec_update_fwm_tanh/__init__.py:263-302
  *   sum rule            algorithmic/fast_transformers/__init__.py:145-152
+ *   Delta LSTM v4       language_modeling/src/utils/fast_lstm_v4/__init__.py:397-432
  *
  * The backward functions are the plain reverse-mode adjoint of those loops with
  * every intermediate state W_t kept in memory (what autograd does for the
@@ -267,6 +268,141 @@ void FN(fwp_oracle_rnn_bwd)(const REAL *z, const REAL *k, const REAL *v,
                                 gk + r * D, gv + r * D, gbeta + r, tmp, D, D);
         }
         free(Wall); free(dall); free(sall); free(h); free(gh); free(gs); free(gW); free(tmp);
+    }
+}
+
+/* ------------------------------------------------------------ Delta LSTM v4 */
+
+/* Three delta-rule memories (gate order i, u, o) read with s = softmax(h_{t-1}):
+ *   W_g += k_g (x) beta_g (v_g - W_g^T k_g)          g in {i, u, o}
+ *   i = sigmoid(W_i^T s + z_i), u = W_u^T s + z_u, o = sigmoid(W_o^T s + z_o)
+ *   c_t = i u + (1 - i) c_{t-1},  h_t = o c_t
+ * (loop of the reference's self test, fast_lstm_v4/__init__.py:397-432; the kernel adds
+ * 1e-6 to the softmax denominator, fast_lstm_v4_cuda.cu:113,256, the loop does not).
+ * Z,K,V [3,N,H,L,D], B [3,N,H,L], W [3,N,H,D,D] in/out, h,c [N,H,D] in/out. */
+void FN(fwp_oracle_lstm_fwd)(const REAL *Z, const REAL *K, const REAL *V, const REAL *B,
+                             REAL *W, REAL *h0, REAL *c0, REAL *out, REAL *cell, int N,
+                             int H, int L, int D) {
+    const size_t gs_vec = (size_t)N * H * L * D, gs_b = (size_t)N * H * L,
+                 gs_W = (size_t)N * H * D * D;
+#pragma omp parallel for schedule(static)
+    for (int s = 0; s < N * H; s++) {
+        REAL *h = h0 + (size_t)s * D, *c = c0 + (size_t)s * D;
+        REAL *buf = (REAL *)malloc(sizeof(REAL) * 5 * D);
+        REAL *d = buf, *sm = buf + D, *a = buf + 2 * D; /* a: 3 pre-activations */
+        for (int t = 0; t < L; t++) {
+            size_t r = (size_t)s * L + t;
+            FN(softmax_vec)(h, sm, D);
+            for (int g = 0; g < 3; g++) {
+                REAL *Wg = W + g * gs_W + (size_t)s * D * D;
+                FN(delta_write)(Wg, K + g * gs_vec + r * D, V + g * gs_vec + r * D,
+                                B[g * gs_b + r], d, D, D);
+                FN(matTvec)(Wg, sm, a + g * D, D, D);
+                for (int m = 0; m < D; m++) a[g * D + m] += Z[g * gs_vec + r * D + m];
+            }
+            for (int m = 0; m < D; m++) {
+                REAL gi = (REAL)1 / ((REAL)1 + EXP(-a[m]));
+                REAL go_ = (REAL)1 / ((REAL)1 + EXP(-a[2 * D + m]));
+                c[m] = gi * a[D + m] + ((REAL)1 - gi) * c[m];
+                h[m] = go_ * c[m];
+                out[r * D + m] = h[m];
+                cell[r * D + m] = c[m];
+            }
+        }
+        free(buf);
+    }
+}
+
+/* Reverse-mode adjoint of the loop above for an upstream gradient on `out` only
+ * (the reference's backward ignores the gradient of the cell output,
+ * fast_lstm_v4/__init__.py:128).  All states kept in memory. */
+void FN(fwp_oracle_lstm_bwd)(const REAL *Z, const REAL *K, const REAL *V, const REAL *B,
+                             const REAL *W0, const REAL *h0, const REAL *c0, const REAL *go,
+                             REAL *gZ, REAL *gK, REAL *gV, REAL *gB, int N, int H, int L,
+                             int D) {
+    const size_t gs_vec = (size_t)N * H * L * D, gs_b = (size_t)N * H * L,
+                 gs_W = (size_t)N * H * D * D;
+#pragma omp parallel for schedule(static)
+    for (int s = 0; s < N * H; s++) {
+        size_t DD = (size_t)D * D;
+        REAL *Wall = (REAL *)malloc(sizeof(REAL) * 3 * DD * (L + 1)); /* [g][t][D][D] */
+        REAL *dall = (REAL *)malloc(sizeof(REAL) * 3 * (size_t)D * L);
+        REAL *sall = (REAL *)malloc(sizeof(REAL) * (size_t)D * L);
+        REAL *act = (REAL *)malloc(sizeof(REAL) * 3 * (size_t)D * L); /* i, u, o */
+        REAL *call = (REAL *)malloc(sizeof(REAL) * (size_t)D * (L + 1));
+        REAL *h = (REAL *)malloc(sizeof(REAL) * D);
+        REAL *gh = (REAL *)calloc(D, sizeof(REAL));
+        REAL *gc = (REAL *)calloc(D, sizeof(REAL));
+        REAL *gs = (REAL *)malloc(sizeof(REAL) * D);
+        REAL *ga = (REAL *)malloc(sizeof(REAL) * 3 * D);
+        REAL *gW = (REAL *)calloc(3 * DD, sizeof(REAL));
+        REAL *tmp = (REAL *)malloc(sizeof(REAL) * 2 * D);
+        for (int g = 0; g < 3; g++)
+            memcpy(Wall + g * DD * (L + 1), W0 + g * gs_W + (size_t)s * DD, sizeof(REAL) * DD);
+        memcpy(h, h0 + (size_t)s * D, sizeof(REAL) * D);
+        memcpy(call, c0 + (size_t)s * D, sizeof(REAL) * D);
+        for (int t = 0; t < L; t++) {
+            size_t r = (size_t)s * L + t;
+            REAL *st = sall + (size_t)t * D;
+            FN(softmax_vec)(h, st, D);
+            for (int g = 0; g < 3; g++) {
+                REAL *Wg = Wall + g * DD * (L + 1);
+                memcpy(Wg + (t + 1) * DD, Wg + t * DD, sizeof(REAL) * DD);
+                FN(delta_write)(Wg + (t + 1) * DD, K + g * gs_vec + r * D, V + g * gs_vec + r * D,
+                                B[g * gs_b + r], dall + ((size_t)g * L + t) * D, D, D);
+                REAL *a = act + ((size_t)g * L + t) * D;
+                FN(matTvec)(Wg + (t + 1) * DD, st, a, D, D);
+                for (int m = 0; m < D; m++) {
+                    a[m] += Z[g * gs_vec + r * D + m];
+                    if (g != 1) a[m] = (REAL)1 / ((REAL)1 + EXP(-a[m]));
+                }
+            }
+            const REAL *gi = act + (size_t)t * D, *u = act + ((size_t)L + t) * D,
+                       *o = act + ((size_t)2 * L + t) * D;
+            for (int m = 0; m < D; m++) {
+                REAL cn = gi[m] * u[m] + ((REAL)1 - gi[m]) * call[(size_t)t * D + m];
+                call[(size_t)(t + 1) * D + m] = cn;
+                h[m] = o[m] * cn;
+            }
+        }
+        for (int t = L - 1; t >= 0; t--) {
+            size_t r = (size_t)s * L + t;
+            const REAL *st = sall + (size_t)t * D;
+            const REAL *gi = act + (size_t)t * D, *u = act + ((size_t)L + t) * D,
+                       *o = act + ((size_t)2 * L + t) * D;
+            const REAL *cp = call + (size_t)t * D, *cn = call + (size_t)(t + 1) * D;
+            for (int m = 0; m < D; m++) {
+                REAL ghm = gh[m] + go[r * D + m];
+                REAL gct = gc[m] + ghm * o[m];                 /* h = o c */
+                ga[2 * D + m] = ghm * cn[m] * o[m] * ((REAL)1 - o[m]);
+                ga[m] = gct * (u[m] - cp[m]) * gi[m] * ((REAL)1 - gi[m]);
+                ga[D + m] = gct * gi[m];
+                gc[m] = gct * ((REAL)1 - gi[m]);
+            }
+            for (int e = 0; e < D; e++) gs[e] = 0;
+            for (int g = 0; g < 3; g++) {
+                const REAL *Wg = Wall + g * DD * (L + 1);
+                REAL *gWg = gW + g * DD;
+                for (int m = 0; m < D; m++) gZ[g * gs_vec + r * D + m] = ga[g * D + m];
+                for (int e = 0; e < D; e++)
+                    for (int m = 0; m < D; m++) gWg[e * D + m] += st[e] * ga[g * D + m];
+                FN(matvec)(Wg + (t + 1) * DD, ga + g * D, tmp, D, D);
+                for (int e = 0; e < D; e++) gs[e] += tmp[e];
+            }
+            REAL dot = 0;
+            for (int e = 0; e < D; e++) dot += gs[e] * st[e];
+            for (int e = 0; e < D; e++) gh[e] = st[e] * (gs[e] - dot);
+            for (int g = 0; g < 3; g++) {
+                const REAL *Wg = Wall + g * DD * (L + 1);
+                REAL *gk = gK + g * gs_vec + r * D;
+                for (int e = 0; e < D; e++) gk[e] = 0;
+                FN(delta_write_adj)(gW + g * DD, Wg + t * DD, K + g * gs_vec + r * D,
+                                    dall + ((size_t)g * L + t) * D, B[g * gs_b + r], gk,
+                                    gV + g * gs_vec + r * D, gB + g * gs_b + r, tmp, D, D);
+            }
+        }
+        free(Wall); free(dall); free(sall); free(act); free(call); free(h); free(gh); free(gc);
+        free(gs); free(ga); free(gW); free(tmp);
     }
 }
 

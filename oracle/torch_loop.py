@@ -8,6 +8,8 @@ time on the host is the reference's CPU path.
   delta rule           algorithmic/fast_weight/__init__.py:178-187
   Delta RNN v2         algorithmic/fast_weight_rnn_v2/__init__.py:205-217
   Recurrent Delta Net  algorithmic/rec_update_fwm_tanh/__init__.py:263-302
+  sum rule             algorithmic/fast_transformers/__init__.py:145-152
+  Delta LSTM v4        language_modeling/src/utils/fast_lstm_v4/__init__.py:397-432
 
 The state is kept as ``W[N,H,E,M]`` (the operators' layout) instead of the
 reference loop's transposed ``[N*H,M,E]``; the arithmetic per step is the same.
@@ -58,6 +60,25 @@ def rnn_v2_loop(z, k, v, W0, beta, h0):
         h = _read(W, s) + z[:, :, t]
         outs.append(h)
     return torch.stack(outs, dim=2), W, h.unsqueeze(2)
+
+
+def lstm_v4_loop(zi, ki, vi, bi, Wi, zu, ku, vu, bu, Wu, zo, ko, vo, bo, Wo, h0, c0):
+    """Argument order of the reference op. -> (out, cell_out, (W_i, W_u, W_o), h_L, c_L)."""
+    h, c = h0[:, :, 0], c0[:, :, 0]
+    outs, cells = [], []
+    for t in range(zi.shape[2]):
+        Wi = _write(Wi, ki[:, :, t], vi[:, :, t], bi[:, :, t])
+        Wu = _write(Wu, ku[:, :, t], vu[:, :, t], bu[:, :, t])
+        Wo = _write(Wo, ko[:, :, t], vo[:, :, t], bo[:, :, t])
+        s = torch.softmax(h, dim=-1)
+        gate_i = torch.sigmoid(_read(Wi, s) + zi[:, :, t])
+        upd = _read(Wu, s) + zu[:, :, t]
+        gate_o = torch.sigmoid(_read(Wo, s) + zo[:, :, t])
+        c = gate_i * upd + (1.0 - gate_i) * c
+        h = c * gate_o
+        outs.append(h)
+        cells.append(c)
+    return torch.stack(outs, dim=2), torch.stack(cells, dim=2), (Wi, Wu, Wo), h.unsqueeze(2), c.unsqueeze(2)
 
 
 def rec_update_loop(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0):

@@ -52,6 +52,20 @@ def rec_inputs(seed, N, H, L, D, dtype=np.float64, w0=False, rscale=None):
     return qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0, go
 
 
+def lstm_inputs(seed, N, H, L, D, dtype=np.float64, w0=False):
+    """Delta LSTM v4: (Zs, Ks, Vs, Bs, Ws, h0, c0, go), the first five as (i, u, o) triples."""
+    g = rng(seed)
+    Zs = [g.standard_normal((N, H, L, D)).astype(dtype) for _ in range(3)]
+    Ks = [softmax(g.standard_normal((N, H, L, D))).astype(dtype) for _ in range(3)]
+    Vs = [g.standard_normal((N, H, L, D)).astype(dtype) for _ in range(3)]
+    Bs = [sigmoid(g.standard_normal((N, H, L, 1))).astype(dtype) for _ in range(3)]
+    Ws = [(g.standard_normal((N, H, D, D)) * (0.5 if w0 else 0.0)).astype(dtype) for _ in range(3)]
+    h0 = (g.standard_normal((N, H, 1, D)) * (1.0 if w0 else 0.0)).astype(dtype)
+    c0 = (g.standard_normal((N, H, 1, D)) * (1.0 if w0 else 0.0)).astype(dtype)
+    go = g.standard_normal((N, H, L, D)).astype(dtype)
+    return Zs, Ks, Vs, Bs, Ws, h0, c0, go
+
+
 def max_abs(a, b):
     return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)))) if np.size(a) else 0.0
 
