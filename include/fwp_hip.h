@@ -132,6 +132,38 @@ int fwp_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                 int L, int D, int chunk, void *stream);
 
 /*
+ * Delta LSTM v4 forward.  Replaces fast_lstm_v4_forward
+ * (language_modeling/src/utils/fast_lstm_v4/fast_lstm_v4_cuda.cu:377-497, kernel :30-373).
+ * Three delta-rule memories, gate order i (input gate), u (update), o (output gate), all
+ * read with s = softmax(h_{t-1}):
+ *   W_g += k_g (x) beta_g (v_g - W_g^T k_g)
+ *   i = sigmoid(W_i^T s + z_i)   u = W_u^T s + z_u   o = sigmoid(W_o^T s + z_o)
+ *   c_t = i u + (1 - i) c_{t-1}   h_t = o c_t
+ * z, k, v, beta: host arrays of 3 views ([N,H,L,D]; beta [N,H,L,1]); W: host array of 3
+ * device pointers to [N,H,D,D] states (in/out); h, c [N,H,D] in/out (the reference's
+ * `states`, `cells`); out, cell [N,H,L,D].
+ * Saved for backward, all three or none: gates [3,N,H,L,D] (i, u, o),
+ * vdiff [3,N,H,L,D], ckpt [3,N,H,nchunk,D,D].
+ */
+int fwp_lstm_fwd(const fwp_view *z, const fwp_view *k, const fwp_view *v,
+                 const fwp_view *beta, float *const *W, float *h, float *c,
+                 float *out, float *cell, float *gates, float *vdiff, float *ckpt,
+                 int N, int H, int L, int D, int chunk, void *stream);
+
+/*
+ * Delta LSTM v4 backward.  Replaces fast_lstm_v4_backward
+ * (fast_lstm_v4_cuda.cu:1072-1220, kernel :499-1068).  The upstream gradient is that of
+ * `out`; as in the reference the cell output carries none (fast_lstm_v4/__init__.py:128).
+ * h_init, c_init [N,H,D]: the states before the first step.
+ * gz, gk, gv [3,N,H,L,D], gbeta [3,N,H,L], gate order i, u, o.
+ */
+int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff,
+                 const float *gates, const float *out, const float *cell,
+                 const float *h_init, const float *c_init, fwp_view grad_out,
+                 const float *ckpt, float *gz, float *gk, float *gv, float *gbeta,
+                 int N, int H, int L, int D, int chunk, void *stream);
+
+/*
  * Recurrent Delta Net forward.  Replaces rec_update_fwm_tanh_forward
  * (algorithmic/rec_update_fwm_tanh/rec_update_fwm_tanh.cu:349-444, kernel :25-345).
  *   qx,kx,vx [N,H,L,D] and bx [N,H,L,1] are pre-activation

@@ -8,11 +8,13 @@ of ``libfwp_hip.so``; there is no other implementation behind these names.
 from . import _lib
 from .fast_weight import DeltaFastWeight, fast_weight_delta
 from .fast_transformers import FastWeightSum, fast_weight_sum
+from .fast_lstm_v4 import FastLSTMv4, fast_lstm_v4
 from .fast_weight_rnn_v2 import FastRNNv2, fast_rnn_v2
 from .rec_update_fwm_tanh import FastWeightRecUpdateTanh, rec_update_fwm_tanh
 from .layers import DeltaNetDecoderLayer, DeltaNetLayer, PositionalEmbedding, PositionwiseFF
 from .lm import DeltaNetLM
 
 __all__ = ["DeltaFastWeight", "fast_weight_delta", "FastWeightSum", "fast_weight_sum", "FastRNNv2", "fast_rnn_v2",
+           "FastLSTMv4", "fast_lstm_v4",
            "FastWeightRecUpdateTanh", "rec_update_fwm_tanh", "DeltaNetLayer",
            "DeltaNetDecoderLayer", "PositionwiseFF", "PositionalEmbedding", "DeltaNetLM"]

@@ -25,6 +25,7 @@ class FwpError(RuntimeError):
 
 
 _P, _I, _V = ctypes.c_void_p, ctypes.c_int, View
+_VP = ctypes.POINTER(View)          # host array of views (one per gate)
 _SIGNATURES = {
     "fwp_delta_fwd": [_V] * 4 + [_P] * 4 + [_I] * 6 + [_P],
     "fwp_delta_bwd": [_V] * 3 + [_P, _V, _P] + [_P] * 4 + [_I] * 6 + [_P],
@@ -32,6 +33,8 @@ _SIGNATURES = {
     "fwp_sum_bwd": [_V] * 4 + [_P] * 5 + [_I] * 6 + [_P],
     "fwp_rnn_fwd": [_V] * 4 + [_P] * 5 + [_I] * 5 + [_P],
     "fwp_rnn_bwd": [_V, _V, _P, _P, _P, _V, _P] + [_P] * 4 + [_I] * 5 + [_P],
+    "fwp_lstm_fwd": [_VP] * 4 + [_P] * 8 + [_I] * 5 + [_P],
+    "fwp_lstm_bwd": [_VP] * 2 + [_P] * 6 + [_V] + [_P] * 5 + [_I] * 5 + [_P],
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
 }

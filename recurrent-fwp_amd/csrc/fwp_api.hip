@@ -143,6 +143,40 @@ int fwp_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                            D, chunk, (hipStream_t)stream);
 }
 
+int fwp_lstm_fwd(const fwp_view *z, const fwp_view *k, const fwp_view *v, const fwp_view *beta,
+                 float *const *W, float *h, float *c, float *out, float *cell, float *gates,
+                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, void *stream) {
+    if (!z || !k || !v || !beta || !W || !h || !c || !out || !cell) return FWP_E_NULL;
+    LstmGates g;
+    for (int a = 0; a < 3; a++) {
+        if (bad_view(z[a]) || bad_view(k[a]) || bad_view(v[a]) || bad_view(beta[a]) || !W[a])
+            return FWP_E_NULL;
+        g.z[a] = z[a]; g.k[a] = k[a]; g.v[a] = v[a]; g.beta[a] = beta[a]; g.W[a] = W[a];
+    }
+    const int saved = (gates != nullptr) + (vdiff != nullptr) + (ckpt != nullptr);
+    if (saved != 0 && saved != 3) return FWP_E_NULL;
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    return generic_lstm_fwd(g, h, c, out, cell, gates, vdiff, ckpt, N, H, L, D, chunk,
+                            (hipStream_t)stream);
+}
+
+int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff, const float *gates,
+                 const float *out, const float *cell, const float *h_init, const float *c_init,
+                 fwp_view grad_out, const float *ckpt, float *gz, float *gk, float *gv,
+                 float *gbeta, int N, int H, int L, int D, int chunk, void *stream) {
+    if (!k || !beta || !vdiff || !gates || !out || !cell || !h_init || !c_init ||
+        bad_view(grad_out) || !ckpt || !gz || !gk || !gv || !gbeta)
+        return FWP_E_NULL;
+    LstmGates g = {};
+    for (int a = 0; a < 3; a++) {
+        if (bad_view(k[a]) || bad_view(beta[a])) return FWP_E_NULL;
+        g.k[a] = k[a]; g.beta[a] = beta[a];
+    }
+    if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    return generic_lstm_bwd(g, vdiff, gates, out, cell, h_init, c_init, grad_out, ckpt, gz, gk, gv,
+                            gbeta, N, H, L, D, chunk, (hipStream_t)stream);
+}
+
 int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
                 const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,
                 float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,

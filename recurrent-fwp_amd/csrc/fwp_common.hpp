@@ -17,6 +17,12 @@ __device__ __forceinline__ const float *row(const fwp_view &v, int n, int h, int
     return v.ptr + (int64_t)n * v.sN + (int64_t)h * v.sH + (int64_t)t * v.sL;
 }
 
+// Per-gate arguments of the Delta LSTM kernels, gate order i (input), u (update), o (output).
+struct LstmGates {
+    fwp_view z[3], k[3], v[3], beta[3];
+    float *W[3];
+};
+
 // Launchers of the LDS-state kernels (any E, M that fit the LDS).
 int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                       float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
@@ -35,6 +41,13 @@ int generic_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W,
 int generic_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                     const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
                     float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s);
+int generic_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, float *gates,
+                     float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
+                     hipStream_t s);
+int generic_lstm_bwd(const LstmGates &g, const float *vdiff, const float *gates, const float *out,
+                     const float *cell, const float *h_init, const float *c_init, fwp_view go,
+                     const float *ckpt, float *gz, float *gk, float *gv, float *gbeta, int N, int H,
+                     int L, int D, int chunk, hipStream_t s);
 int generic_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
                     const float *Rk, const float *Rv, const float *rb, float *W, float *h,
                     float *out, float *q_act, float *k_act, float *beta_act, float *vdiff,

@@ -335,6 +335,148 @@ __global__ __launch_bounds__(NT) void k_rnn_bwd(fwp_view k, fwp_view beta, const
     }
 }
 
+// ------------------------------------------------------------ Delta LSTM v4
+
+// Three delta-rule memories (gate order i, u, o) read with the softmax of the previous output.
+__global__ __launch_bounds__(NT) void k_lstm_fwd(LstmGates g, float *hstate, float *cstate,
+                                                 float *out, float *cell, float *gates,
+                                                 float *vdiff, float *ckpt, int N, int H, int L,
+                                                 int D, int chunk, int nchunk) {
+    extern __shared__ float lds[];
+    const int lda = pitch(D);
+    const int WS = D * lda;
+    float *sW = lds, *sk = sW + 3 * WS, *sv = sk + 3 * D, *sz = sv + 3 * D, *su = sz + 3 * D,
+          *sh = su + 3 * D, *sc = sh + D, *ss = sc + D, *tmp = ss + D;
+    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    const int64_t seq = blockIdx.x;
+    const int64_t gate_stride = (int64_t)N * H * L * D;        // between the stacked per-gate buffers
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+    for (int a = 0; a < 3; a++) load_state(sW + a * WS, lda, g.W[a] + seq * D * D, D, D);
+    load_vec(sh, hstate + seq * D, D);
+    load_vec(sc, cstate + seq * D, D);
+    for (int t = 0; t < L; t++) {
+        __syncthreads();
+        for (int a = 0; a < 3; a++) {
+            load_vec(sk + a * D, row(g.k[a], n, h, t), D);
+            load_vec(sv + a * D, row(g.v[a], n, h, t), D);
+            load_vec(sz + a * D, row(g.z[a], n, h, t), D);
+        }
+        __syncthreads();
+        softmax_lds(sh, ss, tmp, D);
+        for (int i = threadIdx.x; i < 3 * D; i += NT) {
+            const int a = i / D, m = i - a * D;
+            const float d = sv[i] - col_dot(sW + a * WS, lda, sk + a * D, D, m);
+            su[i] = *row(g.beta[a], n, h, t) * d;
+            if (vdiff) vdiff[a * gate_stride + (seq * L + t) * D + m] = d;
+        }
+        __syncthreads();
+        for (int a = 0; a < 3; a++) rank1(sW + a * WS, lda, sk + a * D, su + a * D, D, D, 1.f);
+        __syncthreads();
+        for (int m = threadIdx.x; m < D; m += NT) {
+            const float ai = col_dot(sW, lda, ss, D, m) + sz[m];
+            const float u = col_dot(sW + WS, lda, ss, D, m) + sz[D + m];
+            const float ao = col_dot(sW + 2 * WS, lda, ss, D, m) + sz[2 * D + m];
+            const float gi = 1.f / (1.f + expf(-ai)), go_ = 1.f / (1.f + expf(-ao));
+            const float c = gi * u + (1.f - gi) * sc[m];
+            const float hv = go_ * c;
+            const int64_t o = (seq * L + t) * D + m;
+            out[o] = hv;
+            cell[o] = c;
+            if (gates) {
+                gates[o] = gi;
+                gates[gate_stride + o] = u;
+                gates[2 * gate_stride + o] = go_;
+            }
+            sc[m] = c;
+            sh[m] = hv;      // softmax_lds of this step is done with sh (barriers above)
+        }
+        if (ckpt && ((t + 1) % chunk == 0 || t == L - 1))
+            for (int a = 0; a < 3; a++)
+                store_state(ckpt + a * ckpt_stride + (seq * nchunk + t / chunk) * D * D,
+                            sW + a * WS, lda, D, D);
+    }
+    __syncthreads();
+    for (int a = 0; a < 3; a++) store_state(g.W[a] + seq * D * D, sW + a * WS, lda, D, D);
+    load_vec(hstate + seq * D, sh, D);
+    load_vec(cstate + seq * D, sc, D);
+}
+
+__global__ __launch_bounds__(NT) void k_lstm_bwd(LstmGates g, const float *vdiff,
+                                                 const float *gates, const float *out,
+                                                 const float *cell, const float *h_init,
+                                                 const float *c_init, fwp_view go,
+                                                 const float *ckpt, float *gz, float *gk,
+                                                 float *gv, float *gbeta, int N, int H, int L,
+                                                 int D, int chunk, int nchunk) {
+    extern __shared__ float lds[];
+    const int lda = pitch(D);
+    const int WS = D * lda;
+    float *sW = lds, *sG = sW + 3 * WS, *sk = sG + 3 * WS, *sd = sk + 3 * D, *sga = sd + 3 * D,
+          *su = sga + 3 * D, *sa = su + D, *sp = sa + D, *sgk = sp + D, *ss = sgk + D,
+          *shp = ss + D, *sds = shp + D, *sdh = sds + D, *sdc = sdh + D, *tmp = sdc + D,
+          *sgb = tmp + D;
+    const int n = blockIdx.x / H, h = blockIdx.x % H;
+    const int64_t seq = blockIdx.x;
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t beta_stride = (int64_t)N * H * L;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+    for (int i = threadIdx.x; i < 3 * WS; i += NT) sG[i] = 0.f;
+    for (int i = threadIdx.x; i < D; i += NT) sdh[i] = sdc[i] = 0.f;
+    for (int j = nchunk - 1; j >= 0; j--) {
+        __syncthreads();
+        for (int a = 0; a < 3; a++)
+            load_state(sW + a * WS, lda, ckpt + a * ckpt_stride + (seq * nchunk + j) * D * D, D, D);
+        const int t_hi = min((j + 1) * chunk, L) - 1;
+        for (int t = t_hi; t >= j * chunk; t--) {
+            __syncthreads();
+            const int64_t r = seq * L + t;
+            for (int a = 0; a < 3; a++) {
+                load_vec(sk + a * D, row(g.k[a], n, h, t), D);
+                load_vec(sd + a * D, vdiff + a * gate_stride + r * D, D);
+            }
+            load_vec(shp, t > 0 ? out + (r - 1) * D : h_init + seq * D, D);
+            const float *gor = row(go, n, h, t);
+            const float *cprev = t > 0 ? cell + (r - 1) * D : c_init + seq * D;
+            for (int m = threadIdx.x; m < D; m += NT) {
+                const float gi = gates[r * D + m], u = gates[gate_stride + r * D + m],
+                            o = gates[2 * gate_stride + r * D + m];
+                const float gh = sdh[m] + gor[m];
+                const float gc = sdc[m] + gh * o;
+                const float ga_o = gh * cell[r * D + m] * o * (1.f - o);
+                const float ga_i = gc * (u - cprev[m]) * gi * (1.f - gi);
+                const float ga_u = gc * gi;
+                sdc[m] = gc * (1.f - gi);
+                sga[m] = ga_i;
+                sga[D + m] = ga_u;
+                sga[2 * D + m] = ga_o;
+                gz[r * D + m] = ga_i;
+                gz[gate_stride + r * D + m] = ga_u;
+                gz[2 * gate_stride + r * D + m] = ga_o;
+            }
+            __syncthreads();
+            softmax_lds(shp, ss, tmp, D);
+            for (int a = 0; a < 3; a++) rank1(sG + a * WS, lda, ss, sga + a * D, D, D, 1.f);
+            for (int e = threadIdx.x; e < D; e += NT)
+                sds[e] = row_dot(sW, lda, sga, D, e) + row_dot(sW + WS, lda, sga + D, D, e) +
+                         row_dot(sW + 2 * WS, lda, sga + 2 * D, D, e);
+            __syncthreads();
+            {
+                const float dot = dot_lds(sds, ss, D);
+                __syncthreads();
+                for (int e = threadIdx.x; e < D; e += NT) sdh[e] = ss[e] * (sds[e] - dot);
+            }
+            for (int a = 0; a < 3; a++) {
+                const float b = *row(g.beta[a], n, h, t);
+                delta_write_adjoint(sW + a * WS, sG + a * WS, lda, sk + a * D, sd + a * D, b, su, sa,
+                                    sp, sgk, gv + a * gate_stride + r * D, sgb, D, D);
+                for (int e = threadIdx.x; e < D; e += NT) gk[a * gate_stride + r * D + e] = sgk[e];
+                if (threadIdx.x == 0) gbeta[a * beta_stride + r] = *sgb;
+                __syncthreads();
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------ Recurrent Delta Net
 
 __global__ __launch_bounds__(NT) void k_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx,
@@ -573,6 +715,29 @@ int generic_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_rnn_bwd, dim3(N * H), dim3(NT), bytes, s, k, beta, vdiff, out, h_init, go,
                        ckpt, gz, gk, gv, gbeta, H, L, D, chunk, nchunk);
+    return launched();
+}
+
+int generic_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, float *gates,
+                     float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
+                     hipStream_t s) {
+    size_t bytes = sizeof(float) * ((size_t)3 * D * pitch(D) + 16 * D);
+    if (int rc = prepare(k_lstm_fwd, bytes)) return rc;
+    int nchunk = (L + chunk - 1) / chunk;
+    hipLaunchKernelGGL(k_lstm_fwd, dim3(N * H), dim3(NT), bytes, s, g, h, c, out, cell, gates, vdiff,
+                       ckpt, N, H, L, D, chunk, nchunk);
+    return launched();
+}
+
+int generic_lstm_bwd(const LstmGates &g, const float *vdiff, const float *gates, const float *out,
+                     const float *cell, const float *h_init, const float *c_init, fwp_view go,
+                     const float *ckpt, float *gz, float *gk, float *gv, float *gbeta, int N, int H,
+                     int L, int D, int chunk, hipStream_t s) {
+    size_t bytes = sizeof(float) * ((size_t)6 * D * pitch(D) + 19 * D + 1);
+    if (int rc = prepare(k_lstm_bwd, bytes)) return rc;
+    int nchunk = (L + chunk - 1) / chunk;
+    hipLaunchKernelGGL(k_lstm_bwd, dim3(N * H), dim3(NT), bytes, s, g, vdiff, gates, out, cell,
+                       h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, D, chunk, nchunk);
     return launched();
 }
 
