@@ -38,7 +38,8 @@ _SIGNATURES = {
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
 }
-EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device"])
+EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config"])
+CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED = 0, 0, 1, 2
 
 _lib = None
 _checked_devices = set()
@@ -62,6 +63,8 @@ def lib():
         handle.fwp_query.argtypes = [ctypes.c_int]
         handle.fwp_query.restype = ctypes.c_int
         handle.fwp_check_device.restype = ctypes.c_int
+        handle.fwp_config.argtypes = [ctypes.c_int, ctypes.c_int]
+        handle.fwp_config.restype = ctypes.c_int
         _lib = handle
     return _lib
 
@@ -76,6 +79,10 @@ def query(what):
 
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
+
+
+def config(key, value):
+    check(lib().fwp_config(int(key), int(value)), "fwp_config")
 
 
 def strerror(code):

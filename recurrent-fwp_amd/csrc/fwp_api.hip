@@ -20,9 +20,20 @@ int check_dims(int N, int H, int L, int E, int M, int chunk) {
     return 0;
 }
 
+// fwp_config(FWP_CFG_DELTA_KERNELS, .)
+int g_delta_kernels = FWP_DELTA_AUTO;
+
 }  // namespace
 
 extern "C" {
+
+int fwp_config(int key, int value) {
+    if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_CHUNKED) {
+        g_delta_kernels = value;
+        return FWP_OK;
+    }
+    return FWP_E_SHAPE;
+}
 
 const char *fwp_strerror(int code) {
     switch (code) {
@@ -66,9 +77,17 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
-        aligned16(vdiff) && aligned16(ckpt) && aligned16(out))
+        aligned16(vdiff) && aligned16(ckpt) && aligned16(out)) {
+        // blocks of 16 steps on the matrix cores pay off from about two blocks on; single steps
+        // (stepwise inference) stay on the scan kernel
+        const bool chunked = g_delta_kernels == FWP_DELTA_CHUNKED ||
+                             (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
+        if (chunked)
+            return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
+                                  (hipStream_t)stream);
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                              (hipStream_t)stream);
+    }
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
                              (hipStream_t)stream);
 }

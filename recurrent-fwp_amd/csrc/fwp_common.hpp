@@ -70,6 +70,10 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                   int L, int D, int chunk, hipStream_t s);
 
+// Chunked delta-rule forward on the matrix cores (same arguments and results as reg_delta_fwd).
+int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                   float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+
 // Sum rule on the same kernels (no v_old, beta = 1).
 int reg_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                 int L, int D, int chunk, hipStream_t s);

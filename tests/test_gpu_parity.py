@@ -39,8 +39,18 @@ DELTA_SHAPES = [
 ]
 
 
+@pytest.fixture(params=["scan", "chunked"])
+def delta_kernels(request, fwp):
+    """Both delta-rule forward kernels for D = 16/32: the step-by-step scan and the 16-step blocks
+    on the matrix cores (other shapes take the LDS kernels whatever the setting)."""
+    L_ = fwp._lib
+    L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED}[request.param])
+    yield request.param
+    L_.config(L_.CFG_DELTA_KERNELS, L_.DELTA_AUTO)
+
+
 @pytest.mark.parametrize("N,H,L,E,M,w0", DELTA_SHAPES)
-def test_delta(fwp, N, H, L, E, M, w0):
+def test_delta(fwp, delta_kernels, N, H, L, E, M, w0):
     q, k, v, beta, W0, go = delta_inputs(100 + L + E, N, H, L, E, M, w0=w0)
     tq, tk, tv, tb = (dev(x, True) for x in (q, k, v, beta))
     W = dev(W0)
@@ -54,7 +64,23 @@ def test_delta(fwp, N, H, L, E, M, w0):
     check("W after backward", W, ref_W)     # backward does not rewind the caller's state
 
 
-def test_delta_strided_views_and_segments(fwp):
+@pytest.mark.parametrize("L", [15, 16, 17, 31, 33, 47, 48, 100])
+@pytest.mark.parametrize("D", [16, 32])
+def test_delta_block_edges(fwp, delta_kernels, L, D):
+    # lengths around the 16-step block and 32-step prefetch boundaries of the blocked kernel
+    q, k, v, beta, W0, go = delta_inputs(500 + L + D, 2, 2, L, D, D, w0=True)
+    tq, tk, tv, tb = (dev(x, True) for x in (q, k, v, beta))
+    W = dev(W0)
+    out = fwp.fast_weight_delta(tq, tk, tv, tb, W)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("q k v beta".split(), (tq, tk, tv, tb), oracle.delta_bwd(q, k, v, beta, W0, go)):
+        check("grad_" + name, t.grad, r)
+
+
+def test_delta_strided_views_and_segments(fwp, delta_kernels):
     # inputs as the layers pass them: [L,N,H,*] storage permuted to [N,H,L,*], and a carried state
     N, H, L, D = 2, 3, 48, 16
     q, k, v, beta, W0, go = delta_inputs(7, N, H, L, D, D, w0=True)
