@@ -43,6 +43,9 @@ WORKLOADS = {
     "rnn": dict(B=64, H=8, T=256, D=32, flop_c=20, fwd_bytes=lambda D: (4 * D + 1) * 4,
                 bwd_bytes=lambda D: (8 * D + 2) * 4,
                 label="Delta RNN fast_rnn_v2 fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
+    "lstm": dict(B=64, H=8, T=256, D=32, flop_c=60, fwd_bytes=lambda D: (18 * D + 3) * 4,
+                 bwd_bytes=lambda D: (23 * D + 6) * 4,
+                 label="Delta LSTM fast_lstm_v4 fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
     "rec": dict(B=64, H=8, T=256, D=32, flop_c=38, fwd_bytes=lambda D: (4 * D + 1) * 4,
                 bwd_bytes=lambda D: (8 * D + 2) * 4,
                 label="Recurrent Delta Net rec_update_fwm_tanh fwd+bwd, B=64 H=8 T=256 D=32, fp32"),
@@ -51,12 +54,15 @@ WORKLOADS = {
 
 def make_inputs(name, w):
     import numpy as np
-    from helpers import delta_inputs, rec_inputs, rnn_inputs
+    from helpers import delta_inputs, lstm_inputs, rec_inputs, rnn_inputs
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
     if name.startswith("delta") or name == "sum":
         return delta_inputs(0, B, H, T, D, D, dtype=np.float32)
     if name == "rnn":
         return rnn_inputs(0, B, H, T, D, dtype=np.float32)
+    if name == "lstm":
+        Zs, Ks, Vs, Bs, Ws, h0, c0, go = lstm_inputs(0, B, H, T, D, dtype=np.float32)
+        return [*Zs, *Ks, *Vs, *Bs, *Ws, h0, c0, go]
     return rec_inputs(0, B, H, T, D, dtype=np.float32)
 
 
@@ -83,6 +89,21 @@ def gpu_step_fn(name, pkg, arrays):
         def step():
             W.zero_()
             out = pkg.fast_weight_sum(*diff, W)
+            torch.autograd.grad(out, diff, go)
+            return out
+    elif name == "lstm":
+        Zs, Ks, Vs, Bs, Ws = (dev[3 * i:3 * i + 3] for i in range(5))
+        h, c = dev[15].clone(), dev[16].clone()
+        diff = [t.requires_grad_(True) for t in (*Zs, *Ks, *Vs, *Bs)]
+        Ws = [w.clone() for w in Ws]
+
+        def step():
+            for t in (*Ws, h, c):
+                t.zero_()
+            args = []
+            for a in range(3):
+                args += [Zs[a], Ks[a], Vs[a], Bs[a], Ws[a]]
+            out, _ = pkg.fast_lstm_v4(*args, h, c)
             torch.autograd.grad(out, diff, go)
             return out
     elif name == "rnn":
@@ -132,7 +153,7 @@ def kernel_times(name, pkg, arrays, iters):
         nch = (T + chunk - 1) // chunk
         W = W0.clone()
         out, vdiff = torch.empty_like(v), torch.empty_like(v)
-        ckpt = torch.empty((N, H, nch, E, M), **f32)
+        ckpt = torch.empty(L.delta_ckpt_floats(N, H, T, E, M, chunk), **f32)
         gq, gk, gv, gb = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(beta)
 
         def fwd():
@@ -161,6 +182,39 @@ def kernel_times(name, pkg, arrays, iters):
             return lib.fwp_sum_bwd(view(q), view(k), view(v), view(go), L.ptr(ckpt), None, L.ptr(gq), L.ptr(gk),
                                    L.ptr(gv), N, H, T, E, M, chunk, stream_of())
         reset = lambda: W.copy_(W0)
+    elif name == "lstm":
+        import ctypes
+        Zs, Ks, Vs, Bs, Ws0 = (dev[3 * i:3 * i + 3] for i in range(5))
+        h0, c0 = dev[15], dev[16]
+        N, H, T, D = Zs[0].shape
+        nch = (T + chunk - 1) // chunk
+        Ws = [w.clone() for w in Ws0]
+        h, c = h0.clone(), c0.clone()
+        out, cell = torch.empty_like(Zs[0]), torch.empty_like(Zs[0])
+        gates, vdiff = torch.empty((3, N, H, T, D), **f32), torch.empty((3, N, H, T, D), **f32)
+        ckpt = torch.empty((3, N, H, nch, D, D), **f32)
+        gz, gk, gv = (torch.empty((3, N, H, T, D), **f32) for _ in range(3))
+        gb = torch.empty((3, N, H, T, 1), **f32)
+        views = lambda ts: (L.View * 3)(*[view(t) for t in ts])
+        Wp = (ctypes.c_void_p * 3)(*[w.data_ptr() for w in Ws])
+
+        def fwd():
+            return lib.fwp_lstm_fwd(views(Zs), views(Ks), views(Vs), views(Bs), Wp, L.ptr(h), L.ptr(c), L.ptr(out),
+                                    L.ptr(cell), L.ptr(gates), L.ptr(vdiff), L.ptr(ckpt), N, H, T, D, chunk,
+                                    stream_of())
+
+        def bwd():
+            return lib.fwp_lstm_bwd(views(Ks), views(Bs), L.ptr(vdiff), L.ptr(gates), L.ptr(out), L.ptr(cell),
+                                    L.ptr(h0), L.ptr(c0), view(go), L.ptr(ckpt), L.ptr(gz), L.ptr(gk), L.ptr(gv),
+                                    L.ptr(gb), N, H, T, D, chunk, stream_of())
+
+        W = Ws[0]
+
+        def reset():
+            for w, w0 in zip(Ws, Ws0):
+                w.copy_(w0)
+            h.copy_(h0)
+            c.copy_(c0)
     elif name == "rnn":
         z, k, v, W0, beta, h0 = dev[:6]
         N, H, T, D = z.shape
@@ -227,7 +281,10 @@ def kernel_times(name, pkg, arrays, iters):
 
     def abi_step():
         """state reset + forward + backward, straight through the C ABI on preallocated buffers"""
-        W.zero_()
+        if name == "lstm":
+            reset()
+        else:
+            W.zero_()
         if name in ("rnn", "rec"):
             h.zero_()
         L.check(fwd(), "forward")
@@ -251,6 +308,12 @@ def cpu_baseline(name, arrays, w, reps):
         loop, inputs, idx = torch_loop.delta_loop, ts[:5], [0, 1, 2, 3]
     elif name == "sum":
         loop, inputs, idx = torch_loop.sum_loop, [ts[0], ts[1], ts[2], ts[4]], [0, 1, 2]
+    elif name == "lstm":
+        order = []
+        for a in range(3):                       # (Z, K, V, beta, W) per gate, then h0, c0
+            order += [ts[a], ts[3 + a], ts[6 + a], ts[9 + a], ts[12 + a]]
+        loop, inputs = torch_loop.lstm_v4_loop, order + [ts[15], ts[16]]
+        idx = [5 * a + j for a in range(3) for j in range(4)]
     elif name == "rnn":
         loop, inputs, idx = torch_loop.rnn_v2_loop, ts[:6], [0, 1, 2, 4]
     else:

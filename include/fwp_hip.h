@@ -69,11 +69,20 @@ int fwp_config(int key, int value);
 int fwp_check_device(void);
 
 /*
+ * Number of floats the delta rule's `ckpt` buffer must hold (-1 for invalid dimensions):
+ * the N*H*nchunk*E*M checkpointed states and, for E = M in {16, 32}, a header and one 16x16
+ * matrix per 16 steps that the blocked forward kernel leaves for the blocked backward.
+ * No counterpart in the reference.
+ */
+long long fwp_delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);
+
+/*
  * Delta rule forward.  Replaces fast_weight_forward
  * (algorithmic/fast_weight/fast_weight_cuda.cu:182-240, kernel :17-178).
  *   q,k [N,H,L,E]  v [N,H,L,M]  beta [N,H,L,1]
  *   W [N,H,E,M] in/out: initial state in, state after step L-1 out
- *   out [N,H,L,M]; vdiff [N,H,L,M] = v - v_old; ckpt [N,H,nchunk,E,M]
+ *   out [N,H,L,M]; vdiff [N,H,L,M] = v - v_old;
+ *   ckpt: fwp_delta_ckpt_floats(...) floats, states first as [N,H,nchunk,E,M]
  * vdiff and ckpt may both be NULL for a forward that will not be differentiated.
  */
 int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,

@@ -38,7 +38,8 @@ _SIGNATURES = {
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
 }
-EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config"])
+EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
+                                       "fwp_delta_ckpt_floats"])
 CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED = 0, 0, 1, 2
 
 _lib = None
@@ -63,6 +64,8 @@ def lib():
         handle.fwp_query.argtypes = [ctypes.c_int]
         handle.fwp_query.restype = ctypes.c_int
         handle.fwp_check_device.restype = ctypes.c_int
+        handle.fwp_delta_ckpt_floats.argtypes = [ctypes.c_int] * 6
+        handle.fwp_delta_ckpt_floats.restype = ctypes.c_longlong
         handle.fwp_config.argtypes = [ctypes.c_int, ctypes.c_int]
         handle.fwp_config.restype = ctypes.c_int
         _lib = handle
@@ -79,6 +82,13 @@ def query(what):
 
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
+
+
+def delta_ckpt_floats(N, H, L, E, M, chunk):
+    n = int(lib().fwp_delta_ckpt_floats(N, H, L, E, M, chunk))
+    if n < 0:
+        raise FwpError(f"invalid dimensions N={N} H={H} L={L} E={E} M={M} chunk={chunk}")
+    return n
 
 
 def config(key, value):
@@ -114,14 +124,23 @@ def rows(t):
     buffer, such as v inside a fused q|k|v|beta projection): one elementwise pass costs far
     less than giving up the kernels that read rows with 16-byte loads.
     """
-    if t.dtype != torch.float32:
+    if t.dtype is not torch.float32:
         raise FwpError(f"fast-weight operators are fp32 only, got {t.dtype}")
     if t.dim() != 4:
         raise FwpError(f"expected a 4-D [N,H,L,D] tensor, got {t.dim()}-D")
+    if t.is_contiguous():            # the common case, kept short: this runs eight times per step
+        p = t.data_ptr()
+        _, h, l, d = t.shape
+        if d % 4 or p % 16 == 0:
+            ld = l * d
+            return t, View(p, h * ld, ld, d)
+        t = t.clone()
+        return t, View(t.data_ptr(), h * l * d, l * d, d)
     d = t.shape[-1]
-    if d != 1 and t.stride(-1) != 1:
+    sn, sh, sl, sd = t.stride()
+    if d != 1 and sd != 1:
         t = t.contiguous()
-    elif d % 4 == 0 and (t.data_ptr() % 16 or any(s % 4 for s in t.stride()[:3])):
+    elif d % 4 == 0 and (t.data_ptr() % 16 or sn % 4 or sh % 4 or sl % 4):
         t = t.contiguous()
     return t, View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 
@@ -130,8 +149,14 @@ def ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t):
-    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    """The current HIP stream of the tensor's device, as the C ABI takes it."""
+    if _raw_stream is not None:
+        return _raw_stream(t.device.index)
+    return torch.cuda.current_stream(t.device).cuda_stream
 
 
 class on_device:

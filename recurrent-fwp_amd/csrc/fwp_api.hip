@@ -59,6 +59,11 @@ int fwp_query(int what) {
     }
 }
 
+long long fwp_delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk) {
+    if (check_dims(N, H, L, E, M, chunk)) return -1;
+    return delta_ckpt_floats(N, H, L, E, M, chunk);
+}
+
 int fwp_check_device(void) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
@@ -85,9 +90,12 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
         if (chunked)
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                                   (hipStream_t)stream);
+        if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, chunk, (hipStream_t)stream)) return rc;
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                              (hipStream_t)stream);
     }
+    if (reg_delta_supported(E, M))
+        if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, chunk, (hipStream_t)stream)) return rc;
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
                              (hipStream_t)stream);
 }
@@ -100,9 +108,15 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
-        aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv))
+        aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv)) {
+        const bool chunked = g_delta_kernels == FWP_DELTA_CHUNKED ||
+                             (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
+        if (chunked)
+            return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
+                                  chunk, (hipStream_t)stream);
         return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
                              chunk, (hipStream_t)stream);
+    }
     return generic_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
                              chunk, (hipStream_t)stream);
 }

@@ -74,6 +74,14 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
 int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
 
+// Size of the delta rule's checkpoint buffer: the states, plus (E = M in {16, 32}) a header and one
+// 16x16 matrix per 16 steps that the blocked forward leaves for the blocked backward.
+int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);
+int delta_aux_invalidate(float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
+                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
+                   int L, int D, int chunk, hipStream_t s);
+
 // Sum rule on the same kernels (no v_old, beta = 1).
 int reg_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                 int L, int D, int chunk, hipStream_t s);

@@ -16,6 +16,7 @@
 // data movement between products; transposed inputs (K^T, Q^T) are single 16-byte loads per lane,
 // and the output is produced as O^T so that it leaves with 16-byte stores.  No LDS is used.
 #include "fwp_common.hpp"
+#include "fwp_wave.hpp"
 
 #include <type_traits>
 
@@ -34,6 +35,20 @@ __device__ __forceinline__ v4f tn(v4f X, v4f Y, v4f acc) {
 }
 
 constexpr int kBlk = 16;   // steps per block = MFMA tile edge
+constexpr int kAuxHeader = 16;   // floats before the per-block matrices in the auxiliary buffer
+
+// (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At
+// (accumulator layout): (I - At)(I + At^2)(I + At^4)(I + At^8), 8 products.
+__device__ __forceinline__ v4f inv_unit_triangular(v4f A, v4f At, v4f identity) {
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f T = identity - At;
+    const v4f A2 = tn(At, A, zero), At2 = tn(A, At, zero);
+    T = tn(A2, T, T);
+    const v4f A4 = tn(At2, A2, zero), At4 = tn(A2, At2, zero);
+    T = tn(A4, T, T);
+    const v4f A8 = tn(At4, A4, zero);
+    return tn(A8, T, T);
+}
 
 // Position of this lane's four registers in the accumulator layout.
 struct Geo16 {
@@ -127,13 +142,21 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
                                                        fwp_view beta, float *__restrict__ W,
                                                        float *__restrict__ out,
                                                        float *__restrict__ vdiff,
-                                                       float *__restrict__ ckpt, int H, int L,
+                                                       float *__restrict__ ckpt,
+                                                       float *__restrict__ aux, int H, int L,
                                                        int chunk, int nchunk) {
     constexpr int D = 16 * NB;
     const Geo16 p(threadIdx.x);
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
+    // aux (with ckpt): a header whose first float says that the per-block matrices T = (I + A)^-1
+    // follow, row-major, [sequence][block][16][16]; backward then does not invert again.
+    if (aux && seq == 0 && threadIdx.x == 0) aux[0] = 1.f;
+    float *aux_T = aux ? aux + kAuxHeader + seq * ((L + kBlk - 1) / kBlk) * 256 + c * 16 + 4 * g : nullptr;
+    auto save_T = [&](int ib, const v4f &Tt) {   // register r = T[c][4g + r]
+        if (aux_T) *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = make_float4(Tt[0], Tt[1], Tt[2], Tt[3]);
+    };
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
                 *bb = row(beta, n, h, 0);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
@@ -247,6 +270,7 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
                     make_float4(Ot[mb][0], Ot[mb][1], Ot[mb][2], Ot[mb][3]);
         }
         pre_stage(3, nxt, pre_nxt);
+        if (t0 + kBlk < L) save_T(ib + 1, pre_nxt.Tt);
         if (vdiff) {
 #pragma unroll
             for (int mb = 0; mb < NB; mb++) {
@@ -277,6 +301,7 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
     load_block(rawB, kBlk);
 #pragma unroll
     for (int st = 0; st < 4; st++) pre_stage(st, rawA, preA);
+    save_T(0, preA.Tt);
     const std::true_type full;
     const std::false_type ragged;
     auto step = [&](int ib, const RawBlock<NB> &cur, const RawBlock<NB> &nxt, RawBlock<NB> &fut,
@@ -298,17 +323,327 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
                 W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
 }
 
+// ----------------------------------------------------------------- backward
+//
+// Blocked reverse pass.  With S0 the state at the start of a block, U = diag(b) d (d = v - v_old, saved
+// by forward), T = (I + A)^-1, Pm = lower(Q K^T), dO the block's upstream gradient and dS the
+// gradient of the state after the block:
+//     dU = K dS + Pm^T dO            dY = T^T dU  (gradient of u with its effect on later steps)
+//     g_beta = rowsum(dY . d)        dX = diag(b) dY = g_v
+//     dPm = lower(dO U^T)            M = strict_lower(dX U^T)
+//     g_q = dO S0^T + dPm K
+//     g_k = U dS^T + dPm^T Q - dX S0^T - (M + M^T) K
+//     dS <- dS + Q^T dO - K^T dX
+// The state is kept transposed (all its uses contract over the value index) and is rewound block
+// by block from the checkpoints, S0^T = S'^T - U^T K.  Gradients are produced transposed so that
+// they leave with 16-byte stores.
+
+template <int NB>
+struct RawBwd {
+    v4f Kt[NB], Qt[NB], Kc[NB], Qc[NB], Oc[NB], Ot[NB], Dc[NB], Dt[NB];   // O: upstream gradient, D: vdiff
+    v4f T;                   // (I + A)^-1 when forward saved it
+    float bcol, brow[4];
+};
+
+template <int NB>
+__global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, fwp_view beta,
+                                                       const float *__restrict__ vdiff, fwp_view go,
+                                                       const float *__restrict__ ckpt,
+                                                       const float *__restrict__ aux,
+                                                       float *__restrict__ gq, float *__restrict__ gk,
+                                                       float *__restrict__ gv,
+                                                       float *__restrict__ gbeta, int H, int L,
+                                                       int chunk, int nchunk) {
+    constexpr int D = 16 * NB;
+    const Geo16 p(threadIdx.x);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
+                *bb = row(beta, n, h, 0), *db = vdiff + seq * L * D;
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f ident;
+#pragma unroll
+    for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+    // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
+    const bool have_T = aux && aux[0] == 1.f;
+    const float *aux_T = have_T ? aux + kAuxHeader + seq * ((L + kBlk - 1) / kBlk) * 256 + 4 * g * 16 + c : nullptr;
+
+    // per-lane element offsets inside a block (32-bit: a block spans 16 rows)
+    unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g),
+             o_ot = (unsigned)(c * go.sL + 4 * g), o_dt = (unsigned)(c * D + 4 * g),
+             o_bc = (unsigned)(c * beta.sL);
+    unsigned o_kr[4], o_qr[4], o_or[4], o_dr[4], o_br[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + c);
+        o_or[r] = (unsigned)((4 * g + r) * go.sL + c);
+        o_dr[r] = (unsigned)((4 * g + r) * D + c);
+        o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+    }
+    auto as_v4f = [](const float *ptr) {
+        const float4 x = *reinterpret_cast<const float4 *>(ptr);
+        return v4f{x.x, x.y, x.z, x.w};
+    };
+    auto load = [&](RawBwd<NB> &w, int t0) {
+        if (have_T) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.T[r] = aux_T[(int64_t)(t0 / kBlk) * 256 + 16 * r];
+        }
+        if (t0 + kBlk <= L) {    // whole block inside the sequence: uniform block base + lane offsets
+            const float *kblk = kb + (int64_t)t0 * k.sL, *qblk = qb + (int64_t)t0 * q.sL,
+                        *oblk = gob + (int64_t)t0 * go.sL, *dblk = db + (int64_t)t0 * D,
+                        *bblk = bb + (int64_t)t0 * beta.sL;
+            w.bcol = bblk[o_bc];
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.brow[r] = bblk[o_br[r]];
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
+                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+                w.Ot[b] = as_v4f(oblk + (o_ot + 16 * b));
+                w.Dt[b] = as_v4f(dblk + (o_dt + 16 * b));
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
+                    w.Qc[b][r] = qblk[o_qr[r] + 16 * b];
+                    w.Oc[b][r] = oblk[o_or[r] + 16 * b];
+                    w.Dc[b][r] = dblk[o_dr[r] + 16 * b];
+                }
+            }
+            return;
+        }
+        // ragged last block; rows beyond L: clamped loads, beta = 0 and a zero upstream gradient
+        const bool col_ok = t0 + c < L;
+        const int64_t tc = min(t0 + c, L - 1);
+        w.bcol = col_ok ? bb[tc * beta.sL] : 0.f;
+        int64_t tr[4];
+        bool row_ok[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            row_ok[r] = t0 + 4 * g + r < L;
+            tr[r] = min(t0 + 4 * g + r, L - 1);
+            w.brow[r] = row_ok[r] ? bb[tr[r] * beta.sL] : 0.f;
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const int ct = 16 * b + 4 * g, cc = 16 * b + c;
+            const float4 kk = *reinterpret_cast<const float4 *>(kb + tc * k.sL + ct);
+            const float4 qq = *reinterpret_cast<const float4 *>(qb + tc * q.sL + ct);
+            const float4 oo = *reinterpret_cast<const float4 *>(gob + tc * go.sL + ct);
+            const float4 dd = *reinterpret_cast<const float4 *>(db + tc * D + ct);
+            w.Kt[b] = v4f{kk.x, kk.y, kk.z, kk.w};
+            w.Qt[b] = v4f{qq.x, qq.y, qq.z, qq.w};
+            w.Ot[b] = col_ok ? v4f{oo.x, oo.y, oo.z, oo.w} : zero;
+            w.Dt[b] = v4f{dd.x, dd.y, dd.z, dd.w};
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Kc[b][r] = kb[tr[r] * k.sL + cc];
+                w.Qc[b][r] = qb[tr[r] * q.sL + cc];
+                w.Oc[b][r] = row_ok[r] ? gob[tr[r] * go.sL + cc] : 0.f;
+                w.Dc[b][r] = db[tr[r] * D + cc];
+            }
+        }
+    };
+
+    // St[mb][eb]: register r = S[16eb + c][16mb + 4g + r]  (block (mb, eb) of S^T)
+    // dS[eb][mb]: register r = dS[16eb + 4g + r][16mb + c]
+    v4f St[NB][NB], dS[NB][NB];
+#pragma unroll
+    for (int a = 0; a < NB; a++)
+#pragma unroll
+        for (int b = 0; b < NB; b++) dS[a][b] = zero;
+
+    auto block = [&](auto full_tag, int ib, const RawBwd<NB> &w) {
+        constexpr bool FULL = decltype(full_tag)::value;     // the block lies inside the sequence
+        const int t0 = ib * kBlk;
+        const int t_end = min(t0 + kBlk, L);
+        if (t_end % chunk == 0 || t_end == L) {      // last block of a chunk: the state after it is checkpointed
+            const float *src = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+                for (int eb = 0; eb < NB; eb++) {
+                    const float4 x = *reinterpret_cast<const float4 *>(src + (16 * eb + c) * D + 16 * mb + 4 * g);
+                    St[mb][eb] = v4f{x.x, x.y, x.z, x.w};
+                }
+        }
+        v4f U[NB], Ut[NB], nU[NB];
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            Ut[mb] = w.bcol * w.Dt[mb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) U[mb][r] = w.brow[r] * w.Dc[mb][r];
+            nU[mb] = -U[mb];
+        }
+        // state at the start of the block, transposed: S0^T = S'^T - U^T K
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) St[mb][eb] = tn(nU[mb], w.Kc[eb], St[mb][eb]);
+
+        // Pm = lower(Q K^T); T = (I + A)^-1 from forward, or inverted again here
+        v4f QK = zero;
+#pragma unroll
+        for (int b = 0; b < NB; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
+        v4f Pm;
+#pragma unroll
+        for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
+        v4f T = w.T;
+        if (!have_T) {
+            v4f G = zero, A, At;
+#pragma unroll
+            for (int b = 0; b < NB; b++) G = tn(w.Kt[b], w.Kt[b], G);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
+                At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
+            }
+            T = inv_unit_triangular(At, A, ident);      // (I + A)^-1
+        }
+
+        // gradient of u and everything that hangs off it
+        v4f dX[NB], dXt[NB], ndX[NB], ndXt[NB];
+        float gb = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            v4f dU = tn(Pm, w.Oc[mb], zero);
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) dU = tn(w.Kt[eb], dS[eb][mb], dU);
+            const v4f dY = tn(T, dU, zero), dYt = tn(dU, T, zero);
+            dXt[mb] = w.bcol * dYt;
+            ndXt[mb] = -dXt[mb];
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                dX[mb][r] = w.brow[r] * dY[r];
+                gb = fmaf(dYt[r], w.Dt[mb][r], gb);
+            }
+            ndX[mb] = -dX[mb];
+            if (FULL || t0 + c < L)        // g_v: register r = dX[t0 + c][16mb + 4g + r]
+                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                    make_float4(dXt[mb][0], dXt[mb][1], dXt[mb][2], dXt[mb][3]);
+        }
+        {   // g_beta[t0 + c] = sum over the value index: the four 16-lane rows hold partial sums
+            float y = gb;
+            swap16(gb, y);
+            gb += y;
+            y = gb;
+            swap32(gb, y);
+            gb += y;
+            if (g == 0 && (FULL || t0 + c < L)) gbeta[seq * L + t0 + c] = gb;
+        }
+        v4f Z = zero, Zt = zero, M = zero, Mt = zero;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            Z = tn(w.Ot[mb], Ut[mb], Z);          // dO U^T
+            Zt = tn(Ut[mb], w.Ot[mb], Zt);
+            M = tn(dXt[mb], Ut[mb], M);           // dX U^T
+            Mt = tn(Ut[mb], dXt[mb], Mt);
+        }
+        v4f dPm, dPmt, nMs;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
+            dPmt[r] = (p.up[r] || p.di[r]) ? Zt[r] : 0.f;
+            nMs[r] = -((p.lo[r] ? M[r] : 0.f) + (p.up[r] ? Mt[r] : 0.f));
+        }
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) {
+            v4f gQt = tn(w.Kc[eb], dPmt, zero);
+            v4f gKt = tn(w.Qc[eb], dPm, zero);
+            gKt = tn(w.Kc[eb], nMs, gKt);
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) {
+                const v4f dSt = tn(dS[eb][mb], ident, zero);       // block (mb, eb) of dS^T
+                gQt = tn(St[mb][eb], w.Ot[mb], gQt);
+                gKt = tn(dSt, Ut[mb], gKt);
+                gKt = tn(St[mb][eb], ndXt[mb], gKt);
+            }
+            if (FULL || t0 + c < L) {
+                float *dq = gq + (seq * L + t0 + c) * D + 16 * eb + 4 * g;
+                float *dk = gk + (seq * L + t0 + c) * D + 16 * eb + 4 * g;
+                *reinterpret_cast<float4 *>(dq) = make_float4(gQt[0], gQt[1], gQt[2], gQt[3]);
+                *reinterpret_cast<float4 *>(dk) = make_float4(gKt[0], gKt[1], gKt[2], gKt[3]);
+            }
+        }
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) {
+                dS[eb][mb] = tn(w.Qc[eb], w.Oc[mb], dS[eb][mb]);
+                dS[eb][mb] = tn(w.Kc[eb], ndX[mb], dS[eb][mb]);
+            }
+    };
+
+    const int nblk = (L + kBlk - 1) / kBlk;
+    RawBwd<NB> rawA, rawB;
+    load(rawA, (nblk - 1) * kBlk);
+    auto step = [&](int ib, const RawBwd<NB> &w) {
+        if ((ib + 1) * kBlk <= L) block(std::true_type(), ib, w);
+        else block(std::false_type(), ib, w);
+    };
+    for (int ib = nblk - 1; ib >= 0; ib -= 2) {
+        load(rawB, max(ib - 1, 0) * kBlk);
+        step(ib, rawA);
+        if (ib >= 1) {
+            load(rawA, max(ib - 2, 0) * kBlk);
+            step(ib - 1, rawB);
+        }
+    }
+}
+
 }  // namespace
+
+int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    int64_t n = (int64_t)N * H * nchunk * E * M;
+    if (reg_delta_supported(E, M)) n += kAuxHeader + (int64_t)N * H * ((L + kBlk - 1) / kBlk) * 256;
+    return n;
+}
+
+// The auxiliary part of the checkpoint buffer starts right after the states.
+static float *aux_of(const float *ckpt, int N, int H, int L, int D, int chunk) {
+    if (!ckpt) return nullptr;
+    const int nchunk = (L + chunk - 1) / chunk;
+    return const_cast<float *>(ckpt) + (int64_t)N * H * nchunk * D * D;
+}
+
+namespace {
+__global__ void k_store_float(float *dst, float x) { *dst = x; }
+}  // namespace
+
+// Forward kernels that do not leave the per-block matrices say so in the header.
+int delta_aux_invalidate(float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
+    if (!ckpt) return 0;
+    hipLaunchKernelGGL(k_store_float, dim3(1), dim3(1), 0, s, aux_of(ckpt, N, H, L, D, chunk), 0.f);
+    return (int)hipGetLastError();
+}
 
 int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
+    float *aux = aux_of(ckpt, N, H, L, D, chunk);
     if (D == 16)
         hipLaunchKernelGGL(k_delta_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
-                           vdiff, ckpt, H, L, chunk, nchunk);
+                           vdiff, ckpt, aux, H, L, chunk, nchunk);
     else
         hipLaunchKernelGGL(k_delta_fwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
-                           vdiff, ckpt, H, L, chunk, nchunk);
+                           vdiff, ckpt, aux, H, L, chunk, nchunk);
+    return (int)hipGetLastError();
+}
+
+int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
+                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
+                   int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    const float *aux = aux_of(ckpt, N, H, L, D, chunk);
+    if (D == 16)
+        hipLaunchKernelGGL(k_delta_bwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, beta, vdiff, go,
+                           ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+    else
+        hipLaunchKernelGGL(k_delta_bwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, beta, vdiff, go,
+                           ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
     return (int)hipGetLastError();
 }
 

@@ -39,7 +39,8 @@ class DeltaFastWeight(torch.autograd.Function):
         vdiff = ckpt = None
         if need_grad:
             vdiff = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
-            ckpt = torch.empty((N, H, _nchunk(L, chunk), E, M), device=Q.device, dtype=torch.float32)
+            ckpt = torch.empty(_lib.delta_ckpt_floats(N, H, L, E, M, chunk), device=Q.device,
+                               dtype=torch.float32)
         with _lib.on_device(Q):
             rc = _lib.lib().fwp_delta_fwd(
                 qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out),
@@ -49,6 +50,7 @@ class DeltaFastWeight(torch.autograd.Function):
         if need_grad:
             ctx.save_for_backward(Q, K, beta, vdiff, ckpt)
             ctx.dims = (N, H, L, E, M, chunk)
+            ctx.views = (qv, kv, bv)        # of the saved tensors, which keep the memory alive
         ctx.set_materialize_grads(False)
         return out
 
@@ -58,9 +60,7 @@ class DeltaFastWeight(torch.autograd.Function):
             return None, None, None, None, None
         Q, K, beta, vdiff, ckpt = ctx.saved_tensors
         N, H, L, E, M, chunk = ctx.dims
-        _, qv = _lib.rows(Q)
-        _, kv = _lib.rows(K)
-        _, bv = _lib.rows(beta)
+        qv, kv, bv = ctx.views
         grad_out, gv_ = _lib.rows(grad_out)
         grad_Q = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
         grad_K = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
