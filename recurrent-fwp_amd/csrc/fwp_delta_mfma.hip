@@ -226,12 +226,49 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
     // `pre_cur`) interleaved with the stages of block ib + 1 (`nxt` -> `pre_nxt`), while the loads of
     // block ib + 2 (`fut`) are in flight.  Everything past the end is clamped and its results unused,
     // so the body is one basic block for the scheduler.
+    // Results of a block are kept in registers and stored at the top of the next block, right
+    // after its prefetch loads: the memory counter is shared by loads and stores and waits on it
+    // come out as "everything outstanding", so a store must be a block old by the time the next
+    // wait comes or that wait pays the store's latency.
+    v4f pend_O[NB], pend_D[NB], pend_T;
+    auto flush = [&](auto full_tag, int ib) {        // stores of block ib; S still is the state after it
+        constexpr bool FULL = decltype(full_tag)::value;
+        const int t0 = ib * kBlk;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            if (FULL || t0 + c < L)         // register r = O[t0 + c][16mb + 4g + r]
+                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                    make_float4(pend_O[mb][0], pend_O[mb][1], pend_O[mb][2], pend_O[mb][3]);
+            if (vdiff) {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (FULL || t0 + 4 * g + r < L)
+                        vdiff[(seq * L + t0 + 4 * g + r) * D + 16 * mb + c] = pend_D[mb][r];
+            }
+        }
+        if (t0 + kBlk < L) save_T(ib + 1, pend_T);
+        const int t_end = min(t0 + kBlk, L);
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+                for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+        }
+    };
+
     auto block = [&](auto full_tag, int ib, const RawBlock<NB> &cur, const RawBlock<NB> &nxt,
                      RawBlock<NB> &fut, const PreBlock &pre_cur, PreBlock &pre_nxt) {
         constexpr bool FULL = decltype(full_tag)::value;   // blocks ib .. ib+2 lie inside the sequence
         const int t0 = ib * kBlk;
         if constexpr (FULL) fut.load_full(q, k, v, beta, qb, kb, vb, bb, lo, t0 + 2 * kBlk);
         else fut.load_clamped(q, k, v, beta, qb, kb, vb, bb, t0 + 2 * kBlk, L, p);
+        if (ib > 0) flush(std::true_type(), ib - 1);
+        // loads and stores stay here, a whole block ahead of the next wait
+        __builtin_amdgcn_sched_barrier(0);
 
         v4f X[NB], U[NB], Ot[NB];
 #pragma unroll
@@ -263,57 +300,39 @@ __global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, f
         pre_stage(2, nxt, pre_nxt);
 #pragma unroll
         for (int mb = 0; mb < NB; mb++) {
-            Ot[mb] = tn(U[mb], pre_cur.Rm, Ot[mb]);
-            // register r = O[t0 + c][16mb + 4g + r]
-            if (FULL || t0 + c < L)
-                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
-                    make_float4(Ot[mb][0], Ot[mb][1], Ot[mb][2], Ot[mb][3]);
+            pend_O[mb] = tn(U[mb], pre_cur.Rm, Ot[mb]);
         }
         pre_stage(3, nxt, pre_nxt);
-        if (t0 + kBlk < L) save_T(ib + 1, pre_nxt.Tt);
+        pend_T = pre_nxt.Tt;
         if (vdiff) {
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) {
-                const v4f GU = tn(pre_cur.Gu, U[mb], zero);
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (FULL || t0 + 4 * g + r < L)
-                        vdiff[(seq * L + t0 + 4 * g + r) * D + 16 * mb + c] = X[mb][r] - GU[r];
-            }
-        }
-        const int t_end = min(t0 + kBlk, L);
-        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
-            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
-#pragma unroll
-            for (int eb = 0; eb < NB; eb++)
-#pragma unroll
-                for (int mb = 0; mb < NB; mb++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+            for (int mb = 0; mb < NB; mb++) pend_D[mb] = X[mb] - tn(pre_cur.Gu, U[mb], zero);
         }
     };
 
-    // three raw buffers and three results rotate through the roles, so nothing is copied
-    RawBlock<NB> rawA, rawB, rawC;
-    PreBlock preA, preB, preC;
-    load_block(rawA, 0);
-    load_block(rawB, kBlk);
+    // Main loop: the blocks whose prefetch (two blocks on) still lies inside the sequence; the last
+    // blocks take the clamped variant.
+    RawBlock<NB> cur, nxt, fut;
+    PreBlock pre_cur, pre_nxt;
+    load_block(cur, 0);
+    load_block(nxt, kBlk);
 #pragma unroll
-    for (int st = 0; st < 4; st++) pre_stage(st, rawA, preA);
-    save_T(0, preA.Tt);
-    const std::true_type full;
-    const std::false_type ragged;
-    auto step = [&](int ib, const RawBlock<NB> &cur, const RawBlock<NB> &nxt, RawBlock<NB> &fut,
-                    const PreBlock &pre_cur, PreBlock &pre_nxt) {
-        if ((ib + 3) * kBlk <= L) block(full, ib, cur, nxt, fut, pre_cur, pre_nxt);
-        else block(ragged, ib, cur, nxt, fut, pre_cur, pre_nxt);
-    };
-    for (int ib = 0; ib < nblk; ib += 3) {
-        step(ib, rawA, rawB, rawC, preA, preB);
-        if (ib + 1 < nblk) step(ib + 1, rawB, rawC, rawA, preB, preC);
-        if (ib + 2 < nblk) step(ib + 2, rawC, rawA, rawB, preC, preA);
+    for (int st = 0; st < 4; st++) pre_stage(st, cur, pre_cur);
+    save_T(0, pre_cur.Tt);
+    int ib = 0;
+    for (; (ib + 3) * kBlk <= L; ib++) {
+        block(std::true_type(), ib, cur, nxt, fut, pre_cur, pre_nxt);
+        cur = nxt;
+        nxt = fut;
+        pre_cur = pre_nxt;
     }
+    for (; ib < nblk; ib++) {
+        block(std::false_type(), ib, cur, nxt, fut, pre_cur, pre_nxt);
+        cur = nxt;
+        nxt = fut;
+        pre_cur = pre_nxt;
+    }
+    flush(std::false_type(), nblk - 1);
 #pragma unroll
     for (int eb = 0; eb < NB; eb++)
 #pragma unroll
@@ -342,6 +361,7 @@ template <int NB>
 struct RawBwd {
     v4f Kt[NB], Qt[NB], Kc[NB], Qc[NB], Oc[NB], Ot[NB], Dc[NB], Dt[NB];   // O: upstream gradient, D: vdiff
     v4f T;                   // (I + A)^-1 when forward saved it
+    v4f Sck[NB][NB];         // checkpointed state of the block's chunk, transposed (used by the chunk's last block)
     float bcol, brow[4];
 };
 
@@ -387,6 +407,14 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
         return v4f{x.x, x.y, x.z, x.w};
     };
     auto load = [&](RawBwd<NB> &w, int t0) {
+        {   // always loaded, so that no load is left to be issued (and waited for) inside the block
+            const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * D * D;
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+                for (int eb = 0; eb < NB; eb++)
+                    w.Sck[mb][eb] = as_v4f(src + (16 * eb + c) * D + 16 * mb + 4 * g);
+        }
         if (have_T) {
 #pragma unroll
             for (int r = 0; r < 4; r++) w.T[r] = aux_T[(int64_t)(t0 / kBlk) * 256 + 16 * r];
@@ -455,19 +483,37 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
 #pragma unroll
         for (int b = 0; b < NB; b++) dS[a][b] = zero;
 
+    // Gradients of a block wait in registers and are stored at the top of the next block (see the
+    // forward kernel).
+    v4f pend_gv[NB], pend_gq[NB], pend_gk[NB];
+    float pend_gb = 0.f;
+    auto flush = [&](auto full_tag, int ib) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        const int t0 = ib * kBlk;
+        if (FULL || t0 + c < L) {      // register r = gradient[t0 + c][16b + 4g + r]
+            const int64_t o = (seq * L + t0 + c) * D + 4 * g;
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                *reinterpret_cast<float4 *>(gv + o + 16 * b) =
+                    make_float4(pend_gv[b][0], pend_gv[b][1], pend_gv[b][2], pend_gv[b][3]);
+                *reinterpret_cast<float4 *>(gq + o + 16 * b) =
+                    make_float4(pend_gq[b][0], pend_gq[b][1], pend_gq[b][2], pend_gq[b][3]);
+                *reinterpret_cast<float4 *>(gk + o + 16 * b) =
+                    make_float4(pend_gk[b][0], pend_gk[b][1], pend_gk[b][2], pend_gk[b][3]);
+            }
+            if (g == 0) gbeta[seq * L + t0 + c] = pend_gb;
+        }
+    };
+
     auto block = [&](auto full_tag, int ib, const RawBwd<NB> &w) {
         constexpr bool FULL = decltype(full_tag)::value;     // the block lies inside the sequence
         const int t0 = ib * kBlk;
         const int t_end = min(t0 + kBlk, L);
         if (t_end % chunk == 0 || t_end == L) {      // last block of a chunk: the state after it is checkpointed
-            const float *src = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
 #pragma unroll
             for (int mb = 0; mb < NB; mb++)
 #pragma unroll
-                for (int eb = 0; eb < NB; eb++) {
-                    const float4 x = *reinterpret_cast<const float4 *>(src + (16 * eb + c) * D + 16 * mb + 4 * g);
-                    St[mb][eb] = v4f{x.x, x.y, x.z, x.w};
-                }
+                for (int eb = 0; eb < NB; eb++) St[mb][eb] = w.Sck[mb][eb];
         }
         v4f U[NB], Ut[NB], nU[NB];
 #pragma unroll
@@ -520,9 +566,7 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
                 gb = fmaf(dYt[r], w.Dt[mb][r], gb);
             }
             ndX[mb] = -dX[mb];
-            if (FULL || t0 + c < L)        // g_v: register r = dX[t0 + c][16mb + 4g + r]
-                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
-                    make_float4(dXt[mb][0], dXt[mb][1], dXt[mb][2], dXt[mb][3]);
+            pend_gv[mb] = dXt[mb];
         }
         {   // g_beta[t0 + c] = sum over the value index: the four 16-lane rows hold partial sums
             float y = gb;
@@ -531,7 +575,7 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
             y = gb;
             swap32(gb, y);
             gb += y;
-            if (g == 0 && (FULL || t0 + c < L)) gbeta[seq * L + t0 + c] = gb;
+            pend_gb = gb;
         }
         v4f Z = zero, Zt = zero, M = zero, Mt = zero;
 #pragma unroll
@@ -560,12 +604,8 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
                 gKt = tn(dSt, Ut[mb], gKt);
                 gKt = tn(St[mb][eb], ndXt[mb], gKt);
             }
-            if (FULL || t0 + c < L) {
-                float *dq = gq + (seq * L + t0 + c) * D + 16 * eb + 4 * g;
-                float *dk = gk + (seq * L + t0 + c) * D + 16 * eb + 4 * g;
-                *reinterpret_cast<float4 *>(dq) = make_float4(gQt[0], gQt[1], gQt[2], gQt[3]);
-                *reinterpret_cast<float4 *>(dk) = make_float4(gKt[0], gKt[1], gKt[2], gKt[3]);
-            }
+            pend_gq[eb] = gQt;
+            pend_gk[eb] = gKt;
         }
 #pragma unroll
         for (int eb = 0; eb < NB; eb++)
@@ -576,21 +616,31 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
             }
     };
 
+    // The ragged last block first (clamped variant), then one straight-line loop over whole blocks.
     const int nblk = (L + kBlk - 1) / kBlk;
-    RawBwd<NB> rawA, rawB;
-    load(rawA, (nblk - 1) * kBlk);
-    auto step = [&](int ib, const RawBwd<NB> &w) {
-        if ((ib + 1) * kBlk <= L) block(std::true_type(), ib, w);
-        else block(std::false_type(), ib, w);
-    };
-    for (int ib = nblk - 1; ib >= 0; ib -= 2) {
-        load(rawB, max(ib - 1, 0) * kBlk);
-        step(ib, rawA);
-        if (ib >= 1) {
-            load(rawA, max(ib - 2, 0) * kBlk);
-            step(ib - 1, rawB);
-        }
+    RawBwd<NB> cur, nxt;
+    load(cur, (nblk - 1) * kBlk);
+    int ib = nblk - 1;
+    const bool ragged = nblk * kBlk != L;
+    if (ragged) {
+        load(nxt, max(ib - 1, 0) * kBlk);
+        __builtin_amdgcn_sched_barrier(0);
+        block(std::false_type(), ib, cur);
+        cur = nxt;
+        ib--;
     }
+    for (; ib >= 0; ib--) {
+        load(nxt, max(ib - 1, 0) * kBlk);
+        if (ib + 1 < nblk) {        // the block done before this one
+            if (ragged && ib + 2 == nblk) flush(std::false_type(), ib + 1);
+            else flush(std::true_type(), ib + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);      // loads and stores stay a whole block ahead of the next wait
+        block(std::true_type(), ib, cur);
+        cur = nxt;
+    }
+    if (nblk == 1 && ragged) flush(std::false_type(), 0);
+    else flush(std::true_type(), 0);
 }
 
 }  // namespace
