@@ -189,6 +189,13 @@ int fwp_lstm_fwd(const fwp_view *z, const fwp_view *k, const fwp_view *v, const 
     const int saved = (gates != nullptr) + (vdiff != nullptr) + (ckpt != nullptr);
     if (saved != 0 && saved != 3) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    bool reg = reg_lstm_supported(D) && aligned16(h) && aligned16(c) && aligned16(out) &&
+               aligned16(cell) && aligned16(gates) && aligned16(vdiff) && aligned16(ckpt);
+    for (int a = 0; a < 3; a++)
+        reg = reg && reg_view_ok(z[a]) && reg_view_ok(k[a]) && reg_view_ok(v[a]) && aligned16(W[a]);
+    if (reg)
+        return reg_lstm_fwd(g, h, c, out, cell, gates, vdiff, ckpt, N, H, L, D, chunk,
+                            (hipStream_t)stream);
     return generic_lstm_fwd(g, h, c, out, cell, gates, vdiff, ckpt, N, H, L, D, chunk,
                             (hipStream_t)stream);
 }
@@ -206,6 +213,13 @@ int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff, co
         g.k[a] = k[a]; g.beta[a] = beta[a];
     }
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    bool reg = reg_lstm_supported(D) && reg_view_ok(grad_out) && aligned16(vdiff) && aligned16(gates) &&
+               aligned16(out) && aligned16(cell) && aligned16(h_init) && aligned16(c_init) &&
+               aligned16(ckpt) && aligned16(gz) && aligned16(gk) && aligned16(gv);
+    for (int a = 0; a < 3; a++) reg = reg && reg_view_ok(k[a]);
+    if (reg)
+        return reg_lstm_bwd(g, vdiff, gates, out, cell, h_init, c_init, grad_out, ckpt, gz, gk, gv,
+                            gbeta, N, H, L, D, chunk, (hipStream_t)stream);
     return generic_lstm_bwd(g, vdiff, gates, out, cell, h_init, c_init, grad_out, ckpt, gz, gk, gv,
                             gbeta, N, H, L, D, chunk, (hipStream_t)stream);
 }

@@ -96,6 +96,14 @@ int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                 const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
                 float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s);
 
+bool reg_lstm_supported(int D);
+int reg_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, float *gates,
+                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+int reg_lstm_bwd(const LstmGates &g, const float *vdiff, const float *gates, const float *out,
+                 const float *cell, const float *h_init, const float *c_init, fwp_view go,
+                 const float *ckpt, float *gz, float *gk, float *gv, float *gbeta, int N, int H, int L,
+                 int D, int chunk, hipStream_t s);
+
 bool reg_rec_supported(int D);
 int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
                 const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,

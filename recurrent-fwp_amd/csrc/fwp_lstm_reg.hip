@@ -1,0 +1,497 @@
+// Register-state kernels of the Delta LSTM v4 for D in {16, 32}: three delta-rule memories (gate
+// order i, u, o), each held like the single memory of the Delta RNN kernels (fwp_rnn_reg.hip), read
+// with the softmax of the previous output; i = sigmoid, u linear, o = sigmoid, c = i u + (1 - i) c,
+// h = o c.  One wave64 per sequence.  Tiles of TL steps (8 at D = 32, 16 at D = 16) keep the LDS
+// footprint of the nine (fifteen in backward) streamed tensors small enough for several waves per CU.
+//
+// Backward: what the cell needs per step is four coefficients, o, c o (1 - o), (u - c_prev) i (1 - i)
+// and i; like the softmax of the delayed output they are computed for a whole tile when the tile is
+// committed, off the sequential path.
+#include "fwp_reg.hpp"
+
+namespace fwp {
+namespace {
+
+__device__ __forceinline__ float sigmoidf_fast(float x) { return __fdividef(1.f, 1.f + __expf(-x)); }
+
+template <int D>
+constexpr int lstm_tile() { return D == 32 ? 8 : 16; }
+
+// ------------------------------------------------------------------ forward
+
+template <int D>
+struct LstmFwdOps {
+    float k[3][Geo<D>::NP], v[3], z[3], b[3];
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_lstm_fwd_reg(LstmGates g, float *__restrict__ hstate,
+                                                              float *__restrict__ cstate,
+                                                              float *__restrict__ out,
+                                                              float *__restrict__ cell,
+                                                              float *__restrict__ gates,
+                                                              float *__restrict__ vdiff,
+                                                              float *__restrict__ ckpt, int N, int H,
+                                                              int L, int chunk, int nchunk, int nseq) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    using Tile = TileRegs<D, TL>;
+    static_assert(TL % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sz_[WPB][3][2][TL * D];
+    __shared__ __align__(16) float sk_[WPB][3][2][TL * D];
+    __shared__ __align__(16) float sv_[WPB][3][2][TL * D];
+    __shared__ __align__(16) float sb_[WPB][3][2][16];
+    // staged outputs: vdiff i,u,o, gates i,u,o, out, cell
+    __shared__ __align__(16) float sout_[WPB][8][TL * D + 16];
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sz = sz_[wave];
+    auto &sk = sk_[wave];
+    auto &sv = sv_[wave];
+    auto &sb = sb_[wave];
+    auto &sout = sout_[wave];
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+
+    float Wc[3][R];  // W_a[reg_index(jj)][col]
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++)
+            Wc[a][jj] = g.W[a][(seq * D + reg_index<D>(lane, jj)) * D + col];
+    float hcur = hstate[seq * D + col], ccur = cstate[seq * D + col];
+
+    Tile pz[3], pk[3], pv[3];
+    float pb[3] = {0.f, 0.f, 0.f};
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *zlane[3], *klane[3], *vlane[3], *bb[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        zlane[a] = row(g.z[a], n, h, 0) + lrow * g.z[a].sL + 4 * lc4;
+        klane[a] = row(g.k[a], n, h, 0) + lrow * g.k[a].sL + 4 * lc4;
+        vlane[a] = row(g.v[a], n, h, 0) + lrow * g.v[a].sL + 4 * lc4;
+        bb[a] = row(g.beta[a], n, h, 0);
+    }
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            if (t0 + TL <= L) {
+                pz[a].template fetch<true>(zlane[a], g.z[a].sL, t0, L, lane);
+                pk[a].template fetch<true>(klane[a], g.k[a].sL, t0, L, lane);
+                pv[a].template fetch<true>(vlane[a], g.v[a].sL, t0, L, lane);
+            } else {
+                pz[a].template fetch<false>(zlane[a], g.z[a].sL, t0, L, lane);
+                pk[a].template fetch<false>(klane[a], g.k[a].sL, t0, L, lane);
+                pv[a].template fetch<false>(vlane[a], g.v[a].sL, t0, L, lane);
+            }
+            pb[a] = bb[a][(int64_t)min(t0 + per % TL, L - 1) * g.beta[a].sL];
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            pz[a].commit(sz[a][buf], lane);
+            pk[a].commit(sk[a][buf], lane);
+            pv[a].commit(sv[a][buf], lane);
+            sb[a][buf][per % TL] = pb[a];
+        }
+    };
+    auto flush = [&](int t0) {
+        const int64_t base = seq * L * D;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            if (vdiff) flush_tile<D, TL>(sout[a], vdiff + a * gate_stride + base, t0, L, lane);
+            if (gates) flush_tile<D, TL>(sout[3 + a], gates + a * gate_stride + base, t0, L, lane);
+        }
+        flush_tile<D, TL>(sout[6], out + base, t0, L, lane);
+        flush_tile<D, TL>(sout[7], cell + base, t0, L, lane);
+    };
+
+    auto load_ops = [&](LstmFwdOps<D> &o, int buf, int tt) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) o.k[a][p] = sk[a][buf][tt * D + 16 * p + per];
+            o.v[a] = sv[a][buf][tt * D + col];
+            o.z[a] = sz[a][buf][tt * D + col];
+            o.b[a] = sb[a][buf][tt];
+        }
+    };
+    auto compute = [&](const LstmFwdOps<D> &o, int tt) {
+        const float mx = across_groups<S>(hcur, OpMax());
+        const float e = __expf(hcur - mx);
+        const float s_m = __fdividef(e, across_groups<S>(e, OpSum()));
+        float s[NP];
+        to_periodic<D>(s_m, s, lane);
+        float d[3], pre[3];
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            d[a] = o.v[a] - group_sum<S>(dot_rot<D>(Wc[a], o.k[a]));
+            rank1_rot<D>(Wc[a], o.k[a], o.b[a] * d[a]);
+            pre[a] = group_sum<S>(dot_rot<D>(Wc[a], s)) + o.z[a];
+        }
+        const float gi = sigmoidf_fast(pre[0]), go = sigmoidf_fast(pre[2]);
+        ccur = fmaf(gi, pre[1] - ccur, ccur);          // i u + (1 - i) c
+        hcur = pinned(go * ccur);
+        const float val[8] = {pinned(d[0]), pinned(d[1]), pinned(d[2]), pinned(gi),
+                              pinned(pre[1]), pinned(go), hcur, pinned(ccur)};
+        // one LDS write covers S output tiles: lane s of a group writes value S*j + s
+#pragma unroll
+        for (int j = 0; j < 8 / S; j++) {
+            float x = val[S * j];
+#pragma unroll
+            for (int q = 1; q < S; q++) x = sl == q ? val[S * j + q] : x;
+            sout[S * j + sl][tt * D + col] = x;
+        }
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    fetch(0);
+    commit(0);
+    if (ntile > 1) fetch(TL);
+    LstmFwdOps<D> ring[RING];
+#pragma unroll
+    for (int p = 0; p < PF; p++) load_ops(ring[p], 0, p);
+
+    for (int it = 0; it < ntile; it++) {
+        const int buf = it & 1, t0 = it * TL;
+        const int nst = min(TL, L - t0);
+        if (it + 1 < ntile) commit(buf ^ 1);
+        if (it > 0) flush(t0 - TL);
+        if (it + 2 < ntile) fetch(t0 + 2 * TL);
+        if (nst == TL) {
+#pragma unroll
+            for (int tt = 0; tt < TL; tt++) {
+                const int nt = tt + PF;
+                if (nt < TL) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[nt % RING], buf ^ 1, nt - TL);
+                compute(ring[tt % RING], tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                LstmFwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt);
+            }
+        }
+        const int t_end = t0 + nst;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+#pragma unroll
+            for (int a = 0; a < 3; a++) {
+                float *c = ckpt + a * ckpt_stride + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+                for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[a][jj];
+            }
+        }
+    }
+    flush((ntile - 1) * TL);
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++)
+            g.W[a][(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[a][jj];
+    if (sl == 0) {
+        hstate[seq * D + col] = hcur;
+        cstate[seq * D + col] = ccur;
+    }
+}
+
+// ----------------------------------------------------------------- backward
+
+template <int D>
+struct LstmBwdOps {
+    float k[3][Geo<D>::NP], u[3][Geo<D>::NP], k_i[3], d_i[3], b[3];
+    float s[Geo<D>::NP], s_i, go_i, po, pa, pb, pi;
+};
+
+template <int D, int RING, int PF, int WPB>
+__global__ __launch_bounds__(kWave * WPB) void k_lstm_bwd_reg(
+    LstmGates g, const float *__restrict__ vdiff, const float *__restrict__ gates,
+    const float *__restrict__ out, const float *__restrict__ cell, const float *__restrict__ h_init,
+    const float *__restrict__ c_init, fwp_view go, const float *__restrict__ ckpt,
+    float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv, float *__restrict__ gbeta,
+    int N, int H, int L, int chunk, int nchunk, int nseq) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    using Tile = TileRegs<D, TL>;
+    static_assert(TL % RING == 0 && PF < RING, "ring must divide the tile");
+    __shared__ __align__(16) float sk_[WPB][3][2][TL * D];
+    __shared__ __align__(16) float sd_[WPB][3][2][TL * D];
+    __shared__ __align__(16) float sb_[WPB][3][2][16];
+    __shared__ __align__(16) float sgo_[WPB][2][TL * D];
+    __shared__ __align__(16) float ss_[WPB][2][TL * D];        // softmax of the delayed output
+    __shared__ __align__(16) float sco_[WPB][4][2][TL * D];    // o, c o (1-o), (u - c_prev) i (1-i), i
+    __shared__ __align__(16) float spd_[WPB][3][TL * D];
+    __shared__ __align__(16) float sgrad_[WPB][9][TL * D + 16];   // staged gz, gk, gv of the three gates
+
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
+    if (seq >= nseq) return;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    auto &sk = sk_[wave];
+    auto &sd = sd_[wave];
+    auto &sb = sb_[wave];
+    auto &sgo = sgo_[wave];
+    auto &ss = ss_[wave];
+    auto &sco = sco_[wave];
+    auto &spd = spd_[wave];
+    auto &sgrad = sgrad_[wave];
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t beta_stride = (int64_t)N * H * L;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+    const int64_t base = seq * L * D;
+
+    // per gate: Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
+    float Wr[3][R], Gr[3][R], Gc[3][R];
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Gr[a][jj] = Gc[a][jj] = Wr[a][jj] = 0.f;
+    float dh_i = 0.f, dc_i = 0.f;   // gradients carried to the previous output and cell, entry i
+
+    Tile pk[3], pd[3], pgo, ps, pco[4];
+    float pb[3] = {0.f, 0.f, 0.f};
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane[3], *bb[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        klane[a] = row(g.k[a], n, h, 0) + lrow * g.k[a].sL + 4 * lc4;
+        bb[a] = row(g.beta[a], n, h, 0);
+    }
+    const float *golane = row(go, n, h, 0) + lrow * go.sL + 4 * lc4;
+    const int64_t lane_off = (int64_t)lrow * D + 4 * lc4;     // into the contiguous saved tensors
+    auto fetch = [&](int t0) {
+        const bool full = t0 + TL <= L;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float *dl = vdiff + a * gate_stride + base + lane_off;
+            if (full) {
+                pk[a].template fetch<true>(klane[a], g.k[a].sL, t0, L, lane);
+                pd[a].template fetch<true>(dl, D, t0, L, lane);
+            } else {
+                pk[a].template fetch<false>(klane[a], g.k[a].sL, t0, L, lane);
+                pd[a].template fetch<false>(dl, D, t0, L, lane);
+            }
+            pb[a] = bb[a][(int64_t)min(t0 + per % TL, L - 1) * g.beta[a].sL];
+        }
+        if (full) pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+        else pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+        // gates, cell, delayed cell and delayed output of the tile's rows -> coefficients
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            const int t = t0 + lrow + Tile::kRowsPerLoad * x;
+            const int64_t r = (int64_t)min(t, L - 1) * D + 4 * lc4;
+            const float4 gi = *reinterpret_cast<const float4 *>(gates + base + r);
+            const float4 gu = *reinterpret_cast<const float4 *>(gates + gate_stride + base + r);
+            const float4 go_ = *reinterpret_cast<const float4 *>(gates + 2 * gate_stride + base + r);
+            const float4 ct = *reinterpret_cast<const float4 *>(cell + base + r);
+            // row t of a delayed tensor is row t-1, or the initial state for t = 0
+            const int64_t rp = (int64_t)(min(t, L) - 1) * D + 4 * lc4;
+            const float4 cp = *reinterpret_cast<const float4 *>(t == 0 ? c_init + seq * D + 4 * lc4
+                                                                       : cell + base + rp);
+            ps.r[x] = *reinterpret_cast<const float4 *>(t == 0 ? h_init + seq * D + 4 * lc4
+                                                                : out + base + rp);
+            pco[0].r[x] = go_;
+            pco[1].r[x] = make_float4(ct.x * go_.x * (1.f - go_.x), ct.y * go_.y * (1.f - go_.y),
+                                      ct.z * go_.z * (1.f - go_.z), ct.w * go_.w * (1.f - go_.w));
+            pco[2].r[x] = make_float4((gu.x - cp.x) * gi.x * (1.f - gi.x), (gu.y - cp.y) * gi.y * (1.f - gi.y),
+                                      (gu.z - cp.z) * gi.z * (1.f - gi.z), (gu.w - cp.w) * gi.w * (1.f - gi.w));
+            pco[3].r[x] = gi;
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            pk[a].commit(sk[a][buf], lane);
+            pd[a].commit(sd[a][buf], lane);
+            sb[a][buf][per % TL] = pb[a];
+        }
+        pgo.commit(sgo[buf], lane);
+#pragma unroll
+        for (int x = 0; x < 4; x++) pco[x].commit(sco[x][buf], lane);
+        // softmax of each row of the delayed output, off the sequential path
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            float4 &r = ps.r[x];
+            const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
+            r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
+            const float inv = 1.f / row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum());
+            r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
+        }
+        ps.commit(ss[buf], lane);
+    };
+    // The states are re-anchored once per chunk, straight from the checkpoint (no prefetch: the
+    // registers a prefetch would hold are the difference between fitting and spilling at D = 32).
+    auto load_state = [&](int c) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float *src = ckpt + a * ckpt_stride + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[a][jj] = src[reg_index<D>(lane, jj)];
+        }
+    };
+
+    auto load_ops = [&](LstmBwdOps<D> &o, int buf, int tt) {
+        const int off = tt * D;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            o.b[a] = sb[a][buf][tt];
+#pragma unroll
+            for (int p = 0; p < NP; p++) {
+                o.k[a][p] = sk[a][buf][off + 16 * p + per];
+                o.u[a][p] = o.b[a] * sd[a][buf][off + 16 * p + per];     // u = beta d
+            }
+            o.k_i[a] = sk[a][buf][off + i];
+            o.d_i[a] = sd[a][buf][off + i];
+        }
+#pragma unroll
+        for (int p = 0; p < NP; p++) o.s[p] = ss[buf][off + 16 * p + per];
+        o.s_i = ss[buf][off + i];
+        o.go_i = sgo[buf][off + i];
+        o.po = sco[0][buf][off + i];
+        o.pa = sco[1][buf][off + i];
+        o.pb = sco[2][buf][off + i];
+        o.pi = sco[3][buf][off + i];
+    };
+    auto compute = [&](const LstmBwdOps<D> &o, int tt) {
+        // cell: h = o c, c = i u + (1 - i) c_prev
+        const float gh = dh_i + o.go_i;
+        const float gc = fmaf(gh, o.po, dc_i);
+        const float ga[3] = {gc * o.pb, gc * o.pi, gh * o.pa};     // gradients of the pre-activations = grad_z
+        dc_i = gc * (1.f - o.pi);
+        float ds_part = 0.f;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            float gp[NP], ap[NP];
+            to_periodic<D>(ga[a], gp, lane);
+            // G' = G + s (x) ga (both layouts);  r = G'^T k
+            rank1_rot<D>(Gc[a], o.s, ga[a]);
+            const float r_i = group_sum<S>(dot_rot<D>(Gc[a], o.k[a]));
+            const float gv_i = o.b[a] * r_i;
+            const float a_i = -gv_i;                               // gradient w.r.t. v_old
+            to_periodic<D>(a_i, ap, lane);
+            spd[a][tt * D + i] = r_i * o.d_i[a];
+            rank1_rot<D>(Gr[a], gp, o.s_i);
+            ds_part = dot_rot<D>(Wr[a], gp, ds_part);              // (W_t ga)[i], summed over the gates
+            rank1_rot<D, true>(Wr[a], o.u[a], o.k_i[a]);           // W_{t-1}
+            rank1_rot<D>(Gc[a], o.k[a], a_i);
+            float gk_i = dot_rot<D>(Gr[a], o.u[a]);                // G' u + W_{t-1} a
+            gk_i = group_sum<S>(dot_rot<D>(Wr[a], ap, gk_i));
+            rank1_rot<D>(Gr[a], ap, o.k_i[a]);
+            // staged gz, gk, gv of this gate; lanes of a group pick their tile by s
+            const float o_z = pinned(ga[a]), o_k = pinned(gk_i), o_v = pinned(gv_i);
+            if constexpr (S == 4) {
+                sgrad[sl == 0 ? a : (sl == 1 ? 3 + a : 6 + a)][tt * D + i] = sl == 0 ? o_z : (sl == 1 ? o_k : o_v);
+            } else {
+                sgrad[sl == 0 ? a : 3 + a][tt * D + i] = sl == 0 ? o_z : o_k;
+                sgrad[6 + a][tt * D + i] = o_v;
+            }
+        }
+        // gradient of s = softmax(h_{t-1}) back to h_{t-1}
+        const float ds_i = group_sum<S>(ds_part);
+        const float dot = across_groups<S>(ds_i * o.s_i, OpSum());
+        dh_i = o.s_i * (ds_i - dot);
+    };
+    auto flush = [&](int t0, int nst) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            flush_tile<D, TL>(sgrad[a], gz + a * gate_stride + base, t0, L, lane);
+            flush_tile<D, TL>(sgrad[3 + a], gk + a * gate_stride + base, t0, L, lane);
+            flush_tile<D, TL>(sgrad[6 + a], gv + a * gate_stride + base, t0, L, lane);
+        }
+        // gbeta of the tile's steps: sums of spd[a][tt][:] over the D entries, four lanes per step
+        const int tt = lane / 4, part = lane % 4;
+        if (tt < TL) {
+#pragma unroll
+            for (int a = 0; a < 3; a++) {
+                float acc = 0.f;
+#pragma unroll
+                for (int j = 0; j < D / 4; j += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(&spd[a][tt * D + part * (D / 4) + j]);
+                    acc += (x.x + x.y) + (x.z + x.w);
+                }
+                acc = group_sum<4>(acc);
+                if (tt < nst) gbeta[a * beta_stride + seq * L + t0 + tt] = acc;
+            }
+        }
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    fetch((ntile - 1) * TL);
+    commit((ntile - 1) & 1);
+    if (ntile > 1) fetch((ntile - 2) * TL);
+    LstmBwdOps<D> ring[RING];
+    bool primed = false;
+
+    for (int it = ntile - 1; it >= 0; it--) {
+        const int buf = it & 1, t0 = it * TL;
+        const int nst = min(TL, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) load_state((t_end - 1) / chunk);  // first tile (in reverse) of a chunk
+        if (it >= 1) commit(buf ^ 1);
+        if (it + 1 < ntile) flush(t0 + TL, min(TL, L - t0 - TL));
+        if (it >= 2) fetch(t0 - 2 * TL);
+        if (nst == TL) {
+            if (!primed) {
+#pragma unroll
+                for (int p = 0; p < PF; p++) load_ops(ring[(TL - 1 - p) % RING], buf, TL - 1 - p);
+                primed = true;
+            }
+#pragma unroll
+            for (int tt = TL - 1; tt >= 0; tt--) {
+                const int nt = tt - PF;
+                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
+                else load_ops(ring[(nt + TL) % RING], buf ^ 1, nt + TL);
+                compute(ring[tt % RING], tt);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                LstmBwdOps<D> o;
+                load_ops(o, buf, tt);
+                compute(o, tt);
+            }
+        }
+    }
+    flush(0, min(TL, L));
+}
+
+}  // namespace
+
+bool reg_lstm_supported(int D) { return D == 16 || D == 32; }
+
+int reg_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, float *gates,
+                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_lstm_fwd_reg<16, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, g,
+                           h, c, out, cell, gates, vdiff, ckpt, N, H, L, chunk, nchunk, nseq);
+    else
+        hipLaunchKernelGGL((k_lstm_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, g,
+                           h, c, out, cell, gates, vdiff, ckpt, N, H, L, chunk, nchunk, nseq);
+    return (int)hipGetLastError();
+}
+
+int reg_lstm_bwd(const LstmGates &g, const float *vdiff, const float *gates, const float *out,
+                 const float *cell, const float *h_init, const float *c_init, fwp_view go,
+                 const float *ckpt, float *gz, float *gk, float *gv, float *gbeta, int N, int H, int L,
+                 int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (D == 16)
+        hipLaunchKernelGGL((k_lstm_bwd_reg<16, 2, 1, 1>), dim3(nseq), dim3(kWave), 0, s, g, vdiff, gates,
+                           out, cell, h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, chunk, nchunk,
+                           nseq);
+    else
+        hipLaunchKernelGGL((k_lstm_bwd_reg<32, 2, 1, 1>), dim3(nseq), dim3(kWave), 0, s, g, vdiff, gates,
+                           out, cell, h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, chunk, nchunk,
+                           nseq);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fwp
