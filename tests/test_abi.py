@@ -49,6 +49,30 @@ def test_bad_arguments_are_rejected_without_a_device(fwp):
     assert lib.fwp_rnn_fwd(v, v, v, v, p, None, p, p, p, 1, 1, 4, 16, 64, None) == -1
 
 
+def test_ckpt_size_and_config_entry_points(fwp):
+    L = fwp._lib
+    lib = L.lib()
+    chunk = L.query(L.Q_DEFAULT_CHUNK)
+    # states only when the blocked kernels do not apply, states + header + one 16x16 matrix per 16 steps otherwise
+    assert L.delta_ckpt_floats(2, 3, 100, 24, 8, chunk) == 2 * 3 * 2 * 24 * 8
+    n16 = L.delta_ckpt_floats(2, 3, 100, 16, 16, chunk)
+    assert n16 > 2 * 3 * 2 * 256 and (n16 - 2 * 3 * 2 * 256 - 2 * 3 * 7 * 256) in range(0, 65)
+    assert lib.fwp_delta_ckpt_floats(0, 3, 100, 16, 16, chunk) == -1
+    with pytest.raises(L.FwpError):
+        L.delta_ckpt_floats(1, 1, 8, 16, 16, chunk + 1)
+    for value in (L.DELTA_SCAN, L.DELTA_CHUNKED, L.DELTA_AUTO):
+        L.config(L.CFG_DELTA_KERNELS, value)
+    assert lib.fwp_config(L.CFG_DELTA_KERNELS, 7) != 0 and lib.fwp_config(99, 0) != 0
+    # Delta LSTM and sum rule: NULL checks come before any launch
+    null3 = (L.View * 3)()
+    assert lib.fwp_lstm_fwd(null3, null3, null3, null3, None, None, None, None, None, None, None, None,
+                            1, 1, 4, 16, chunk, None) == -1
+    v = L.View(4096, 64, 32, 16)
+    p = ctypes.c_void_p(4096)
+    assert lib.fwp_sum_fwd(v, v, v, None, p, p, 1, 1, 4, 16, 16, chunk, None) == -1
+    assert lib.fwp_sum_bwd(v, v, v, v, p, None, p, p, p, 1, 1, 4, 16, 16, 24, None) == -3
+
+
 def test_operators_refuse_cpu_tensors(fwp):
     import torch
     q = torch.zeros(1, 1, 2, 4)

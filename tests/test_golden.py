@@ -42,6 +42,24 @@ def test_oracle_reproduces_rnn_and_rec_fixtures():
         assert max_abs(a, g["g" + n]) < 1e-10
 
 
+def test_oracle_reproduces_sum_and_lstm_fixtures():
+    g = load("sum_b3h5t7e11m4.npz")
+    out, W = oracle.sum_fwd(*d(g["q"], g["k"], g["v"], g["W0"]))
+    assert max_abs(out, g["out"]) < 1e-12 and max_abs(W, g["W"]) < 1e-12
+    gq, gk, gv = oracle.sum_bwd(*d(g["q"], g["k"], g["v"], g["W0"], g["go"]))
+    assert max(max_abs(gq, g["gq"]), max_abs(gk, g["gk"]), max_abs(gv, g["gv"])) < 1e-12
+    assert max_abs(oracle.sum_bwd(*d(g["q"], g["k"], g["v"], g["W0"], g["go"]), through_state=True)[0],
+                   g["gq_exact"]) < 1e-12
+    g = load("lstm_b1h2t24d16.npz")
+    gates = [list(d(*g[n])) for n in ("Z", "K", "V", "B", "W0")]
+    out, cell, Wn, h, c = oracle.lstm_fwd(*gates, *d(g["h0"], g["c0"]))
+    assert max_abs(out, g["out"]) < 1e-12 and max_abs(cell, g["cell"]) < 1e-12
+    assert max_abs(np.stack(Wn), g["W"]) < 1e-12 and max_abs(h, g["h"]) < 1e-12 and max_abs(c, g["c"]) < 1e-12
+    grads = oracle.lstm_bwd(*gates, *d(g["h0"], g["c0"], g["go"]))
+    for got, n in zip(grads, ("gZ", "gK", "gV", "gB")):
+        assert max_abs(np.stack(got), g[n]) < 1e-10
+
+
 def test_float32_oracle_is_inside_the_parity_budget_on_the_fixtures():
     g = load("delta_b2h2t64d16.npz")
     out, _ = oracle.delta_fwd(g["q"], g["k"], g["v"], g["beta"], g["W0"])
@@ -98,3 +116,42 @@ def test_hip_rec_matches_fixture(fwp):
     _check("h", h, g["h"])
     for t, n in zip(ts, names):
         _check("g" + n, t.grad, g["g" + n])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode,key", [("reference", "gq"), ("exact", "gq_exact")])
+def test_hip_sum_matches_fixture(fwp, mode, key):
+    g = load("sum_b3h5t7e11m4.npz")
+    ts = [_dev(g[n], True) for n in ("q", "k", "v")]
+    W = _dev(g["W0"])
+    fwp.FastWeightSum.state_gradient = mode
+    try:
+        out = fwp.fast_weight_sum(*ts, W)
+        out.backward(_dev(g["go"]))
+    finally:
+        fwp.FastWeightSum.state_gradient = "reference"
+    _check("out", out, g["out"])
+    _check("W", W, g["W"])
+    for t, n in zip(ts, (key, "gk", "gv")):
+        _check(n, t.grad, g[n])
+
+
+@pytest.mark.gpu
+def test_hip_lstm_matches_fixture(fwp):
+    g = load("lstm_b1h2t24d16.npz")
+    diff = [[_dev(g[n][a], True) for n in ("Z", "K", "V", "B")] for a in range(3)]
+    Ws = [_dev(g["W0"][a]) for a in range(3)]
+    h, c = _dev(g["h0"]), _dev(g["c0"])
+    args = []
+    for a in range(3):
+        args += diff[a] + [Ws[a]]
+    out, cell = fwp.fast_lstm_v4(*args, h, c)
+    out.backward(_dev(g["go"]))
+    _check("out", out, g["out"])
+    _check("cell", cell, g["cell"])
+    _check("h", h, g["h"])
+    _check("c", c, g["c"])
+    for a in range(3):
+        _check(f"W[{a}]", Ws[a], g["W"][a])
+        for j, n in enumerate(("gZ", "gK", "gV", "gB")):
+            _check(f"{n}[{a}]", diff[a][j].grad, g[n][a])
