@@ -184,6 +184,23 @@ int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff,
                  int N, int H, int L, int D, int chunk, void *stream);
 
 /*
+ * Pre-step of the Delta-Net layer, fused.  Replaces the elementwise lines between the layer's
+ * projection and its call of the operator
+ * (language_modeling/src/utils/cuda_fast_weight_layer.py:108-125): from qkvb [T,B,H,3D+1]
+ * (contiguous; per head q | k | v | beta logit) to the operator's inputs, contiguous [B,H,T,.]:
+ *   q, k = (elu(x) + 1) / sum_D(elu(x) + 1)    v = copy    beta = sigmoid(logit)
+ * D must be 16, 32 or 64 (FWP_E_SHAPE otherwise).
+ */
+int fwp_deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta,
+                          int T, int B, int H, int D, void *stream);
+
+/* Adjoint of fwp_deltanet_prep_fwd: gradients of q, k, v, beta ([B,H,T,.] contiguous) to the
+ * gradient of qkvb [T,B,H,3D+1] (every element written). */
+int fwp_deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
+                          const float *gbeta, float *gqkvb, int T, int B, int H, int D,
+                          void *stream);
+
+/*
  * Recurrent Delta Net forward.  Replaces rec_update_fwm_tanh_forward
  * (algorithmic/rec_update_fwm_tanh/rec_update_fwm_tanh.cu:349-444, kernel :25-345).
  *   qx,kx,vx [N,H,L,D] and bx [N,H,L,1] are pre-activation

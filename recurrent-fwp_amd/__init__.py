@@ -11,10 +11,10 @@ from .fast_transformers import FastWeightSum, fast_weight_sum
 from .fast_lstm_v4 import FastLSTMv4, fast_lstm_v4
 from .fast_weight_rnn_v2 import FastRNNv2, fast_rnn_v2
 from .rec_update_fwm_tanh import FastWeightRecUpdateTanh, rec_update_fwm_tanh
-from .layers import DeltaNetDecoderLayer, DeltaNetLayer, PositionalEmbedding, PositionwiseFF
+from .layers import DeltaNetDecoderLayer, DeltaNetLayer, DeltaNetPrep, PositionalEmbedding, PositionwiseFF
 from .lm import DeltaNetLM
 
 __all__ = ["DeltaFastWeight", "fast_weight_delta", "FastWeightSum", "fast_weight_sum", "FastRNNv2", "fast_rnn_v2",
            "FastLSTMv4", "fast_lstm_v4",
-           "FastWeightRecUpdateTanh", "rec_update_fwm_tanh", "DeltaNetLayer",
+           "FastWeightRecUpdateTanh", "rec_update_fwm_tanh", "DeltaNetLayer", "DeltaNetPrep",
            "DeltaNetDecoderLayer", "PositionwiseFF", "PositionalEmbedding", "DeltaNetLM"]

@@ -35,6 +35,8 @@ _SIGNATURES = {
     "fwp_rnn_bwd": [_V, _V, _P, _P, _P, _V, _P] + [_P] * 4 + [_I] * 5 + [_P],
     "fwp_lstm_fwd": [_VP] * 4 + [_P] * 8 + [_I] * 5 + [_P],
     "fwp_lstm_bwd": [_VP] * 2 + [_P] * 6 + [_V] + [_P] * 5 + [_I] * 5 + [_P],
+    "fwp_deltanet_prep_fwd": [_P] * 5 + [_I] * 4 + [_P],
+    "fwp_deltanet_prep_bwd": [_P] * 6 + [_I] * 4 + [_P],
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
 }

@@ -224,6 +224,20 @@ int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff, co
                             gbeta, N, H, L, D, chunk, (hipStream_t)stream);
 }
 
+int fwp_deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B,
+                          int H, int D, void *stream) {
+    if (!qkvb || !q || !k || !v || !beta) return FWP_E_NULL;
+    if (T < 1 || B < 1 || H < 1 || !prep_supported(D)) return FWP_E_SHAPE;
+    return deltanet_prep_fwd(qkvb, q, k, v, beta, T, B, H, D, (hipStream_t)stream);
+}
+
+int fwp_deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
+                          const float *gbeta, float *gqkvb, int T, int B, int H, int D, void *stream) {
+    if (!qkvb || !gq || !gk || !gv || !gbeta || !gqkvb) return FWP_E_NULL;
+    if (T < 1 || B < 1 || H < 1 || !prep_supported(D)) return FWP_E_SHAPE;
+    return deltanet_prep_bwd(qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, D, (hipStream_t)stream);
+}
+
 int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,
                 const float *Rk, const float *Rv, const float *rb, float *W, float *h, float *out,
                 float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,

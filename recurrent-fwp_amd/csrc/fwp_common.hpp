@@ -115,6 +115,13 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
                 float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
                 int chunk, hipStream_t s);
 
+// Fused pre-step of the Delta-Net layer and its adjoint (D in {16, 32, 64}).
+bool prep_supported(int D);
+int deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B, int H,
+                      int D, hipStream_t s);
+int deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
+                      const float *gbeta, float *gqkvb, int T, int B, int H, int D, hipStream_t s);
+
 // Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
 constexpr size_t kMaxLds = 160 * 1024 - 1024;
 

@@ -1,14 +1,16 @@
 """The caller of ``fast_weight_delta`` in language modelling: the Delta-Net layer and the
 feed-forward block that follows it, with the module and parameter names of the reference
 (language_modeling/src/utils/cuda_fast_weight_layer.py:57-188, utils/model_utils.py:15-67)
-so a reference state_dict loads unchanged.  Everything except the fast-weight operator is
-stock PyTorch; the operator is the HIP one unless a caller passes another (tests do, to
-compare against a step-by-step loop).
+so a reference state_dict loads unchanged.  The fast-weight operator and, on the GPU, the
+elementwise lines in front of it are HIP kernels; the rest is stock PyTorch.  A caller may pass
+another operator (tests do, to compare against a step-by-step loop); the layer then also takes
+the stock-PyTorch form of those lines.
 """
 import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import _lib
 from .fast_weight import fast_weight_delta
 
 
@@ -52,6 +54,48 @@ def sum_normalised_elu(x):
     return x / x.sum(-1, keepdim=True)
 
 
+class DeltaNetPrep(torch.autograd.Function):
+    """``q, k, v, beta = DeltaNetPrep.apply(qkvb, n_head, d_head)``: the lines between the layer's
+    projection and the operator (cuda_fast_weight_layer.py:108-125) as one HIP kernel each way.
+    ``qkvb`` is the contiguous ``[len, bsz, n_head * (3 d_head + 1)]`` projection; the results are
+    contiguous ``[bsz, n_head, len, .]``: q, k through :func:`sum_normalised_elu`, v copied, beta
+    through a sigmoid."""
+
+    @staticmethod
+    def supported(qkvb, d_head):
+        return (qkvb.is_cuda and qkvb.dtype == torch.float32 and qkvb.is_contiguous()
+                and d_head in (16, 32, 64))
+
+    @staticmethod
+    def forward(ctx, qkvb, n_head, d_head):
+        _lib.require_device(qkvb)
+        T, B, _ = qkvb.shape
+        H, D = n_head, d_head
+        f32 = dict(device=qkvb.device, dtype=torch.float32)
+        q, k, v = (torch.empty((B, H, T, D), **f32) for _ in range(3))
+        beta = torch.empty((B, H, T, 1), **f32)
+        with _lib.on_device(qkvb):
+            rc = _lib.lib().fwp_deltanet_prep_fwd(qkvb.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                                  beta.data_ptr(), T, B, H, D, _lib.stream_of(qkvb))
+        _lib.check(rc, "fwp_deltanet_prep_fwd")
+        ctx.save_for_backward(qkvb)
+        ctx.dims = (T, B, H, D)
+        return q, k, v, beta
+
+    @staticmethod
+    def backward(ctx, gq, gk, gv, gbeta):
+        (qkvb,) = ctx.saved_tensors
+        T, B, H, D = ctx.dims
+        gq, gk, gv, gbeta = (g.contiguous() for g in (gq, gk, gv, gbeta))
+        gqkvb = torch.empty_like(qkvb)
+        with _lib.on_device(qkvb):
+            rc = _lib.lib().fwp_deltanet_prep_bwd(qkvb.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
+                                                  gbeta.data_ptr(), gqkvb.data_ptr(), T, B, H, D,
+                                                  _lib.stream_of(qkvb))
+        _lib.check(rc, "fwp_deltanet_prep_bwd")
+        return gqkvb, None, None
+
+
 class DeltaNetLayer(nn.Module):
     """Delta-rule linear-Transformer layer (the reference's
     ``CudaFastWeightLinearTransformerLayer`` with its default
@@ -87,9 +131,13 @@ class DeltaNetLayer(nn.Module):
         # The reference's pre-LN branch adds the normalised input back (it rebinds h, :100-104).
         residual = x
 
-        qkvb = self.qkvb_net(x).view(slen, bsz, H, 3 * D + 1)
-        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in qkvb.split((D, D, D, 1), dim=-1))
-        q, k, beta = sum_normalised_elu(q), sum_normalised_elu(k), torch.sigmoid(beta)
+        qkvb = self.qkvb_net(x)
+        if self.fast_weight_op is fast_weight_delta and DeltaNetPrep.supported(qkvb, D):
+            q, k, v, beta = DeltaNetPrep.apply(qkvb, H, D)       # one fused kernel each way
+        else:
+            qkvb = qkvb.view(slen, bsz, H, 3 * D + 1)
+            q, k, v, beta = (t.permute(1, 2, 0, 3) for t in qkvb.split((D, D, D, 1), dim=-1))
+            q, k, beta = sum_normalised_elu(q), sum_normalised_elu(k), torch.sigmoid(beta)
 
         if mems is None:
             W = torch.zeros(bsz, H, D, D, device=h.device, dtype=h.dtype)
