@@ -126,8 +126,11 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
     if (bad_view(q) || bad_view(k) || bad_view(v) || !W || !out) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
-        aligned16(ckpt) && aligned16(out))
+        aligned16(ckpt) && aligned16(out)) {
+        if (g_delta_kernels == FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32))
+            return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
         return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+    }
     return generic_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
 }
 
@@ -139,9 +142,13 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
-        aligned16(gk) && aligned16(gv))
+        aligned16(gk) && aligned16(gv)) {
+        if (g_delta_kernels == FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32))
+            return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
+                                (hipStream_t)stream);
         return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
                            (hipStream_t)stream);
+    }
     return generic_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
                            (hipStream_t)stream);
 }

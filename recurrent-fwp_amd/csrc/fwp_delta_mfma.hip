@@ -643,6 +643,224 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
     else flush(std::true_type(), 0);
 }
 
+// ------------------------------------------------------------------ sum rule
+//
+// The same blocks without the triangular system: O = Q S + lower(Q K^T) V, S' = S + K^T V, and in
+// reverse g_v = K dS + lower(Q K^T)^T dO, g_q = dO S0^T + lower(dO V^T) K,
+// g_k = V dS^T + lower(dO V^T)^T Q, dS += Q^T dO.
+
+// Loads of one 16-step block of a [.., L, D] tensor in both orientations.  Rows beyond L: clamped
+// loads, zeroed if `zero_tail`.
+template <int NB>
+struct BothWays {
+    v4f t[NB], c[NB];   // t: register r = X[t0 + c][16b + 4g + r];  c: register r = X[t0 + 4g + r][16b + c]
+    __device__ __forceinline__ void load(const float *base, int64_t sL, int t0, int L, const Geo16 &p,
+                                         bool zero_tail) {
+        const int64_t tc = min(t0 + p.c, L - 1);
+        const bool col_ok = !zero_tail || t0 + p.c < L;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            const float4 x = *reinterpret_cast<const float4 *>(base + tc * sL + 16 * b + 4 * p.g);
+            t[b] = col_ok ? v4f{x.x, x.y, x.z, x.w} : v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t tr = min(t0 + 4 * p.g + r, L - 1);
+                const float y = base[tr * sL + 16 * b + p.c];
+                c[b][r] = (!zero_tail || t0 + 4 * p.g + r < L) ? y : 0.f;
+            }
+        }
+    }
+};
+
+template <int NB>
+__global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
+                                                     float *__restrict__ W, float *__restrict__ out,
+                                                     float *__restrict__ ckpt, int H, int L, int chunk,
+                                                     int nchunk) {
+    constexpr int D = 16 * NB;
+    const Geo16 p(threadIdx.x);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0);
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f S[NB][NB];
+#pragma unroll
+    for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                S[eb][mb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+
+    struct Raw { BothWays<NB> K, Q, V; };
+    auto load = [&](Raw &w, int t0) {
+        w.K.load(kb, k.sL, t0, L, p, true);       // zero rows beyond L: they then write nothing
+        w.Q.load(qb, q.sL, t0, L, p, false);
+        w.V.load(vb, v.sL, t0, L, p, false);
+    };
+    const int nblk = (L + kBlk - 1) / kBlk;
+    Raw cur, nxt;
+    load(cur, 0);
+    for (int ib = 0; ib < nblk; ib++) {
+        const int t0 = ib * kBlk;
+        load(nxt, min(ib + 1, nblk - 1) * kBlk);
+        __builtin_amdgcn_sched_barrier(0);
+        v4f R = zero;
+#pragma unroll
+        for (int b = 0; b < NB; b++) R = tn(cur.K.t[b], cur.Q.t[b], R);      // K Q^T [s][t]
+#pragma unroll
+        for (int r = 0; r < 4; r++) R[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;   // lower(Q K^T)^T
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            v4f Ot = tn(cur.V.c[mb], R, zero);
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) Ot = tn(S[eb][mb], cur.Q.t[eb], Ot);
+            if (t0 + c < L)
+                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                    make_float4(Ot[0], Ot[1], Ot[2], Ot[3]);
+        }
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) S[eb][mb] = tn(cur.K.c[eb], cur.V.c[mb], S[eb][mb]);
+        const int t_end = min(t0 + kBlk, L);
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+                for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+        }
+        cur = nxt;
+    }
+#pragma unroll
+    for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++)
+                W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+}
+
+template <int NB>
+__global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp_view v, fwp_view go,
+                                                     const float *__restrict__ ckpt,
+                                                     const float *__restrict__ W_init,
+                                                     float *__restrict__ gq, float *__restrict__ gk,
+                                                     float *__restrict__ gv, int H, int L, int chunk,
+                                                     int nchunk) {
+    constexpr int D = 16 * NB;
+    const Geo16 p(threadIdx.x);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
+                *gob = row(go, n, h, 0);
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f ident;
+#pragma unroll
+    for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+
+    struct Raw { BothWays<NB> K, Q, V, O; v4f Sck[NB][NB]; };
+    auto load = [&](Raw &w, int t0) {
+        const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * D * D;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) {     // block (mb, eb) of S^T, minus the carried-in state if asked
+                const int64_t o = (16 * eb + c) * D + 16 * mb + 4 * g;
+                float4 x = *reinterpret_cast<const float4 *>(src + o);
+                if (W_init) {
+                    const float4 y = *reinterpret_cast<const float4 *>(W_init + seq * D * D + o);
+                    x = make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w);
+                }
+                w.Sck[mb][eb] = v4f{x.x, x.y, x.z, x.w};
+            }
+        w.K.load(kb, k.sL, t0, L, p, false);
+        w.Q.load(qb, q.sL, t0, L, p, false);
+        w.V.load(vb, v.sL, t0, L, p, true);       // rows beyond L wrote nothing
+        w.O.load(gob, go.sL, t0, L, p, true);     // and carry no gradient
+    };
+
+    v4f St[NB][NB], dS[NB][NB];
+#pragma unroll
+    for (int a = 0; a < NB; a++)
+#pragma unroll
+        for (int b = 0; b < NB; b++) dS[a][b] = zero;
+
+    const int nblk = (L + kBlk - 1) / kBlk;
+    Raw cur, nxt;
+    load(cur, (nblk - 1) * kBlk);
+    for (int ib = nblk - 1; ib >= 0; ib--) {
+        const int t0 = ib * kBlk;
+        load(nxt, max(ib - 1, 0) * kBlk);
+        __builtin_amdgcn_sched_barrier(0);
+        const int t_end = min(t0 + kBlk, L);
+        if (t_end % chunk == 0 || t_end == L) {
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++)
+#pragma unroll
+                for (int eb = 0; eb < NB; eb++) St[mb][eb] = cur.Sck[mb][eb];
+        }
+        // state before the block, transposed: S0^T = S'^T - V^T K
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            const v4f nV = -cur.V.c[mb];
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) St[mb][eb] = tn(nV, cur.K.c[eb], St[mb][eb]);
+        }
+        v4f QK = zero, Z = zero, Zt = zero;
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            QK = tn(cur.Q.t[b], cur.K.t[b], QK);          // Q K^T   [t][s]
+            Z = tn(cur.O.t[b], cur.V.t[b], Z);            // dO V^T  [t][s]
+            Zt = tn(cur.V.t[b], cur.O.t[b], Zt);
+        }
+        v4f Pm, dPm, dPmt;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const bool low = p.lo[r] || p.di[r], upp = p.up[r] || p.di[r];
+            Pm[r] = low ? QK[r] : 0.f;
+            dPm[r] = low ? Z[r] : 0.f;
+            dPmt[r] = upp ? Zt[r] : 0.f;
+        }
+        const bool col_ok = t0 + c < L;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {        // g_v^T = dS^T K^T + dO^T Pm
+            v4f gVt = tn(cur.O.c[mb], Pm, zero);
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) gVt = tn(dS[eb][mb], cur.K.t[eb], gVt);
+            if (col_ok)
+                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                    make_float4(gVt[0], gVt[1], gVt[2], gVt[3]);
+        }
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) {
+            v4f gQt = tn(cur.K.c[eb], dPmt, zero);
+            v4f gKt = tn(cur.Q.c[eb], dPm, zero);
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) {
+                gQt = tn(St[mb][eb], cur.O.t[mb], gQt);
+                gKt = tn(tn(dS[eb][mb], ident, zero), cur.V.t[mb], gKt);      // dS V^T
+            }
+            if (col_ok) {
+                const int64_t o = (seq * L + t0 + c) * D + 16 * eb + 4 * g;
+                *reinterpret_cast<float4 *>(gq + o) = make_float4(gQt[0], gQt[1], gQt[2], gQt[3]);
+                *reinterpret_cast<float4 *>(gk + o) = make_float4(gKt[0], gKt[1], gKt[2], gKt[3]);
+            }
+        }
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) dS[eb][mb] = tn(cur.Q.c[eb], cur.O.c[mb], dS[eb][mb]);
+        cur = nxt;
+    }
+}
+
 }  // namespace
 
 int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk) {
@@ -694,6 +912,31 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
     else
         hipLaunchKernelGGL(k_delta_bwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, beta, vdiff, go,
                            ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+    return (int)hipGetLastError();
+}
+
+int mfma_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+                 int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    if (D == 16)
+        hipLaunchKernelGGL(k_sum_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, W, out, ckpt, H, L,
+                           chunk, nchunk);
+    else
+        hipLaunchKernelGGL(k_sum_fwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, W, out, ckpt, H, L,
+                           chunk, nchunk);
+    return (int)hipGetLastError();
+}
+
+int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+                 const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int D,
+                 int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    if (D == 16)
+        hipLaunchKernelGGL(k_sum_bwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, go, ckpt, W_init, gq,
+                           gk, gv, H, L, chunk, nchunk);
+    else
+        hipLaunchKernelGGL(k_sum_bwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, go, ckpt, W_init, gq,
+                           gk, gv, H, L, chunk, nchunk);
     return (int)hipGetLastError();
 }
 

@@ -39,16 +39,6 @@ DELTA_SHAPES = [
 ]
 
 
-@pytest.fixture(params=["scan", "chunked"])
-def delta_kernels(request, fwp):
-    """Both delta-rule forward kernels for D = 16/32: the step-by-step scan and the 16-step blocks
-    on the matrix cores (other shapes take the LDS kernels whatever the setting)."""
-    L_ = fwp._lib
-    L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED}[request.param])
-    yield request.param
-    L_.config(L_.CFG_DELTA_KERNELS, L_.DELTA_AUTO)
-
-
 @pytest.mark.parametrize("N,H,L,E,M,w0", DELTA_SHAPES)
 def test_delta(fwp, delta_kernels, N, H, L, E, M, w0):
     q, k, v, beta, W0, go = delta_inputs(100 + L + E, N, H, L, E, M, w0=w0)

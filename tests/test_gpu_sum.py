@@ -34,6 +34,8 @@ def inputs(seed, N, H, L, E, M, w0):
 
 SHAPES = [
     (3, 5, 7, 11, 4, False),      # the reference's self test
+    (2, 2, 47, 16, 16, True),     # around the 16-step block boundaries of the blocked kernels
+    (1, 2, 33, 32, 32, True),
     (2, 2, 64, 16, 16, False),
     (2, 3, 130, 16, 16, True),    # ragged tail chunk, carried-in state
     (2, 2, 256, 32, 32, True),
@@ -46,7 +48,7 @@ SHAPES = [
 
 @pytest.mark.parametrize("mode", ["reference", "exact"])
 @pytest.mark.parametrize("N,H,L,E,M,w0", SHAPES)
-def test_sum(fwp, N, H, L, E, M, w0, mode):
+def test_sum(fwp, delta_kernels, N, H, L, E, M, w0, mode):
     q, k, v, W0, go = inputs(200 + L + E, N, H, L, E, M, w0)
     tq, tk, tv = (dev(x, True) for x in (q, k, v))
     W = dev(W0)
@@ -65,7 +67,7 @@ def test_sum(fwp, N, H, L, E, M, w0, mode):
     check("W after backward", W, ref_W)
 
 
-def test_sum_strided_views_segments_and_no_grad(fwp):
+def test_sum_strided_views_segments_and_no_grad(fwp, delta_kernels):
     N, H, L, D = 2, 3, 48, 16
     q, k, v, W0, go = inputs(9, N, H, L, D, D, True)
     lnh = lambda x: dev(np.ascontiguousarray(x.transpose(2, 0, 1, 3))).permute(1, 2, 0, 3)
