@@ -58,11 +58,12 @@ int fwp_query(int what);
  * Process-wide switches (no counterpart in the reference; for measurements and tests).
  * FWP_CFG_DELTA_KERNELS selects the delta-rule kernels for E = M in {16, 32}:
  * FWP_DELTA_AUTO (default: the fastest), FWP_DELTA_SCAN (step-by-step register-state
- * kernels), FWP_DELTA_CHUNKED (16-step blocks on the matrix cores).  All give the
- * same results within the fp32 tolerance.  Returns FWP_E_SHAPE for an unknown key or value.
+ * kernels), FWP_DELTA_CHUNKED (16-step blocks on the matrix cores, one wave per sequence),
+ * FWP_DELTA_SPLIT (the same blocks, a sequence's work split over several waves; the sum rule
+ * takes the one-wave blocks).  All give the same results within the fp32 tolerance.  Returns FWP_E_SHAPE for an unknown key or value.
  */
 enum { FWP_CFG_DELTA_KERNELS = 0 };
-enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2 };
+enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2, FWP_DELTA_SPLIT = 3 };
 int fwp_config(int key, int value);
 
 /* 0 if the current HIP device is a gfx950 part, FWP_E_ARCH otherwise. */

@@ -42,7 +42,7 @@ _SIGNATURES = {
 }
 EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
                                        "fwp_delta_ckpt_floats"])
-CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED = 0, 0, 1, 2
+CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT = 0, 0, 1, 2, 3
 
 _lib = None
 _checked_devices = set()

@@ -23,12 +23,26 @@ int check_dims(int N, int H, int L, int E, int M, int chunk) {
 // fwp_config(FWP_CFG_DELTA_KERNELS, .)
 int g_delta_kernels = FWP_DELTA_AUTO;
 
+// Blocks on the matrix cores pay off from about two blocks on; single steps (stepwise inference)
+// stay on the scan kernel.
+bool delta_chunked(int L) {
+    return g_delta_kernels >= FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
+}
+
+// Several waves per sequence pay off while they find SIMDs of their own: measured on MI355X
+// (1024 SIMDs) the split kernels win up to about two waves per SIMD and lose beyond.
+bool delta_split(int N, int H, int L, int D) {
+    if (!split_delta_supported(L)) return false;
+    if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
+    return g_delta_kernels == FWP_DELTA_AUTO && L >= 32 && (int64_t)N * H * (D / 8) <= 2048;
+}
+
 }  // namespace
 
 extern "C" {
 
 int fwp_config(int key, int value) {
-    if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_CHUNKED) {
+    if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_SPLIT) {
         g_delta_kernels = value;
         return FWP_OK;
     }
@@ -83,14 +97,12 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         aligned16(vdiff) && aligned16(ckpt) && aligned16(out)) {
-        // blocks of 16 steps on the matrix cores pay off from about two blocks on; single steps
-        // (stepwise inference) stay on the scan kernel
-        const bool chunked = g_delta_kernels == FWP_DELTA_CHUNKED ||
-                             (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
-        if (chunked)
+        if (delta_split(N, H, L, E))
+            return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
+                                   (hipStream_t)stream);
+        if (delta_chunked(L))
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                                   (hipStream_t)stream);
-        if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, chunk, (hipStream_t)stream)) return rc;
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                              (hipStream_t)stream);
     }
@@ -109,9 +121,10 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
         aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv)) {
-        const bool chunked = g_delta_kernels == FWP_DELTA_CHUNKED ||
-                             (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
-        if (chunked)
+        if (delta_split(N, H, L, E))
+            return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
+                                   chunk, (hipStream_t)stream);
+        if (delta_chunked(L))
             return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
                                   chunk, (hipStream_t)stream);
         return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
@@ -127,7 +140,7 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         aligned16(ckpt) && aligned16(out)) {
-        if (g_delta_kernels == FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32))
+        if (delta_chunked(L))
             return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
         return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
     }
@@ -143,7 +156,7 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
-        if (g_delta_kernels == FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32))
+        if (delta_chunked(L))
             return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
                                 (hipStream_t)stream);
         return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,

@@ -17,52 +17,12 @@
 // and the output is produced as O^T so that it leaves with 16-byte stores.  No LDS is used.
 #include "fwp_common.hpp"
 #include "fwp_wave.hpp"
+#include "fwp_mfma.hpp"
 
 #include <type_traits>
 
 namespace fwp {
 namespace {
-
-typedef float v4f __attribute__((ext_vector_type(4)));
-
-// acc + X^T Y for 16x16 matrices in the accumulator layout
-__device__ __forceinline__ v4f tn(v4f X, v4f Y, v4f acc) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X[0], Y[0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X[1], Y[1], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X[2], Y[2], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(X[3], Y[3], acc, 0, 0, 0);
-    return acc;
-}
-
-constexpr int kBlk = 16;   // steps per block = MFMA tile edge
-constexpr int kAuxHeader = 16;   // floats before the per-block matrices in the auxiliary buffer
-
-// (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At
-// (accumulator layout): (I - At)(I + At^2)(I + At^4)(I + At^8), 8 products.
-__device__ __forceinline__ v4f inv_unit_triangular(v4f A, v4f At, v4f identity) {
-    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f T = identity - At;
-    const v4f A2 = tn(At, A, zero), At2 = tn(A, At, zero);
-    T = tn(A2, T, T);
-    const v4f A4 = tn(At2, A2, zero), At4 = tn(A2, At2, zero);
-    T = tn(A4, T, T);
-    const v4f A8 = tn(At4, A4, zero);
-    return tn(A8, T, T);
-}
-
-// Position of this lane's four registers in the accumulator layout.
-struct Geo16 {
-    int g, c;
-    bool up[4], lo[4], di[4];   // row < column, row > column, row == column for register r
-    __device__ explicit Geo16(int lane) : g(lane / 16), c(lane % 16) {
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            up[r] = 4 * g + r < c;
-            lo[r] = c < 4 * g + r;
-            di[r] = 4 * g + r == c;
-        }
-    }
-};
 
 // Per-lane element offsets inside a block (32-bit: a block spans 16 rows).
 struct LaneOffs {
@@ -871,7 +831,7 @@ int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk) {
 }
 
 // The auxiliary part of the checkpoint buffer starts right after the states.
-static float *aux_of(const float *ckpt, int N, int H, int L, int D, int chunk) {
+float *delta_aux_of(const float *ckpt, int N, int H, int L, int D, int chunk) {
     if (!ckpt) return nullptr;
     const int nchunk = (L + chunk - 1) / chunk;
     return const_cast<float *>(ckpt) + (int64_t)N * H * nchunk * D * D;
@@ -884,14 +844,14 @@ __global__ void k_store_float(float *dst, float x) { *dst = x; }
 // Forward kernels that do not leave the per-block matrices say so in the header.
 int delta_aux_invalidate(float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     if (!ckpt) return 0;
-    hipLaunchKernelGGL(k_store_float, dim3(1), dim3(1), 0, s, aux_of(ckpt, N, H, L, D, chunk), 0.f);
+    hipLaunchKernelGGL(k_store_float, dim3(1), dim3(1), 0, s, delta_aux_of(ckpt, N, H, L, D, chunk), 0.f);
     return (int)hipGetLastError();
 }
 
 int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    float *aux = aux_of(ckpt, N, H, L, D, chunk);
+    float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
     if (D == 16)
         hipLaunchKernelGGL(k_delta_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
                            vdiff, ckpt, aux, H, L, chunk, nchunk);
@@ -905,7 +865,7 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                    int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    const float *aux = aux_of(ckpt, N, H, L, D, chunk);
+    const float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
     if (D == 16)
         hipLaunchKernelGGL(k_delta_bwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, beta, vdiff, go,
                            ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);

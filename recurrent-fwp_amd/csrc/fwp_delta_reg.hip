@@ -71,6 +71,10 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     const int lane = threadIdx.x % kWave, col = lane / S, sl = lane % S, per = lane % 16;
     const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
     if (seq >= nseq) return;
+    // the word after the checkpoints tells the blocked backward kernel whether the forward pass
+    // left its per-block matrices behind it: this kernel does not
+    if constexpr (!SUM)
+        if (seq == 0 && lane == 0 && ckpt) ckpt[(int64_t)nseq * nchunk * D * D] = 0.f;
     const int n = (int)(seq / H), h = (int)(seq % H);
     auto &sq = sq_[wave];
     auto &sk = sk_[wave];

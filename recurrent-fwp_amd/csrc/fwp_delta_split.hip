@@ -1,0 +1,553 @@
+// Chunked delta-rule kernels with the work of one sequence split over the waves of a workgroup.
+//
+// The algebra is that of the one-wave blocked kernels (16-step blocks, fp32 MFMA, every 16x16 matrix
+// in the accumulator layout).  A sequence is one dependent chain and a wave issues one instruction
+// at a time, so a lone wave leaves the matrix pipe idle while it issues vector instructions or
+// waits for memory; there are fewer sequences than SIMDs, so the spare SIMDs take the part of a
+// block that does not lie on the chain:
+//
+//   forward, D/16 + 1 waves:  wave mb < D/16 owns the state columns [16 mb, 16 mb + 16) and does
+//       the products that need the state (X, U, O, d, S'); the last wave prepares, one block ahead,
+//       what depends on K, Q, beta only: (I + A)^-T, strict_lower(K K^T)^T, lower(Q K^T)^T.
+//   backward, 2 D/16 waves:   wave mb < D/16 ("adjoint") owns the columns of dS and walks the chain
+//       dS -> dU -> dY -> dX -> dS, stores g_v, and forms its share of lower(dO U^T) and
+//       strict_lower(dX U^T); wave D/16 + eb ("state"), one block behind, owns rows
+//       [16 eb, 16 eb + 16) of S, rewinds them and forms g_q, g_k for those columns, and g_beta.
+//
+// Hand-over is through LDS, two slots used alternately, one workgroup barrier per block: every
+// wave executes the same number of barriers whatever its role.  Sequence lengths are multiples of
+// 16 here (the host sends other lengths to the one-wave kernels), so the loops are straight-line.
+#include "fwp_common.hpp"
+#include "fwp_wave.hpp"
+#include "fwp_mfma.hpp"
+
+namespace fwp {
+namespace {
+
+// Workgroup barrier that orders the LDS hand-over only.  __syncthreads() also waits for every
+// global load and store of the wave, the prefetches of the coming blocks included.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
+__device__ __forceinline__ v4f as_v4f(const float *ptr) {
+    const float4 x = *reinterpret_cast<const float4 *>(ptr);
+    return v4f{x.x, x.y, x.z, x.w};
+}
+__device__ __forceinline__ float4 as_float4(const v4f &x) { return make_float4(x[0], x[1], x[2], x[3]); }
+__device__ __forceinline__ v4f from_float4(const float4 &x) { return v4f{x.x, x.y, x.z, x.w}; }
+
+// The per-block loop of one wave: `step(e, raw)` for e = 0 .. n-1 with the data of the coming PF
+// blocks in flight in a ring of registers, one barrier per block.  `load(raw, e)` is asked for
+// e <= n - 1 only (past the end the last block is loaded again and not used).  Memory latency is
+// several block times here, so one block ahead is not enough.
+template <int PF, class Raw, class Load, class Step>
+__device__ __forceinline__ void ring_loop(int n, Load load, Step step) {
+    Raw ring[PF];
+#pragma unroll
+    for (int j = 0; j < PF; j++) load(ring[j], min(j, n - 1));
+    int e = 0;
+    for (; e + PF <= n; e += PF) {
+#pragma unroll
+        for (int j = 0; j < PF; j++) {
+            step(e + j, ring[j]);
+            load(ring[j], min(e + j + PF, n - 1));
+            __builtin_amdgcn_sched_barrier(0);     // the loads are issued here, not next to their use
+            lds_barrier();
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < PF; j++) {
+        if (e + j < n) {
+            step(e + j, ring[j]);
+            lds_barrier();
+        }
+    }
+}
+
+// ------------------------------------------------------------------ forward
+
+// What the preparing wave reads of a block.
+// Kt[b], Qt[b]: register r = K[t0 + c][16b + 4g + r];  bcol = beta[t0 + c], brow[r] = beta[t0 + 4g + r]
+template <int NB>
+struct PrepRaw {
+    v4f Kt[NB], Qt[NB];
+    float bcol, brow[4];
+};
+
+// What a state wave reads of a block: K and Q whole, its own 16 columns of V.
+// Kc[b], Vc: register r = K[t0 + 4g + r][16b + c]
+template <int NB>
+struct MainRaw {
+    v4f Kt[NB], Qt[NB], Kc[NB], Vc;
+    float brow[4];
+};
+
+template <int NB, int PF>   // NB = D / 16, PF = blocks in flight
+__global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
+                                                                  fwp_view beta, float *__restrict__ W,
+                                                                  float *__restrict__ out,
+                                                                  float *__restrict__ vdiff,
+                                                                  float *__restrict__ ckpt,
+                                                                  float *__restrict__ aux, int H, int L,
+                                                                  int chunk, int nchunk) {
+    constexpr int D = 16 * NB;
+    // slot, matrix (0: (I + A)^-T, 1: strict_lower(K K^T)^T, 2: lower(Q K^T)^T), lane
+    __shared__ float4 xch[2][3][64];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int lane = threadIdx.x % 64;
+    const Geo16 p(lane);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
+                *bb = row(beta, n, h, 0);
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    const int nblk = L / kBlk;
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g);
+    unsigned o_br[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+
+    if (wave == NB) {
+        // ------------------------------------------------ preparing wave
+        // aux (with ckpt): a header whose first float says that the per-block matrices
+        // T = (I + A)^-1 follow, row-major, [sequence][block][16][16]; backward then does not
+        // invert again.
+        if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
+        float *aux_T = aux ? aux + kAuxHeader + seq * nblk * 256 + c * 16 + 4 * g : nullptr;
+        const unsigned o_bc = (unsigned)(c * beta.sL);
+        v4f ident;
+#pragma unroll
+        for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+        auto load = [&](PrepRaw<NB> &w, int ib) {
+            const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
+                        *bblk = bb + (int64_t)ib * kBlk * beta.sL;
+            w.bcol = bblk[o_bc];
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.brow[r] = bblk[o_br[r]];
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
+                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+            }
+        };
+        auto prepare = [&](const PrepRaw<NB> &w, int ib) {
+            v4f G = zero, R = zero;
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                G = tn(w.Kt[b], w.Kt[b], G);       // K K^T
+                R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
+            }
+            v4f A, At, Gu, Rm;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
+                At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
+                Gu[r] = p.up[r] ? G[r] : 0.f;
+                Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+            }
+            const v4f Tt = inv_unit_triangular(A, At, ident);     // (I + A)^-T
+            float4(*slot)[64] = xch[ib & 1];
+            slot[0][lane] = as_float4(Tt);
+            slot[1][lane] = as_float4(Gu);
+            slot[2][lane] = as_float4(Rm);
+            if (aux_T)       // register r = T[c][4g + r]
+                *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = as_float4(Tt);
+        };
+        {
+            PrepRaw<NB> first;
+            load(first, 0);
+            prepare(first, 0);
+        }
+        lds_barrier();
+        // while the state waves do block e: block e + 1 (nothing in the last round)
+        ring_loop<PF, PrepRaw<NB>>(
+            nblk, [&](PrepRaw<NB> &w, int e) { load(w, min(e + 1, nblk - 1)); },
+            [&](int e, const PrepRaw<NB> &w) {
+                if (e + 1 < nblk) prepare(w, e + 1);
+            });
+        return;
+    }
+
+    // ---------------------------------------------------- state wave of columns [16 mb, 16 mb + 16)
+    const int mb = wave;
+    unsigned o_kr[4], o_vr[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
+        o_vr[r] = (unsigned)((4 * g + r) * v.sL + 16 * mb + c);
+    }
+    auto load = [&](MainRaw<NB> &w, int ib) {
+        const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
+                    *vblk = vb + (int64_t)ib * kBlk * v.sL, *bblk = bb + (int64_t)ib * kBlk * beta.sL;
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            w.brow[r] = bblk[o_br[r]];
+            w.Vc[r] = vblk[o_vr[r]];
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
+            w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
+        }
+    };
+
+    // S[eb]: register r holds S[16 eb + 4g + r][16 mb + c]
+    v4f S[NB];
+#pragma unroll
+    for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+    float *out_l = out + seq * L * D + c * D + 16 * mb + 4 * g;                  // + t0 * D
+    float *vd_l = vdiff ? vdiff + seq * L * D + 4 * g * D + 16 * mb + c : nullptr;   // + (t0 + r) * D
+
+    auto block = [&](int ib, const MainRaw<NB> &cur) {
+        const float4(*slot)[64] = xch[ib & 1];
+        v4f KS = zero, Ot = zero;
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
+        const v4f Tt = from_float4(slot[0][lane]);
+        const v4f X = cur.Vc - KS;
+        v4f Y;
+#pragma unroll
+        for (int r = 0; r < 4; r++) Y[r] = cur.brow[r] * X[r];
+        const v4f U = tn(Tt, Y, zero);
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
+        const v4f Rm = from_float4(slot[2][lane]);
+        const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
+        *reinterpret_cast<float4 *>(out_l + (int64_t)ib * kBlk * D) = as_float4(O);
+        if (vd_l) {
+            const v4f Gu = from_float4(slot[1][lane]);
+            const v4f Dd = X - tn(Gu, U, zero);
+#pragma unroll
+            for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * D] = Dd[r];
+        }
+        const int t_end = (ib + 1) * kBlk;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][r];
+        }
+    };
+
+    lds_barrier();      // the preparing wave's block 0
+    ring_loop<PF, MainRaw<NB>>(nblk, load, block);
+#pragma unroll
+    for (int eb = 0; eb < NB; eb++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][r];
+}
+
+// ----------------------------------------------------------------- backward
+//
+// With S0 the state at the start of a block, U = diag(b) d (d = v - v_old, saved by forward),
+// T = (I + A)^-1, Pm = lower(Q K^T), dO the block's upstream gradient and dS the gradient of the
+// state after the block:
+//     dU = K dS + Pm^T dO            dY = T^T dU
+//     g_beta = rowsum(dY . d)        dX = diag(b) dY = g_v
+//     dPm = lower(dO U^T)            M = strict_lower(dX U^T)
+//     g_q = dO S0^T + dPm K
+//     g_k = U dS^T + dPm^T Q - dX S0^T - (M + M^T) K
+//     dS <- dS + Q^T dO - K^T dX
+// The adjoint wave of value columns mb hands over, per block: its columns of dS (before the
+// update), dX^T, and its share (the sum over its 16 value columns) of dPm, dPm^T, -(M + M^T) and
+// of g_beta.  The state waves add the shares.
+
+template <int NB>
+struct AdjRaw {
+    v4f Kt[NB], Qt[NB], Kc[NB], Qc[NB];
+    v4f Oc, Ot, Dt;          // upstream gradient and vdiff, the wave's 16 value columns
+    v4f T;                   // (I + A)^-1 when forward saved it
+    float bcol, brow[4];
+};
+
+template <int NB>
+struct StateRaw {
+    v4f Kc, Qc;                          // the wave's 16 key columns
+    v4f Ot[NB], Dc[NB], Dt[NB];
+    v4f Sck[NB];                         // checkpointed state of the block's chunk, transposed, rows of the wave
+    float bcol, brow[4];
+};
+
+template <int NB, int PF>
+__global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_view k, fwp_view beta,
+                                                             const float *__restrict__ vdiff, fwp_view go,
+                                                             const float *__restrict__ ckpt,
+                                                             const float *__restrict__ aux,
+                                                             float *__restrict__ gq, float *__restrict__ gk,
+                                                             float *__restrict__ gv,
+                                                             float *__restrict__ gbeta, int H, int L,
+                                                             int chunk, int nchunk) {
+    constexpr int D = 16 * NB;
+    constexpr int kDX = NB, kDPm = NB + 1, kDPmt = NB + 2, kNMs = NB + 3;
+    // slot, adjoint wave, matrix (dS rows eb = 0..NB-1, then dX^T, dPm, dPm^T, -(M + M^T)), lane
+    __shared__ float4 xch[2][NB][NB + 4][64];
+    __shared__ float gbx[2][NB][16];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int lane = threadIdx.x % 64;
+    const Geo16 p(lane);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
+                *bb = row(beta, n, h, 0), *db = vdiff + seq * L * D;
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f ident;
+#pragma unroll
+    for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+    const int nblk = L / kBlk;
+    const unsigned o_bc = (unsigned)(c * beta.sL);
+    unsigned o_br[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+
+    if (wave < NB) {
+        // ------------------------------------------------ adjoint wave of value columns mb
+        const int mb = wave;
+        // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
+        const bool have_T = aux && aux[0] == 1.f;
+        const float *aux_T = have_T ? aux + kAuxHeader + seq * nblk * 256 + 4 * g * 16 + c : nullptr;
+        const unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g),
+                       o_ot = (unsigned)(c * go.sL + 16 * mb + 4 * g),
+                       o_dt = (unsigned)(c * D + 16 * mb + 4 * g);
+        unsigned o_kr[4], o_qr[4], o_or[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
+            o_qr[r] = (unsigned)((4 * g + r) * q.sL + c);
+            o_or[r] = (unsigned)((4 * g + r) * go.sL + 16 * mb + c);
+        }
+        auto load = [&](AdjRaw<NB> &w, int e) {
+            const int ib = nblk - 1 - e;
+            if (have_T) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.T[r] = aux_T[(int64_t)ib * 256 + 16 * r];
+            }
+            const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
+                        *oblk = gob + (int64_t)ib * kBlk * go.sL, *dblk = db + (int64_t)ib * kBlk * D,
+                        *bblk = bb + (int64_t)ib * kBlk * beta.sL;
+            w.bcol = bblk[o_bc];
+            w.Ot = as_v4f(oblk + o_ot);
+            w.Dt = as_v4f(dblk + o_dt);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.brow[r] = bblk[o_br[r]];
+                w.Oc[r] = oblk[o_or[r]];
+            }
+#pragma unroll
+            for (int b = 0; b < NB; b++) {
+                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
+                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
+                    w.Qc[b][r] = qblk[o_qr[r] + 16 * b];
+                }
+            }
+        };
+
+        // dS[eb]: register r = dS[16 eb + 4g + r][16 mb + c]
+        v4f dS[NB];
+#pragma unroll
+        for (int eb = 0; eb < NB; eb++) dS[eb] = zero;
+        float *gv_l = gv + seq * L * D + c * D + 16 * mb + 4 * g;       // + t0 * D
+        auto block = [&](int e, const AdjRaw<NB> &w) {
+            const int ib = nblk - 1 - e;
+            float4(*slot)[64] = xch[ib & 1][mb];
+            v4f QK = zero;
+#pragma unroll
+            for (int b = 0; b < NB; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
+            v4f Pm;
+#pragma unroll
+            for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
+            v4f T = w.T;
+            if (!have_T) {
+                v4f G = zero, A, At;
+#pragma unroll
+                for (int b = 0; b < NB; b++) G = tn(w.Kt[b], w.Kt[b], G);
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
+                    At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
+                }
+                T = inv_unit_triangular(At, A, ident);      // (I + A)^-1
+            }
+            const v4f Ut = w.bcol * w.Dt;
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) slot[eb][lane] = as_float4(dS[eb]);
+            v4f dU = tn(Pm, w.Oc, zero);
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) dU = tn(w.Kt[eb], dS[eb], dU);
+            const v4f dY = tn(T, dU, zero), dYt = tn(dU, T, zero);
+            const v4f dXt = w.bcol * dYt;
+            v4f ndX;
+            float gb = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                ndX[r] = -(w.brow[r] * dY[r]);
+                gb = fmaf(dYt[r], w.Dt[r], gb);
+            }
+            // register r = g_v[t0 + c][16 mb + 4g + r]
+            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * D) = as_float4(dXt);
+            slot[kDX][lane] = as_float4(dXt);
+#pragma unroll
+            for (int eb = 0; eb < NB; eb++) {
+                dS[eb] = tn(w.Qc[eb], w.Oc, dS[eb]);
+                dS[eb] = tn(w.Kc[eb], ndX, dS[eb]);
+            }
+            {   // share of g_beta[t0 + c]: the four 16-lane rows hold partial sums
+                float y = gb;
+                swap16(gb, y);
+                gb += y;
+                y = gb;
+                swap32(gb, y);
+                gb += y;
+                if (g == 0) gbx[ib & 1][mb][c] = gb;
+            }
+            const v4f Z = tn(w.Ot, Ut, zero), Zt = tn(Ut, w.Ot, zero);     // dO U^T
+            const v4f M = tn(dXt, Ut, zero), Mt = tn(Ut, dXt, zero);       // dX U^T
+            v4f dPm, dPmt, nMs;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
+                dPmt[r] = (p.up[r] || p.di[r]) ? Zt[r] : 0.f;
+                nMs[r] = -((p.lo[r] ? M[r] : 0.f) + (p.up[r] ? Mt[r] : 0.f));
+            }
+            slot[kDPm][lane] = as_float4(dPm);
+            slot[kDPmt][lane] = as_float4(dPmt);
+            slot[kNMs][lane] = as_float4(nMs);
+        };
+        ring_loop<PF, AdjRaw<NB>>(nblk, load, block);
+        lds_barrier();        // the state waves' last block
+        return;
+    }
+
+    // ---------------------------------------------------- state wave of key columns [16 eb, 16 eb + 16)
+    const int eb = wave - NB;
+    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g), o_dt = (unsigned)(c * D + 4 * g);
+    unsigned o_kr[4], o_qr[4], o_dr[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + 16 * eb + c);
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + 16 * eb + c);
+        o_dr[r] = (unsigned)((4 * g + r) * D + c);
+    }
+    const unsigned o_ck = (unsigned)((16 * eb + c) * D + 4 * g);
+    auto load = [&](StateRaw<NB> &w, int e) {
+        const int ib = nblk - 1 - e;
+        {   // always loaded, so that no load is left to be issued (and waited for) inside the block
+            const float *src = ckpt + (seq * nchunk + ((ib + 1) * kBlk - 1) / chunk) * D * D;
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) w.Sck[mb] = as_v4f(src + (o_ck + 16 * mb));
+        }
+        const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
+                    *oblk = gob + (int64_t)ib * kBlk * go.sL, *dblk = db + (int64_t)ib * kBlk * D,
+                    *bblk = bb + (int64_t)ib * kBlk * beta.sL;
+        w.bcol = bblk[o_bc];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            w.brow[r] = bblk[o_br[r]];
+            w.Kc[r] = kblk[o_kr[r]];
+            w.Qc[r] = qblk[o_qr[r]];
+        }
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            w.Ot[b] = as_v4f(oblk + (o_ot + 16 * b));
+            w.Dt[b] = as_v4f(dblk + (o_dt + 16 * b));
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.Dc[b][r] = dblk[o_dr[r] + 16 * b];
+        }
+    };
+
+    // St[mb]: register r = S[16 eb + c][16 mb + 4g + r]  (block (mb, eb) of S^T)
+    v4f St[NB];
+    float *gq_l = gq + seq * L * D + c * D + 16 * eb + 4 * g, *gk_l = gk + seq * L * D + c * D + 16 * eb + 4 * g;
+    float *gb_l = gbeta + seq * L + c;
+    auto block = [&](int e, const StateRaw<NB> &w) {
+        const int ib = nblk - 1 - e;
+        const int t_end = (ib + 1) * kBlk;
+        if (t_end % chunk == 0 || t_end == L) {      // last block of a chunk: the state after it is checkpointed
+#pragma unroll
+            for (int mb = 0; mb < NB; mb++) St[mb] = w.Sck[mb];
+        }
+        // state at the start of the block, transposed: S0^T = S'^T - U^T K
+        v4f Ut[NB];
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            Ut[mb] = w.bcol * w.Dt[mb];
+            v4f nU;
+#pragma unroll
+            for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[mb][r]);
+            St[mb] = tn(nU, w.Kc, St[mb]);
+        }
+        v4f gQt = zero, gKt = zero;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) gQt = tn(St[mb], w.Ot[mb], gQt);
+        // what the adjoint waves left for this block
+        v4f dPm = zero, dPmt = zero, nMs = zero;
+        float gb = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < NB; mb++) {
+            const float4(*slot)[64] = xch[ib & 1][mb];
+            dPm += from_float4(slot[kDPm][lane]);
+            dPmt += from_float4(slot[kDPmt][lane]);
+            nMs += from_float4(slot[kNMs][lane]);
+            gb += gbx[ib & 1][mb][c];
+            const v4f dSb = from_float4(slot[eb][lane]), dXt = from_float4(slot[kDX][lane]);
+            const v4f dSt = tn(dSb, ident, zero);        // block (mb, eb) of dS^T
+            gKt = tn(dSt, Ut[mb], gKt);
+            gKt = tn(St[mb], -dXt, gKt);
+        }
+        gQt = tn(w.Kc, dPmt, gQt);
+        gKt = tn(w.Qc, dPm, gKt);
+        gKt = tn(w.Kc, nMs, gKt);
+        // register r = gradient[t0 + c][16 eb + 4g + r]
+        *reinterpret_cast<float4 *>(gq_l + (int64_t)ib * kBlk * D) = as_float4(gQt);
+        *reinterpret_cast<float4 *>(gk_l + (int64_t)ib * kBlk * D) = as_float4(gKt);
+        if (eb == 0 && g == 0) gb_l[ib * kBlk] = gb;
+    };
+
+    lds_barrier();            // the adjoint waves' first block
+    ring_loop<PF, StateRaw<NB>>(nblk, load, block);
+}
+
+}  // namespace
+
+bool split_delta_supported(int L) { return L >= kBlk && L % kBlk == 0; }
+
+int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
+    if (D == 16)
+        hipLaunchKernelGGL((k_delta_fwd_split<1, 4>), dim3(N * H), dim3(128), 0, s, q, k, v, beta, W,
+                           out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+    else
+        hipLaunchKernelGGL((k_delta_fwd_split<2, 4>), dim3(N * H), dim3(192), 0, s, q, k, v, beta, W,
+                           out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+    return (int)hipGetLastError();
+}
+
+int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
+                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
+                    int L, int D, int chunk, hipStream_t s) {
+    const int nchunk = (L + chunk - 1) / chunk;
+    const float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
+    if (D == 16)
+        hipLaunchKernelGGL((k_delta_bwd_split<1, 3>), dim3(N * H), dim3(128), 0, s, q, k, beta, vdiff,
+                           go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+    else
+        hipLaunchKernelGGL((k_delta_bwd_split<2, 3>), dim3(N * H), dim3(256), 0, s, q, k, beta, vdiff,
+                           go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fwp
