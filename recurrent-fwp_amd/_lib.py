@@ -86,10 +86,19 @@ def query(what):
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
 
 
+_ckpt_floats_cache = {}
+
+
 def delta_ckpt_floats(N, H, L, E, M, chunk):
-    n = int(lib().fwp_delta_ckpt_floats(N, H, L, E, M, chunk))
-    if n < 0:
-        raise FwpError(f"invalid dimensions N={N} H={H} L={L} E={E} M={M} chunk={chunk}")
+    key = (N, H, L, E, M, chunk)
+    n = _ckpt_floats_cache.get(key)
+    if n is None:
+        n = int(lib().fwp_delta_ckpt_floats(N, H, L, E, M, chunk))
+        if n < 0:
+            raise FwpError(f"invalid dimensions N={N} H={H} L={L} E={E} M={M} chunk={chunk}")
+        if len(_ckpt_floats_cache) > 1024:
+            _ckpt_floats_cache.clear()
+        _ckpt_floats_cache[key] = n
     return n
 
 
@@ -148,7 +157,8 @@ def rows(t):
 
 
 def ptr(t):
-    return ctypes.c_void_p(t.data_ptr())
+    """Device address of a tensor as ctypes takes it for a void* parameter."""
+    return t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -161,17 +171,26 @@ def stream_of(t):
     return torch.cuda.current_stream(t.device).cuda_stream
 
 
-class on_device:
-    """Make the tensor's GPU current for the launch; free when it already is."""
-
-    def __init__(self, t):
-        idx = (t if isinstance(t, torch.device) else t.device).index
-        self.guard = None if idx is None or idx == torch.cuda.current_device() else torch.cuda.device(idx)
-
+class _NoGuard:
     def __enter__(self):
-        if self.guard is not None:
-            self.guard.__enter__()
+        return None
 
     def __exit__(self, *exc):
-        if self.guard is not None:
-            self.guard.__exit__(*exc)
+        return False
+
+
+_NO_GUARD = _NoGuard()
+_single_gpu = None
+
+
+def on_device(t):
+    """Context that makes the tensor's GPU current for the launch; free when it already is."""
+    global _single_gpu
+    if _single_gpu is None:
+        _single_gpu = torch.cuda.device_count() == 1
+    if _single_gpu:
+        return _NO_GUARD
+    idx = (t if isinstance(t, torch.device) else t.device).index
+    if idx is None or idx == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(idx)

@@ -37,6 +37,44 @@ __device__ __forceinline__ v4f as_v4f(const float *ptr) {
 __device__ __forceinline__ float4 as_float4(const v4f &x) { return make_float4(x[0], x[1], x[2], x[3]); }
 __device__ __forceinline__ v4f from_float4(const float4 &x) { return v4f{x.x, x.y, x.z, x.w}; }
 
+// A 16x16 matrix in LDS as the 64 lanes' register quadruples (1 KB).  put() followed by get() hands a
+// matrix over as it is; put_t() followed by get() hands over its transpose: lane (g, c) holds
+// X[4g + r][c], which the reader of the transpose wants in lane (c / 4, 4g + r) as register c % 4.
+// A transpose costs four scattered LDS writes instead of the four MFMAs of a product with the
+// identity.  Within one wave LDS operations execute in order, so a wave may read back what it
+// has just written without a barrier.
+struct LdsMat {
+    float4 q[64];
+    __device__ __forceinline__ void put(int lane, const v4f &x) { q[lane] = as_float4(x); }
+    __device__ __forceinline__ void put_t(const Geo16 &p, const v4f &x) {
+        float *f = reinterpret_cast<float *>(q) + 64 * (p.c / 4) + 16 * p.g + p.c % 4;
+#pragma unroll
+        for (int r = 0; r < 4; r++) f[4 * r] = x[r];
+    }
+    __device__ __forceinline__ v4f get(int lane) const { return from_float4(q[lane]); }
+};
+
+// (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At:
+// (I - At)(I + At^2)(I + At^4)(I + At^8) with the transposes of the squares taken through LDS
+// (`scratch`: two matrices owned by the calling wave), 6 products.
+__device__ __forceinline__ v4f inv_unit_triangular_lds(v4f A, v4f At, v4f identity, LdsMat *scratch,
+                                                       const Geo16 &p, int lane) {
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    v4f T = identity - At;
+    const v4f A2 = tn(At, A, zero);
+    scratch[0].put_t(p, A2);
+    T = tn(A2, T, T);
+    __builtin_amdgcn_wave_barrier();
+    const v4f At2 = scratch[0].get(lane);
+    const v4f A4 = tn(At2, A2, zero);
+    scratch[1].put_t(p, A4);
+    T = tn(A4, T, T);
+    __builtin_amdgcn_wave_barrier();
+    const v4f At4 = scratch[1].get(lane);
+    const v4f A8 = tn(At4, A4, zero);
+    return tn(A8, T, T);
+}
+
 // The per-block loop of one wave: `step(e, raw)` for e = 0 .. n-1 with the data of the coming PF
 // blocks in flight in a ring of registers, one barrier per block.  `load(raw, e)` is asked for
 // e <= n - 1 only (past the end the last block is loaded again and not used).  Memory latency is
@@ -93,7 +131,8 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
                                                                   int chunk, int nchunk) {
     constexpr int D = 16 * NB;
     // slot, matrix (0: (I + A)^-T, 1: strict_lower(K K^T)^T, 2: lower(Q K^T)^T), lane
-    __shared__ float4 xch[2][3][64];
+    __shared__ LdsMat xch[2][3];
+    __shared__ LdsMat scratch[2];       // the preparing wave's
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -147,11 +186,11 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
                 Gu[r] = p.up[r] ? G[r] : 0.f;
                 Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
             }
-            const v4f Tt = inv_unit_triangular(A, At, ident);     // (I + A)^-T
-            float4(*slot)[64] = xch[ib & 1];
-            slot[0][lane] = as_float4(Tt);
-            slot[1][lane] = as_float4(Gu);
-            slot[2][lane] = as_float4(Rm);
+            const v4f Tt = inv_unit_triangular_lds(A, At, ident, scratch, p, lane);     // (I + A)^-T
+            LdsMat *slot = xch[ib & 1];
+            slot[0].put(lane, Tt);
+            slot[1].put(lane, Gu);
+            slot[2].put(lane, Rm);
             if (aux_T)       // register r = T[c][4g + r]
                 *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = as_float4(Tt);
         };
@@ -205,13 +244,13 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     float *vd_l = vdiff ? vdiff + seq * L * D + 4 * g * D + 16 * mb + c : nullptr;   // + (t0 + r) * D
 
     auto block = [&](int ib, const MainRaw<NB> &cur) {
-        const float4(*slot)[64] = xch[ib & 1];
+        const LdsMat *slot = xch[ib & 1];
         v4f KS = zero, Ot = zero;
 #pragma unroll
         for (int eb = 0; eb < NB; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
 #pragma unroll
         for (int eb = 0; eb < NB; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
-        const v4f Tt = from_float4(slot[0][lane]);
+        const v4f Tt = slot[0].get(lane);
         const v4f X = cur.Vc - KS;
         v4f Y;
 #pragma unroll
@@ -219,11 +258,11 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
         const v4f U = tn(Tt, Y, zero);
 #pragma unroll
         for (int eb = 0; eb < NB; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
-        const v4f Rm = from_float4(slot[2][lane]);
+        const v4f Rm = slot[2].get(lane);
         const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
         *reinterpret_cast<float4 *>(out_l + (int64_t)ib * kBlk * D) = as_float4(O);
         if (vd_l) {
-            const v4f Gu = from_float4(slot[1][lane]);
+            const v4f Gu = slot[1].get(lane);
             const v4f Dd = X - tn(Gu, U, zero);
 #pragma unroll
             for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * D] = Dd[r];
@@ -258,8 +297,9 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
 //     g_k = U dS^T + dPm^T Q - dX S0^T - (M + M^T) K
 //     dS <- dS + Q^T dO - K^T dX
 // The adjoint wave of value columns mb hands over, per block: its columns of dS (before the
-// update), dX^T, and its share (the sum over its 16 value columns) of dPm, dPm^T, -(M + M^T) and
-// of g_beta.  The state waves add the shares.
+// update, transposed), dX^T, and its share (the sum over its 16 value columns) of dPm, of M, both
+// also transposed, and of g_beta.  The state waves add the shares.  A matrix that is needed
+// transposed is written to LDS transposed instead of being multiplied out a second time.
 
 template <int NB>
 struct AdjRaw {
@@ -287,9 +327,11 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
                                                              float *__restrict__ gbeta, int H, int L,
                                                              int chunk, int nchunk) {
     constexpr int D = 16 * NB;
-    constexpr int kDX = NB, kDPm = NB + 1, kDPmt = NB + 2, kNMs = NB + 3;
-    // slot, adjoint wave, matrix (dS rows eb = 0..NB-1, then dX^T, dPm, dPm^T, -(M + M^T)), lane
-    __shared__ float4 xch[2][NB][NB + 4][64];
+    constexpr int kDX = NB, kDPm = NB + 1, kDPmt = NB + 2, kNM = NB + 3, kNMt = NB + 4;
+    // slot, adjoint wave, matrix: blocks eb = 0..NB-1 of dS^T, then dX^T, dPm, dPm^T,
+    // -strict_lower(dX U^T) and its transpose
+    __shared__ LdsMat xch[2][NB][NB + 5];
+    __shared__ LdsMat scratch[NB][2];       // the adjoint waves'
     __shared__ float gbx[2][NB][16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
@@ -361,7 +403,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         float *gv_l = gv + seq * L * D + c * D + 16 * mb + 4 * g;       // + t0 * D
         auto block = [&](int e, const AdjRaw<NB> &w) {
             const int ib = nblk - 1 - e;
-            float4(*slot)[64] = xch[ib & 1][mb];
+            LdsMat *slot = xch[ib & 1][mb];
             v4f QK = zero;
 #pragma unroll
             for (int b = 0; b < NB; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
@@ -378,31 +420,35 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
                     A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
                     At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
                 }
-                T = inv_unit_triangular(At, A, ident);      // (I + A)^-1
+                T = inv_unit_triangular_lds(At, A, ident, scratch[mb], p, lane);      // (I + A)^-1
             }
             const v4f Ut = w.bcol * w.Dt;
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) slot[eb][lane] = as_float4(dS[eb]);
+            for (int eb = 0; eb < NB; eb++) slot[eb].put_t(p, dS[eb]);
             v4f dU = tn(Pm, w.Oc, zero);
 #pragma unroll
             for (int eb = 0; eb < NB; eb++) dU = tn(w.Kt[eb], dS[eb], dU);
-            const v4f dY = tn(T, dU, zero), dYt = tn(dU, T, zero);
-            const v4f dXt = w.bcol * dYt;
+            const v4f dY = tn(T, dU, zero);
+            scratch[mb][0].put_t(p, dY);
             v4f ndX;
-            float gb = 0.f;
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                ndX[r] = -(w.brow[r] * dY[r]);
-                gb = fmaf(dYt[r], w.Dt[r], gb);
-            }
-            // register r = g_v[t0 + c][16 mb + 4g + r]
-            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * D) = as_float4(dXt);
-            slot[kDX][lane] = as_float4(dXt);
+            for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
 #pragma unroll
             for (int eb = 0; eb < NB; eb++) {
                 dS[eb] = tn(w.Qc[eb], w.Oc, dS[eb]);
                 dS[eb] = tn(w.Kc[eb], ndX, dS[eb]);
             }
+            const v4f Z = tn(w.Ot, Ut, zero);      // dO U^T
+            __builtin_amdgcn_wave_barrier();
+            const v4f dYt = scratch[mb][0].get(lane);
+            const v4f dXt = w.bcol * dYt;
+            float gb = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
+            // register r = g_v[t0 + c][16 mb + 4g + r]
+            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * D) = as_float4(dXt);
+            slot[kDX].put(lane, dXt);
+            const v4f M = tn(dXt, Ut, zero);       // dX U^T
             {   // share of g_beta[t0 + c]: the four 16-lane rows hold partial sums
                 float y = gb;
                 swap16(gb, y);
@@ -412,18 +458,16 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
                 gb += y;
                 if (g == 0) gbx[ib & 1][mb][c] = gb;
             }
-            const v4f Z = tn(w.Ot, Ut, zero), Zt = tn(Ut, w.Ot, zero);     // dO U^T
-            const v4f M = tn(dXt, Ut, zero), Mt = tn(Ut, dXt, zero);       // dX U^T
-            v4f dPm, dPmt, nMs;
+            v4f dPm, nM;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-                dPmt[r] = (p.up[r] || p.di[r]) ? Zt[r] : 0.f;
-                nMs[r] = -((p.lo[r] ? M[r] : 0.f) + (p.up[r] ? Mt[r] : 0.f));
+                nM[r] = p.lo[r] ? -M[r] : 0.f;
             }
-            slot[kDPm][lane] = as_float4(dPm);
-            slot[kDPmt][lane] = as_float4(dPmt);
-            slot[kNMs][lane] = as_float4(nMs);
+            slot[kDPm].put(lane, dPm);
+            slot[kDPmt].put_t(p, dPm);
+            slot[kNM].put(lane, nM);
+            slot[kNMt].put_t(p, nM);
         };
         ring_loop<PF, AdjRaw<NB>>(nblk, load, block);
         lds_barrier();        // the state waves' last block
@@ -496,13 +540,12 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         float gb = 0.f;
 #pragma unroll
         for (int mb = 0; mb < NB; mb++) {
-            const float4(*slot)[64] = xch[ib & 1][mb];
-            dPm += from_float4(slot[kDPm][lane]);
-            dPmt += from_float4(slot[kDPmt][lane]);
-            nMs += from_float4(slot[kNMs][lane]);
+            const LdsMat *slot = xch[ib & 1][mb];
+            dPm += slot[kDPm].get(lane);
+            dPmt += slot[kDPmt].get(lane);
+            nMs += slot[kNM].get(lane) + slot[kNMt].get(lane);
             gb += gbx[ib & 1][mb][c];
-            const v4f dSb = from_float4(slot[eb][lane]), dXt = from_float4(slot[kDX][lane]);
-            const v4f dSt = tn(dSb, ident, zero);        // block (mb, eb) of dS^T
+            const v4f dSt = slot[eb].get(lane), dXt = slot[kDX].get(lane);     // dSt: block (mb, eb) of dS^T
             gKt = tn(dSt, Ut[mb], gKt);
             gKt = tn(St[mb], -dXt, gKt);
         }

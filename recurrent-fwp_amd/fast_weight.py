@@ -36,19 +36,22 @@ class DeltaFastWeight(torch.autograd.Function):
         need_grad = any(ctx.needs_input_grad[:4])
         chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
         out = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
-        vdiff = ckpt = None
+        saved = vdiff = ckpt = None
         if need_grad:
-            vdiff = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
-            ckpt = torch.empty(_lib.delta_ckpt_floats(N, H, L, E, M, chunk), device=Q.device,
-                               dtype=torch.float32)
+            # v - v_old [N,H,L,M] and the checkpoints behind it, one allocation (L*M is a multiple
+            # of 4 floats whenever the kernels need 16-byte alignment of either)
+            n_vdiff = N * H * L * M
+            saved = torch.empty(n_vdiff + _lib.delta_ckpt_floats(N, H, L, E, M, chunk), device=Q.device,
+                                dtype=torch.float32)
+            vdiff = saved.data_ptr()
+            ckpt = vdiff + 4 * n_vdiff
         with _lib.on_device(Q):
-            rc = _lib.lib().fwp_delta_fwd(
-                qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out),
-                _lib.ptr(vdiff) if need_grad else None, _lib.ptr(ckpt) if need_grad else None,
-                N, H, L, E, M, chunk, _lib.stream_of(Q))
-        _lib.check(rc, "fwp_delta_fwd")
+            rc = _lib.lib().fwp_delta_fwd(qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out), vdiff, ckpt,
+                                          N, H, L, E, M, chunk, _lib.stream_of(Q))
+        if rc:
+            _lib.check(rc, "fwp_delta_fwd")
         if need_grad:
-            ctx.save_for_backward(Q, K, beta, vdiff, ckpt)
+            ctx.save_for_backward(Q, K, beta, saved)
             ctx.dims = (N, H, L, E, M, chunk)
             ctx.views = (qv, kv, bv)        # of the saved tensors, which keep the memory alive
         ctx.set_materialize_grads(False)
@@ -58,8 +61,10 @@ class DeltaFastWeight(torch.autograd.Function):
     def backward(ctx, grad_out):
         if grad_out is None:
             return None, None, None, None, None
-        Q, K, beta, vdiff, ckpt = ctx.saved_tensors
+        Q, K, beta, saved = ctx.saved_tensors
         N, H, L, E, M, chunk = ctx.dims
+        vdiff = saved.data_ptr()
+        ckpt = vdiff + 4 * N * H * L * M
         qv, kv, bv = ctx.views
         grad_out, gv_ = _lib.rows(grad_out)
         grad_Q = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
@@ -68,10 +73,11 @@ class DeltaFastWeight(torch.autograd.Function):
         grad_beta = torch.empty((N, H, L, 1), device=Q.device, dtype=torch.float32)
         with _lib.on_device(Q):
             rc = _lib.lib().fwp_delta_bwd(
-                qv, kv, bv, _lib.ptr(vdiff), gv_, _lib.ptr(ckpt), _lib.ptr(grad_Q),
+                qv, kv, bv, vdiff, gv_, ckpt, _lib.ptr(grad_Q),
                 _lib.ptr(grad_K), _lib.ptr(grad_V), _lib.ptr(grad_beta), N, H, L, E, M, chunk,
                 _lib.stream_of(Q))
-        _lib.check(rc, "fwp_delta_bwd")
+        if rc:
+            _lib.check(rc, "fwp_delta_bwd")
         return grad_Q, grad_K, grad_V, grad_beta, None
 
 
