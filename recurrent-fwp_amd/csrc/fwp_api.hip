@@ -2,6 +2,8 @@
 // the register-state kernels (E = M in {16, 32}, 16-byte aligned rows) and the
 // LDS-state kernels (everything else).
 #include "fwp_common.hpp"
+
+#include <initializer_list>
 #include <stdint.h>
 
 #include <string.h>
@@ -31,8 +33,10 @@ bool delta_chunked(int L) {
 
 // Several waves per sequence pay off while they find SIMDs of their own: measured on MI355X
 // (1024 SIMDs) the split kernels win up to about two waves per SIMD and lose beyond.
-bool delta_split(int N, int H, int L, int D) {
+bool delta_split(int N, int H, int L, int D, std::initializer_list<fwp_view> views) {
     if (!split_delta_supported(L)) return false;
+    for (const fwp_view &v : views)      // the split kernels address a sequence with 32-bit byte offsets
+        if (v.sL < 0 || ((int64_t)L * v.sL + D) * 4 >= (int64_t(1) << 31)) return false;
     if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
     return g_delta_kernels == FWP_DELTA_AUTO && L >= 32 && (int64_t)N * H * (D / 8) <= 2048;
 }
@@ -97,7 +101,7 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         aligned16(vdiff) && aligned16(ckpt) && aligned16(out)) {
-        if (delta_split(N, H, L, E))
+        if (delta_split(N, H, L, E, {q, k, v, beta}))
             return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                                    (hipStream_t)stream);
         if (delta_chunked(L))
@@ -121,7 +125,7 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
         aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv)) {
-        if (delta_split(N, H, L, E))
+        if (delta_split(N, H, L, E, {q, k, beta, grad_out}))
             return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
                                    chunk, (hipStream_t)stream);
         if (delta_chunked(L))

@@ -75,6 +75,18 @@ __device__ __forceinline__ v4f inv_unit_triangular_lds(v4f A, v4f At, v4f identi
     return tn(A8, T, T);
 }
 
+// Index of the checkpoint chunk a block lies in: block / blocks_per_chunk as a multiplication
+// (exact while block * blocks_per_chunk < 2^32), the remainder alongside.
+struct ChunkOf {
+    unsigned bpc, magic;
+    __device__ explicit ChunkOf(int chunk) : bpc(chunk / kBlk), magic(0xFFFFFFFFu / bpc + 1) {}
+    __device__ __forceinline__ unsigned operator()(unsigned block) const { return __umulhi(block, magic); }
+    // is `block` the last one of its chunk?
+    __device__ __forceinline__ bool closes(unsigned block) const {
+        return (block + 1) - (*this)(block + 1) * bpc == 0;
+    }
+};
+
 // The per-block loop of one wave: `step(e, raw)` for e = 0 .. n-1 with the data of the coming PF
 // blocks in flight in a ring of registers, one barrier per block.  `load(raw, e)` is asked for
 // e <= n - 1 only (past the end the last block is loaded again and not used).  Memory latency is
@@ -139,14 +151,19 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
-                *bb = row(beta, n, h, 0);
+    // rows of this sequence; lane offsets and block steps in bytes
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + D) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + D) * 4)),
+        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + D) * 4)),
+        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     const int nblk = L / kBlk;
-    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g);
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4;
     unsigned o_br[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
 
     if (wave == NB) {
         // ------------------------------------------------ preparing wave
@@ -155,20 +172,19 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
         // invert again.
         if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
         float *aux_T = aux ? aux + kAuxHeader + seq * nblk * 256 + c * 16 + 4 * g : nullptr;
-        const unsigned o_bc = (unsigned)(c * beta.sL);
+        const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
         v4f ident;
 #pragma unroll
         for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
         auto load = [&](PrepRaw<NB> &w, int ib) {
-            const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
-                        *bblk = bb + (int64_t)ib * kBlk * beta.sL;
-            w.bcol = bblk[o_bc];
+            const unsigned ks = ib * k_step, qs = ib * q_step, bs = ib * b_step;
+            w.bcol = bb.f(o_bc, bs);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.brow[r] = bblk[o_br[r]];
+            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
-                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
             }
         };
         auto prepare = [&](const PrepRaw<NB> &w, int ib) {
@@ -214,23 +230,22 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     unsigned o_kr[4], o_vr[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
-        o_vr[r] = (unsigned)((4 * g + r) * v.sL + 16 * mb + c);
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+        o_vr[r] = (unsigned)((4 * g + r) * v.sL + 16 * mb + c) * 4;
     }
     auto load = [&](MainRaw<NB> &w, int ib) {
-        const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
-                    *vblk = vb + (int64_t)ib * kBlk * v.sL, *bblk = bb + (int64_t)ib * kBlk * beta.sL;
+        const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step, bs = ib * b_step;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            w.brow[r] = bblk[o_br[r]];
-            w.Vc[r] = vblk[o_vr[r]];
+            w.brow[r] = bb.f(o_br[r], bs);
+            w.Vc[r] = vb.f(o_vr[r], vs);
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
-            w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+            w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
+            for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
         }
     };
 
@@ -240,6 +255,7 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     for (int eb = 0; eb < NB; eb++)
 #pragma unroll
         for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+    const ChunkOf chunk_of(chunk);
     float *out_l = out + seq * L * D + c * D + 16 * mb + 4 * g;                  // + t0 * D
     float *vd_l = vdiff ? vdiff + seq * L * D + 4 * g * D + 16 * mb + c : nullptr;   // + (t0 + r) * D
 
@@ -267,9 +283,8 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
             for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * D] = Dd[r];
         }
-        const int t_end = (ib + 1) * kBlk;
-        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
-            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+        if (ckpt && (chunk_of.closes(ib) || ib + 1 == nblk)) {
+            float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * D * D;
 #pragma unroll
             for (int eb = 0; eb < NB; eb++)
 #pragma unroll
@@ -339,59 +354,66 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
-                *bb = row(beta, n, h, 0), *db = vdiff + seq * L * D;
+    // rows of this sequence; lane offsets and block steps in bytes
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + D) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + D) * 4)),
+        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + D) * 4)),
+        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
+        db(vdiff + seq * L * D, (uint32_t)(L * D * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   o_step = (unsigned)(kBlk * go.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
+                   d_step = (unsigned)(kBlk * D * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     v4f ident;
 #pragma unroll
     for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
     const int nblk = L / kBlk;
-    const unsigned o_bc = (unsigned)(c * beta.sL);
+    const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
     unsigned o_br[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
 
     if (wave < NB) {
         // ------------------------------------------------ adjoint wave of value columns mb
         const int mb = wave;
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
         const bool have_T = aux && aux[0] == 1.f;
-        const float *aux_T = have_T ? aux + kAuxHeader + seq * nblk * 256 + 4 * g * 16 + c : nullptr;
-        const unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g),
-                       o_ot = (unsigned)(c * go.sL + 16 * mb + 4 * g),
-                       o_dt = (unsigned)(c * D + 16 * mb + 4 * g);
+        const RowBuf tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0);
+        const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4;
+        const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                       o_ot = (unsigned)(c * go.sL + 16 * mb + 4 * g) * 4,
+                       o_dt = (unsigned)(c * D + 16 * mb + 4 * g) * 4;
         unsigned o_kr[4], o_qr[4], o_or[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
-            o_qr[r] = (unsigned)((4 * g + r) * q.sL + c);
-            o_or[r] = (unsigned)((4 * g + r) * go.sL + 16 * mb + c);
+            o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+            o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
+            o_or[r] = (unsigned)((4 * g + r) * go.sL + 16 * mb + c) * 4;
         }
         auto load = [&](AdjRaw<NB> &w, int e) {
             const int ib = nblk - 1 - e;
             if (have_T) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.T[r] = aux_T[(int64_t)ib * 256 + 16 * r];
+                for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
             }
-            const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
-                        *oblk = gob + (int64_t)ib * kBlk * go.sL, *dblk = db + (int64_t)ib * kBlk * D,
-                        *bblk = bb + (int64_t)ib * kBlk * beta.sL;
-            w.bcol = bblk[o_bc];
-            w.Ot = as_v4f(oblk + o_ot);
-            w.Dt = as_v4f(dblk + o_dt);
+            const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
+                           bs = ib * b_step;
+            w.bcol = bb.f(o_bc, bs);
+            w.Ot = gob.f4(o_ot, os);
+            w.Dt = db.f4(o_dt, ds);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                w.brow[r] = bblk[o_br[r]];
-                w.Oc[r] = oblk[o_or[r]];
+                w.brow[r] = bb.f(o_br[r], bs);
+                w.Oc[r] = gob.f(o_or[r], os);
             }
 #pragma unroll
             for (int b = 0; b < NB; b++) {
-                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
-                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
+                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
-                    w.Qc[b][r] = qblk[o_qr[r] + 16 * b];
+                    w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+                    w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
                 }
             }
         };
@@ -476,38 +498,39 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
 
     // ---------------------------------------------------- state wave of key columns [16 eb, 16 eb + 16)
     const int eb = wave - NB;
-    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g), o_dt = (unsigned)(c * D + 4 * g);
+    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * D + 4 * g) * 4;
     unsigned o_kr[4], o_qr[4], o_dr[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        o_kr[r] = (unsigned)((4 * g + r) * k.sL + 16 * eb + c);
-        o_qr[r] = (unsigned)((4 * g + r) * q.sL + 16 * eb + c);
-        o_dr[r] = (unsigned)((4 * g + r) * D + c);
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + 16 * eb + c) * 4;
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + 16 * eb + c) * 4;
+        o_dr[r] = (unsigned)((4 * g + r) * D + c) * 4;
     }
-    const unsigned o_ck = (unsigned)((16 * eb + c) * D + 4 * g);
+    const RowBuf cb(ckpt + seq * nchunk * D * D, (uint32_t)(nchunk * D * D * 4));
+    const unsigned o_ck = (unsigned)((16 * eb + c) * D + 4 * g) * 4;
+    const ChunkOf chunk_of(chunk);
     auto load = [&](StateRaw<NB> &w, int e) {
         const int ib = nblk - 1 - e;
         {   // always loaded, so that no load is left to be issued (and waited for) inside the block
-            const float *src = ckpt + (seq * nchunk + ((ib + 1) * kBlk - 1) / chunk) * D * D;
+            const unsigned cs = chunk_of(ib) * (D * D * 4);
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) w.Sck[mb] = as_v4f(src + (o_ck + 16 * mb));
+            for (int mb = 0; mb < NB; mb++) w.Sck[mb] = cb.f4(o_ck + 64 * mb, cs);
         }
-        const float *kblk = kb + (int64_t)ib * kBlk * k.sL, *qblk = qb + (int64_t)ib * kBlk * q.sL,
-                    *oblk = gob + (int64_t)ib * kBlk * go.sL, *dblk = db + (int64_t)ib * kBlk * D,
-                    *bblk = bb + (int64_t)ib * kBlk * beta.sL;
-        w.bcol = bblk[o_bc];
+        const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
+                       bs = ib * b_step;
+        w.bcol = bb.f(o_bc, bs);
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            w.brow[r] = bblk[o_br[r]];
-            w.Kc[r] = kblk[o_kr[r]];
-            w.Qc[r] = qblk[o_qr[r]];
+            w.brow[r] = bb.f(o_br[r], bs);
+            w.Kc[r] = kb.f(o_kr[r], ks);
+            w.Qc[r] = qb.f(o_qr[r], qs);
         }
 #pragma unroll
         for (int b = 0; b < NB; b++) {
-            w.Ot[b] = as_v4f(oblk + (o_ot + 16 * b));
-            w.Dt[b] = as_v4f(dblk + (o_dt + 16 * b));
+            w.Ot[b] = gob.f4(o_ot + 64 * b, os);
+            w.Dt[b] = db.f4(o_dt + 64 * b, ds);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.Dc[b][r] = dblk[o_dr[r] + 16 * b];
+            for (int r = 0; r < 4; r++) w.Dc[b][r] = db.f(o_dr[r] + 64 * b, ds);
         }
     };
 
@@ -517,8 +540,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
     float *gb_l = gbeta + seq * L + c;
     auto block = [&](int e, const StateRaw<NB> &w) {
         const int ib = nblk - 1 - e;
-        const int t_end = (ib + 1) * kBlk;
-        if (t_end % chunk == 0 || t_end == L) {      // last block of a chunk: the state after it is checkpointed
+        if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
 #pragma unroll
             for (int mb = 0; mb < NB; mb++) St[mb] = w.Sck[mb];
         }

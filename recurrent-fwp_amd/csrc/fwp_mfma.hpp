@@ -50,4 +50,28 @@ struct Geo16 {
     }
 };
 
+// The buffer-load intrinsics, declared by their LLVM names (the clang builtin for the 128-bit load
+// comes out as a 32-bit load with this compiler).
+typedef int v4i __attribute__((ext_vector_type(4)));
+__device__ float llvm_raw_buffer_load_f32(v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
+__device__ v4f llvm_raw_buffer_load_v4f32(v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
+
+// Read access to one sequence's rows of a tensor through a buffer resource: the address of a load
+// is (descriptor base) + (32-bit byte offset per lane, VGPR) + (byte offset per block, SGPR) +
+// (immediate), so moving on to the next block costs one scalar multiply and no vector address
+// arithmetic.  All offsets stay below 2^31 (checked on the host).
+struct RowBuf {
+    v4i rsrc;       // base address (48 bits, stride 0), size in bytes, 32-bit data format
+    __device__ __forceinline__ RowBuf(const float *base, uint32_t bytes) {
+        const uint64_t a = reinterpret_cast<uint64_t>(base);
+        rsrc = v4i{(int)(uint32_t)a, (int)(uint32_t)((a >> 32) & 0xffff), (int)bytes, 0x00020000};
+    }
+    __device__ __forceinline__ float f(unsigned lane_bytes, unsigned block_bytes) const {
+        return llvm_raw_buffer_load_f32(rsrc, (int)lane_bytes, (int)block_bytes, 0);
+    }
+    __device__ __forceinline__ v4f f4(unsigned lane_bytes, unsigned block_bytes) const {
+        return llvm_raw_buffer_load_v4f32(rsrc, (int)lane_bytes, (int)block_bytes, 0);
+    }
+};
+
 }  // namespace fwp
