@@ -1,0 +1,67 @@
+"""The C++ autograd binding of the delta rule (csrc/fwp_torch.cpp) against the Python
+autograd.Function over the same C ABI: same results bit for bit, same errors, same treatment
+of views and of inputs that need no gradient."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import delta_inputs
+
+
+def native(fwp):
+    mod = fwp.fast_weight._fwp_torch
+    if mod is None:
+        pytest.fail("recurrent-fwp_amd/_fwp_torch.so has not been built (csrc/build_torch.sh)")
+    return mod
+
+
+def test_binding_is_built_and_is_the_default(fwp):
+    assert fwp.fast_weight_delta is native(fwp).fast_weight_delta
+
+
+def test_binding_refuses_what_the_python_function_refuses(fwp):
+    f = native(fwp).fast_weight_delta
+    q = torch.zeros(1, 1, 2, 4)
+    with pytest.raises(fwp._lib.FwpError, match="MI355X"):
+        f(q, q, q, q[..., :1], torch.zeros(1, 1, 4, 4))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,L,E,M", [(2, 2, 64, 16, 16), (2, 3, 130, 32, 32), (1, 2, 37, 24, 8), (1, 2, 1, 16, 16)])
+def test_same_as_python_function(fwp, N, H, L, E, M):
+    q, k, v, beta, W0, go = (torch.from_numpy(a).cuda() for a in delta_inputs(3, N, H, L, E, M, dtype=np.float32))
+    results = []
+    for f in (native(fwp).fast_weight_delta, fwp.DeltaFastWeight.apply):
+        ins = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+        W = W0.clone()
+        out = f(*ins, W)
+        grads = torch.autograd.grad(out, ins, go)
+        results.append([out, W, *grads])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.gpu
+def test_views_no_grad_and_shape_errors(fwp):
+    f = native(fwp).fast_weight_delta
+    N, H, L, D = 2, 2, 48, 16
+    q, k, v, beta, W0, go = (torch.from_numpy(a).cuda() for a in delta_inputs(5, N, H, L, D, D, dtype=np.float32))
+    # [L,N,H,3D+1] storage as the Delta-Net layer hands it over: permuted views, v with unaligned rows
+    packed = torch.cat((q, k, v, beta), -1).permute(2, 0, 1, 3).contiguous()
+    qs, ks, vs, bs = (t.permute(1, 2, 0, 3) for t in packed.split((D, D, D, 1), -1))
+    W1, W2 = W0.clone(), W0.clone()
+    assert torch.equal(f(qs, ks, vs, bs, W1), fwp.DeltaFastWeight.apply(q, k, v, beta, W2))
+    assert torch.equal(W1, W2)
+    # only v wants a gradient
+    vr = v.clone().requires_grad_(True)
+    out = f(q, k, vr, beta, W0.clone())
+    (gv,) = torch.autograd.grad(out, vr, go)
+    vr2 = v.clone().requires_grad_(True)
+    (gv2,) = torch.autograd.grad(fwp.DeltaFastWeight.apply(q, k, vr2, beta, W0.clone()), vr2, go)
+    assert torch.equal(gv, gv2)
+    with torch.no_grad():
+        assert not f(q.requires_grad_(True), k, v, beta, W0.clone()).requires_grad
+    with pytest.raises(fwp._lib.FwpError, match="shape mismatch"):
+        f(q, k[:, :, :-1], v, beta, W0.clone())
+    with pytest.raises(fwp._lib.FwpError, match="W must be"):
+        f(q, k, v, beta, W0.clone().transpose(2, 3))
