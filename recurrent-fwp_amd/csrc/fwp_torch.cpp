@@ -1,8 +1,9 @@
-// The delta-rule operator as a C++ autograd function over the C ABI of libfwp_hip.so.
+// The delta-rule and sum-rule operators as C++ autograd functions over the C ABI of libfwp_hip.so.
 //
-// Same operator, arguments, results and errors as DeltaFastWeight in fast_weight.py (the reference's
-// algorithmic/fast_weight/__init__.py:26-96); it exists because a forward + backward pair of the
-// benchmark shape takes ~50 us on the GPU and ~57 us of interpreter time through a Python
+// Same operators, arguments, results and errors as DeltaFastWeight in fast_weight.py and FastWeightSum
+// in fast_transformers.py (the reference's algorithmic/fast_weight/__init__.py:26-96 and
+// algorithmic/fast_transformers/__init__.py:25-84); they exist because a forward + backward pair of the
+// benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter time through a Python
 // autograd.Function.  Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
 
@@ -149,6 +150,81 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
     }
 };
 
+struct SumFn : torch::autograd::Function<SumFn> {
+    // exact: grad_Q is the gradient of the recurrence as written; otherwise a carried-in state is left
+    // out of it, as the reference's backward does (causal_product_cuda.cu:385)
+    static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Q_in,
+                              const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &W, bool exact,
+                              bool need_grad) {
+        require_device(Q_in);
+        if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
+        const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
+        if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}))
+            fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in));
+        if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
+            fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+        fwp_view qv, kv, vv;
+        const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), V = rows(V_in, vv);
+        const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
+        const auto opts = Q.options();
+        at::Tensor out = at::empty({N, H, L, M}, opts), ckpt, W_init;
+        if (need_grad) {
+            ckpt = at::empty({N, H, (L + chunk - 1) / chunk, E, M}, opts);
+            if (!exact) W_init = W.clone();
+        }
+        {
+            c10::OptionalDeviceGuard guard;
+            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            check(fwp_sum_fwd(qv, kv, vv, W.data_ptr<float>(), out.data_ptr<float>(),
+                              need_grad ? ckpt.data_ptr<float>() : nullptr, (int)N, (int)H, (int)L, (int)E, (int)M,
+                              chunk, stream_of(Q)),
+                  "fwp_sum_fwd");
+        }
+        if (need_grad) {
+            if (exact) ctx->save_for_backward({Q, K, V, ckpt});
+            else ctx->save_for_backward({Q, K, V, ckpt, W_init});
+            ctx->saved_data["chunk"] = (int64_t)chunk;
+        }
+        ctx->set_materialize_grads(false);
+        return out;
+    }
+
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
+                                                 torch::autograd::tensor_list grads) {
+        const at::Tensor none;
+        if (!grads[0].defined()) return {none, none, none, none, none, none};
+        const auto saved = ctx->get_saved_variables();
+        if (saved.size() < 4) fail("backward of a forward pass that kept nothing for it");
+        const at::Tensor &Q = saved[0], &K = saved[1], &V = saved[2], &ckpt = saved[3];
+        const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3), M = V.size(3);
+        const int chunk = (int)ctx->saved_data["chunk"].toInt();
+        fwp_view qv, kv, vv, gv_;
+        rows(Q, qv);        // saved after rows(): no copies here
+        rows(K, kv);
+        rows(V, vv);
+        const at::Tensor go = rows(grads[0], gv_);
+        const auto opts = Q.options();
+        at::Tensor gq = at::empty({N, H, L, E}, opts), gk = at::empty({N, H, L, E}, opts),
+                   gv = at::empty({N, H, L, M}, opts);
+        {
+            c10::OptionalDeviceGuard guard;
+            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            check(fwp_sum_bwd(qv, kv, vv, gv_, ckpt.data_ptr<float>(),
+                              saved.size() > 4 ? saved[4].data_ptr<float>() : nullptr, gq.data_ptr<float>(),
+                              gk.data_ptr<float>(), gv.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E, (int)M,
+                              chunk, stream_of(Q)),
+                  "fwp_sum_bwd");
+        }
+        return {gq, gk, gv, none, none, none};
+    }
+};
+
+at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
+                           bool exact) {
+    const bool need_grad = at::GradMode::is_enabled() && (Q.requires_grad() || K.requires_grad() || V.requires_grad());
+    return SumFn::apply(Q, K, V, W, exact, need_grad);
+}
+
 at::Tensor fast_weight_delta(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V,
                              const at::Tensor &beta, const at::Tensor &W) {
     // decided here: forward itself runs with gradient mode switched off
@@ -174,5 +250,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     });
     m.def("fast_weight_delta", &fast_weight_delta,
           "out = fast_weight_delta(Q, K, V, beta, W): delta-rule fast weight memory; W is updated in place");
+    m.def("fast_weight_sum", &fast_weight_sum,
+          "out = fast_weight_sum(Q, K, V, W, exact): sum-rule fast weight memory; W is updated in place");
     m.def("set_error_class", &set_error_class, "exception class raised for rejected calls");
 }

@@ -4,7 +4,7 @@ language-modelling and RL copies are identical)."""
 import torch
 
 from . import _lib
-from .fast_weight import _nchunk
+from .fast_weight import _fwp_torch, _nchunk
 
 
 class FastWeightSum(torch.autograd.Function):
@@ -76,4 +76,12 @@ class FastWeightSum(torch.autograd.Function):
         return grad_Q, grad_K, grad_V, None
 
 
-fast_weight_sum = FastWeightSum.apply
+def _native_sum(Q, K, V, W):
+    """The same operator as a C++ autograd function (csrc/fwp_torch.cpp)."""
+    mode = FastWeightSum.state_gradient
+    if mode != "reference" and mode != "exact":
+        raise _lib.FwpError("FastWeightSum.state_gradient must be 'reference' or 'exact'")
+    return _fwp_torch.fast_weight_sum(Q, K, V, W, mode == "exact")
+
+
+fast_weight_sum = _native_sum if _fwp_torch is not None else FastWeightSum.apply

@@ -65,3 +65,26 @@ def test_views_no_grad_and_shape_errors(fwp):
         f(q, k[:, :, :-1], v, beta, W0.clone())
     with pytest.raises(fwp._lib.FwpError, match="W must be"):
         f(q, k, v, beta, W0.clone().transpose(2, 3))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("mode", ["reference", "exact"])
+@pytest.mark.parametrize("N,H,L,E,M", [(2, 2, 64, 16, 16), (3, 5, 11, 18, 7), (1, 2, 130, 32, 32)])
+def test_sum_rule_same_as_python_function(fwp, mode, N, H, L, E, M):
+    q, k, v, _, W0, go = (torch.from_numpy(a).cuda() for a in delta_inputs(7, N, H, L, E, M, dtype=np.float32))
+    assert fwp.fast_weight_sum is not fwp.FastWeightSum.apply
+    fwp.FastWeightSum.state_gradient = mode
+    try:
+        results = []
+        for f in (fwp.fast_weight_sum, fwp.FastWeightSum.apply):
+            ins = [t.clone().requires_grad_(True) for t in (q, k, v)]
+            W = W0.clone()
+            out = f(*ins, W)
+            results.append([out, W, *torch.autograd.grad(out, ins, go)])
+        for a, b in zip(*results):
+            assert torch.equal(a, b)
+        fwp.FastWeightSum.state_gradient = "something else"
+        with pytest.raises(fwp._lib.FwpError, match="state_gradient"):
+            fwp.fast_weight_sum(q, k, v, W0.clone())
+    finally:
+        fwp.FastWeightSum.state_gradient = "reference"
