@@ -21,8 +21,9 @@ def fwp():
 
 @pytest.fixture(params=["scan", "chunked", "split"])
 def delta_kernels(request, fwp):
-    """Both kinds of delta-rule and sum-rule kernels for D = 16/32: the step-by-step scan, the
-    16-step blocks on the matrix cores, and those blocks split over several waves (other shapes take the LDS kernels whatever the setting)."""
+    """The kinds of delta-rule kernels for D = 16/32: the step-by-step scan, 16-step blocks on the
+    matrix cores with one wave per sequence, and those blocks split over several waves.  The sum rule
+    has the first two; other shapes take the LDS kernels whatever the setting."""
     L_ = fwp._lib
     L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT}[request.param])
     yield request.param

@@ -61,3 +61,16 @@ def test_forward_and_backward_of_different_kinds(fwp, fwd_kind, bwd_kind):
     got = run(fwp, arrays, 64, fwd_kind, bwd_kind)
     for name, g, w in zip(("out", "W", "gq", "gk", "gv", "gbeta"), got, want):
         assert within(g, w, ATOL, RTOL), f"{fwd_kind}->{bwd_kind} {name}: max abs err {max_abs(g, w):.3e}"
+
+
+@pytest.mark.parametrize("D", [16, 32])
+def test_long_sequence_kinds_agree(fwp, D):
+    """2048 steps (128 blocks, 32 chunks): the three kernel kinds against the oracle and each other."""
+    N, H, T = 1, 3, 2048
+    arrays = delta_inputs(13, N, H, T, D, D, dtype=np.float32, w0=True)
+    q, k, v, beta, W0, go = (a.astype(np.float64) for a in arrays)
+    want = [*oracle.delta_fwd(q, k, v, beta, W0), *oracle.delta_bwd(q, k, v, beta, W0, go)]
+    for kind in KINDS:
+        got = run(fwp, arrays, 64, kind, kind)
+        for name, g, w in zip(("out", "W", "gq", "gk", "gv", "gbeta"), got, want):
+            assert within(g, w, ATOL, RTOL), f"{kind} {name}: max abs err {max_abs(g, w):.3e}"
