@@ -71,8 +71,9 @@ int fwp_check_device(void);
 
 /*
  * Number of floats the delta rule's `ckpt` buffer must hold (-1 for invalid dimensions):
- * the N*H*nchunk*E*M checkpointed states and, for E = M in {16, 32}, a header and one 16x16
- * matrix per 16 steps that the blocked forward kernel leaves for the blocked backward.
+ * the N*H*nchunk*E*M checkpointed states and, for the state shapes the matrix-core kernels take
+ * (E in {16,32,64,96}, M in {16,32,64}, E/16 + M/16 <= 8), a header and one 16x16 matrix per 16
+ * steps that the blocked forward kernel leaves for the blocked backward.
  * No counterpart in the reference.
  */
 long long fwp_delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);

@@ -33,12 +33,21 @@ bool delta_chunked(int L) {
 
 // Several waves per sequence pay off while they find SIMDs of their own: measured on MI355X
 // (1024 SIMDs) the split kernels win up to about two waves per SIMD and lose beyond.
-bool delta_split(int N, int H, int L, int D, std::initializer_list<fwp_view> views) {
-    if (!split_delta_supported(L)) return false;
-    for (const fwp_view &v : views)      // the split kernels address a sequence with 32-bit byte offsets
-        if (v.sL < 0 || ((int64_t)L * v.sL + D) * 4 >= (int64_t(1) << 31)) return false;
+// Shapes that have no other fast kernel (E != M, E or M above 32) always take them.
+bool delta_split(int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
+                 const fwp_view &beta) {
+    if (!split_delta_supported(L) || !split_delta_dims(E, M)) return false;
+    // a sequence is addressed with 32-bit byte offsets
+    const auto in_range = [&](const fwp_view &v) {
+        return v.sL >= 0 && ((int64_t)L * v.sL + (E > M ? E : M)) * 4 < (int64_t(1) << 31);
+    };
+    if (!in_range(beta)) return false;
+    for (const fwp_view &v : views)      // rows read 16 bytes at a time
+        if (!reg_view_ok(v) || !in_range(v)) return false;
     if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
-    return g_delta_kernels == FWP_DELTA_AUTO && L >= 32 && (int64_t)N * H * (D / 8) <= 2048;
+    if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
+    if (!reg_delta_supported(E, M)) return true;
+    return L >= 32 && (int64_t)N * H * (E / 8) <= 2048;
 }
 
 }  // namespace
@@ -99,19 +108,17 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
-        aligned16(vdiff) && aligned16(ckpt) && aligned16(out)) {
-        if (delta_split(N, H, L, E, {q, k, v, beta}))
-            return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
-                                   (hipStream_t)stream);
+    const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(out);
+    if (aligned && delta_split(N, H, L, E, M, {q, k, v}, beta))
+        return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned) {
         if (delta_chunked(L))
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                                   (hipStream_t)stream);
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                              (hipStream_t)stream);
     }
-    if (reg_delta_supported(E, M))
-        if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, chunk, (hipStream_t)stream)) return rc;
+    if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, M, chunk, (hipStream_t)stream)) return rc;
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
                              (hipStream_t)stream);
 }
@@ -123,11 +130,11 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         !gq || !gk || !gv || !gbeta)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) &&
-        aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv)) {
-        if (delta_split(N, H, L, E, {q, k, beta, grad_out}))
-            return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
-                                   chunk, (hipStream_t)stream);
+    const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv);
+    if (aligned && delta_split(N, H, L, E, M, {q, k, grad_out}, beta))
+        return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
+                               (hipStream_t)stream);
+    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) && aligned) {
         if (delta_chunked(L))
             return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
                                   chunk, (hipStream_t)stream);

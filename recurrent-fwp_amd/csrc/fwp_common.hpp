@@ -74,20 +74,22 @@ int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
 int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
 
-// Size of the delta rule's checkpoint buffer: the states, plus (E = M in {16, 32}) a header and one
+// Size of the delta rule's checkpoint buffer: the states, plus (shapes of the blocked kernels) a header and one
 // 16x16 matrix per 16 steps that the blocked forward leaves for the blocked backward.
 int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);
-int delta_aux_invalidate(float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
-float *delta_aux_of(const float *ckpt, int N, int H, int L, int D, int chunk);
+bool delta_has_aux(int E, int M);
+int delta_aux_invalidate(float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s);
+float *delta_aux_of(const float *ckpt, int N, int H, int L, int E, int M, int chunk);
 
 // The same blocks with the work of a sequence split over several waves of one workgroup (same
 // arguments, results and auxiliary buffer as mfma_delta_fwd / mfma_delta_bwd); whole blocks only.
 bool split_delta_supported(int L);
+bool split_delta_dims(int E, int M);      // E = 16 NE, M = 16 NM for the instantiated (NE, NM)
 int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
-                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
+                    float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s);
 int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                     const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
-                    int L, int D, int chunk, hipStream_t s);
+                    int L, int E, int M, int chunk, hipStream_t s);
 int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                    int L, int D, int chunk, hipStream_t s);

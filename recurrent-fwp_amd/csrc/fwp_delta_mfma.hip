@@ -826,32 +826,35 @@ __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp
 int64_t delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk) {
     const int nchunk = (L + chunk - 1) / chunk;
     int64_t n = (int64_t)N * H * nchunk * E * M;
-    if (reg_delta_supported(E, M)) n += kAuxHeader + (int64_t)N * H * ((L + kBlk - 1) / kBlk) * 256;
+    if (delta_has_aux(E, M)) n += kAuxHeader + (int64_t)N * H * ((L + kBlk - 1) / kBlk) * 256;
     return n;
 }
 
 // The auxiliary part of the checkpoint buffer starts right after the states.
-float *delta_aux_of(const float *ckpt, int N, int H, int L, int D, int chunk) {
+float *delta_aux_of(const float *ckpt, int N, int H, int L, int E, int M, int chunk) {
     if (!ckpt) return nullptr;
     const int nchunk = (L + chunk - 1) / chunk;
-    return const_cast<float *>(ckpt) + (int64_t)N * H * nchunk * D * D;
+    return const_cast<float *>(ckpt) + (int64_t)N * H * nchunk * E * M;
 }
+
+// Shapes whose checkpoint buffer has the auxiliary part: those the blocked kernels take.
+bool delta_has_aux(int E, int M) { return reg_delta_supported(E, M) || split_delta_dims(E, M); }
 
 namespace {
 __global__ void k_store_float(float *dst, float x) { *dst = x; }
 }  // namespace
 
 // Forward kernels that do not leave the per-block matrices say so in the header.
-int delta_aux_invalidate(float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
-    if (!ckpt) return 0;
-    hipLaunchKernelGGL(k_store_float, dim3(1), dim3(1), 0, s, delta_aux_of(ckpt, N, H, L, D, chunk), 0.f);
+int delta_aux_invalidate(float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s) {
+    if (!ckpt || !delta_has_aux(E, M)) return 0;
+    hipLaunchKernelGGL(k_store_float, dim3(1), dim3(1), 0, s, delta_aux_of(ckpt, N, H, L, E, M, chunk), 0.f);
     return (int)hipGetLastError();
 }
 
 int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
+    float *aux = delta_aux_of(ckpt, N, H, L, D, D, chunk);
     if (D == 16)
         hipLaunchKernelGGL(k_delta_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
                            vdiff, ckpt, aux, H, L, chunk, nchunk);
@@ -865,7 +868,7 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                    int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    const float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
+    const float *aux = delta_aux_of(ckpt, N, H, L, D, D, chunk);
     if (D == 16)
         hipLaunchKernelGGL(k_delta_bwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, beta, vdiff, go,
                            ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);

@@ -6,12 +6,13 @@
 // waits for memory; there are fewer sequences than SIMDs, so the spare SIMDs take the part of a
 // block that does not lie on the chain:
 //
-//   forward, D/16 + 1 waves:  wave mb < D/16 owns the state columns [16 mb, 16 mb + 16) and does
+// (the state is E x M, NE = E/16 by NM = M/16 tiles; E and M need not be equal here)
+//   forward, NM + 1 waves:    wave mb < NM owns the state columns [16 mb, 16 mb + 16) and does
 //       the products that need the state (X, U, O, d, S'); the last wave prepares, one block ahead,
 //       what depends on K, Q, beta only: (I + A)^-T, strict_lower(K K^T)^T, lower(Q K^T)^T.
-//   backward, 2 D/16 waves:   wave mb < D/16 ("adjoint") owns the columns of dS and walks the chain
+//   backward, NM + NE waves:  wave mb < NM ("adjoint") owns the columns of dS and walks the chain
 //       dS -> dU -> dY -> dX -> dS, stores g_v, and forms its share of lower(dO U^T) and
-//       strict_lower(dX U^T); wave D/16 + eb ("state"), one block behind, owns rows
+//       strict_lower(dX U^T); wave NM + eb ("state"), one block behind, owns rows
 //       [16 eb, 16 eb + 16) of S, rewinds them and forms g_q, g_k for those columns, and g_beta.
 //
 // Hand-over is through LDS, two slots used alternately, one workgroup barrier per block: every
@@ -119,29 +120,29 @@ __device__ __forceinline__ void ring_loop(int n, Load load, Step step) {
 
 // What the preparing wave reads of a block.
 // Kt[b], Qt[b]: register r = K[t0 + c][16b + 4g + r];  bcol = beta[t0 + c], brow[r] = beta[t0 + 4g + r]
-template <int NB>
+template <int NE>
 struct PrepRaw {
-    v4f Kt[NB], Qt[NB];
+    v4f Kt[NE], Qt[NE];
     float bcol, brow[4];
 };
 
 // What a state wave reads of a block: K and Q whole, its own 16 columns of V.
 // Kc[b], Vc: register r = K[t0 + 4g + r][16b + c]
-template <int NB>
+template <int NE>
 struct MainRaw {
-    v4f Kt[NB], Qt[NB], Kc[NB], Vc;
+    v4f Kt[NE], Qt[NE], Kc[NE], Vc;
     float brow[4];
 };
 
-template <int NB, int PF>   // NB = D / 16, PF = blocks in flight
-__global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
+template <int NE, int NM, int PF>   // E = 16 NE, M = 16 NM, PF = blocks in flight
+__global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
                                                                   fwp_view beta, float *__restrict__ W,
                                                                   float *__restrict__ out,
                                                                   float *__restrict__ vdiff,
                                                                   float *__restrict__ ckpt,
                                                                   float *__restrict__ aux, int H, int L,
                                                                   int chunk, int nchunk) {
-    constexpr int D = 16 * NB;
+    constexpr int E = 16 * NE, M = 16 * NM;
     // slot, matrix (0: (I + A)^-T, 1: strict_lower(K K^T)^T, 2: lower(Q K^T)^T), lane
     __shared__ LdsMat xch[2][3];
     __shared__ LdsMat scratch[2];       // the preparing wave's
@@ -152,9 +153,9 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
     // rows of this sequence; lane offsets and block steps in bytes
-    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + D) * 4)),
-        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + D) * 4)),
-        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + D) * 4)),
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
         bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4));
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4);
@@ -165,7 +166,7 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
     for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
 
-    if (wave == NB) {
+    if (wave == NM) {
         // ------------------------------------------------ preparing wave
         // aux (with ckpt): a header whose first float says that the per-block matrices
         // T = (I + A)^-1 follow, row-major, [sequence][block][16][16]; backward then does not
@@ -176,21 +177,21 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
         v4f ident;
 #pragma unroll
         for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-        auto load = [&](PrepRaw<NB> &w, int ib) {
+        auto load = [&](PrepRaw<NE> &w, int ib) {
             const unsigned ks = ib * k_step, qs = ib * q_step, bs = ib * b_step;
             w.bcol = bb.f(o_bc, bs);
 #pragma unroll
             for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
+            for (int b = 0; b < NE; b++) {
                 w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
                 w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
             }
         };
-        auto prepare = [&](const PrepRaw<NB> &w, int ib) {
+        auto prepare = [&](const PrepRaw<NE> &w, int ib) {
             v4f G = zero, R = zero;
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
+            for (int b = 0; b < NE; b++) {
                 G = tn(w.Kt[b], w.Kt[b], G);       // K K^T
                 R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
             }
@@ -211,15 +212,15 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
                 *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = as_float4(Tt);
         };
         {
-            PrepRaw<NB> first;
+            PrepRaw<NE> first;
             load(first, 0);
             prepare(first, 0);
         }
         lds_barrier();
         // while the state waves do block e: block e + 1 (nothing in the last round)
-        ring_loop<PF, PrepRaw<NB>>(
-            nblk, [&](PrepRaw<NB> &w, int e) { load(w, min(e + 1, nblk - 1)); },
-            [&](int e, const PrepRaw<NB> &w) {
+        ring_loop<PF, PrepRaw<NE>>(
+            nblk, [&](PrepRaw<NE> &w, int e) { load(w, min(e + 1, nblk - 1)); },
+            [&](int e, const PrepRaw<NE> &w) {
                 if (e + 1 < nblk) prepare(w, e + 1);
             });
         return;
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
         o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
         o_vr[r] = (unsigned)((4 * g + r) * v.sL + 16 * mb + c) * 4;
     }
-    auto load = [&](MainRaw<NB> &w, int ib) {
+    auto load = [&](MainRaw<NE> &w, int ib) {
         const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step, bs = ib * b_step;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -241,7 +242,7 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
             w.Vc[r] = vb.f(o_vr[r], vs);
         }
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
+        for (int b = 0; b < NE; b++) {
             w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
             w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
@@ -250,22 +251,22 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
     };
 
     // S[eb]: register r holds S[16 eb + 4g + r][16 mb + c]
-    v4f S[NB];
+    v4f S[NE];
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+        for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
     const ChunkOf chunk_of(chunk);
-    float *out_l = out + seq * L * D + c * D + 16 * mb + 4 * g;                  // + t0 * D
-    float *vd_l = vdiff ? vdiff + seq * L * D + 4 * g * D + 16 * mb + c : nullptr;   // + (t0 + r) * D
+    float *out_l = out + seq * L * M + c * M + 16 * mb + 4 * g;                  // + t0 * M
+    float *vd_l = vdiff ? vdiff + seq * L * M + 4 * g * M + 16 * mb + c : nullptr;   // + (t0 + r) * M
 
-    auto block = [&](int ib, const MainRaw<NB> &cur) {
+    auto block = [&](int ib, const MainRaw<NE> &cur) {
         const LdsMat *slot = xch[ib & 1];
         v4f KS = zero, Ot = zero;
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
+        for (int eb = 0; eb < NE; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
+        for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
         const v4f Tt = slot[0].get(lane);
         const v4f X = cur.Vc - KS;
         v4f Y;
@@ -273,31 +274,31 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
         for (int r = 0; r < 4; r++) Y[r] = cur.brow[r] * X[r];
         const v4f U = tn(Tt, Y, zero);
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
+        for (int eb = 0; eb < NE; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
         const v4f Rm = slot[2].get(lane);
         const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
-        *reinterpret_cast<float4 *>(out_l + (int64_t)ib * kBlk * D) = as_float4(O);
+        *reinterpret_cast<float4 *>(out_l + (int64_t)ib * kBlk * M) = as_float4(O);
         if (vd_l) {
             const v4f Gu = slot[1].get(lane);
             const v4f Dd = X - tn(Gu, U, zero);
 #pragma unroll
-            for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * D] = Dd[r];
+            for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * M] = Dd[r];
         }
         if (ckpt && (chunk_of.closes(ib) || ib + 1 == nblk)) {
-            float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * D * D;
+            float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * E * M;
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++)
+            for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][r];
+                for (int r = 0; r < 4; r++) dst[(16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][r];
         }
     };
 
     lds_barrier();      // the preparing wave's block 0
-    ring_loop<PF, MainRaw<NB>>(nblk, load, block);
+    ring_loop<PF, MainRaw<NE>>(nblk, load, block);
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][r];
+        for (int r = 0; r < 4; r++) W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][r];
 }
 
 // ----------------------------------------------------------------- backward
@@ -316,24 +317,24 @@ __global__ __launch_bounds__(64 * (NB + 1)) void k_delta_fwd_split(fwp_view q, f
 // also transposed, and of g_beta.  The state waves add the shares.  A matrix that is needed
 // transposed is written to LDS transposed instead of being multiplied out a second time.
 
-template <int NB>
+template <int NE>
 struct AdjRaw {
-    v4f Kt[NB], Qt[NB], Kc[NB], Qc[NB];
+    v4f Kt[NE], Qt[NE], Kc[NE], Qc[NE];
     v4f Oc, Ot, Dt;          // upstream gradient and vdiff, the wave's 16 value columns
     v4f T;                   // (I + A)^-1 when forward saved it
     float bcol, brow[4];
 };
 
-template <int NB>
+template <int NM>
 struct StateRaw {
     v4f Kc, Qc;                          // the wave's 16 key columns
-    v4f Ot[NB], Dc[NB], Dt[NB];
-    v4f Sck[NB];                         // checkpointed state of the block's chunk, transposed, rows of the wave
+    v4f Ot[NM], Dc[NM], Dt[NM];
+    v4f Sck[NM];                         // checkpointed state of the block's chunk, transposed, rows of the wave
     float bcol, brow[4];
 };
 
-template <int NB, int PF>
-__global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_view k, fwp_view beta,
+template <int NE, int NM, int PF>
+__global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, fwp_view k, fwp_view beta,
                                                              const float *__restrict__ vdiff, fwp_view go,
                                                              const float *__restrict__ ckpt,
                                                              const float *__restrict__ aux,
@@ -341,13 +342,13 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
                                                              float *__restrict__ gv,
                                                              float *__restrict__ gbeta, int H, int L,
                                                              int chunk, int nchunk) {
-    constexpr int D = 16 * NB;
-    constexpr int kDX = NB, kDPm = NB + 1, kDPmt = NB + 2, kNM = NB + 3, kNMt = NB + 4;
-    // slot, adjoint wave, matrix: blocks eb = 0..NB-1 of dS^T, then dX^T, dPm, dPm^T,
+    constexpr int E = 16 * NE, M = 16 * NM;
+    constexpr int kDX = NE, kDPm = NE + 1, kDPmt = NE + 2, kNM = NE + 3, kNMt = NE + 4;
+    // slot, adjoint wave, matrix: blocks eb = 0..NE-1 of dS^T, then dX^T, dPm, dPm^T,
     // -strict_lower(dX U^T) and its transpose
-    __shared__ LdsMat xch[2][NB][NB + 5];
-    __shared__ LdsMat scratch[NB][2];       // the adjoint waves'
-    __shared__ float gbx[2][NB][16];
+    __shared__ LdsMat xch[2][NM][NE + 5];
+    __shared__ LdsMat scratch[NM][2];       // the adjoint waves'
+    __shared__ float gbx[2][NM][16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -355,14 +356,14 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
     // rows of this sequence; lane offsets and block steps in bytes
-    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + D) * 4)),
-        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + D) * 4)),
-        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + D) * 4)),
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + M) * 4)),
         bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
-        db(vdiff + seq * L * D, (uint32_t)(L * D * 4));
+        db(vdiff + seq * L * M, (uint32_t)(L * M * 4));
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    o_step = (unsigned)(kBlk * go.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
-                   d_step = (unsigned)(kBlk * D * 4);
+                   d_step = (unsigned)(kBlk * M * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     v4f ident;
 #pragma unroll
@@ -373,7 +374,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
 #pragma unroll
     for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
 
-    if (wave < NB) {
+    if (wave < NM) {
         // ------------------------------------------------ adjoint wave of value columns mb
         const int mb = wave;
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4;
         const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
                        o_ot = (unsigned)(c * go.sL + 16 * mb + 4 * g) * 4,
-                       o_dt = (unsigned)(c * D + 16 * mb + 4 * g) * 4;
+                       o_dt = (unsigned)(c * M + 16 * mb + 4 * g) * 4;
         unsigned o_kr[4], o_qr[4], o_or[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -390,7 +391,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
             o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
             o_or[r] = (unsigned)((4 * g + r) * go.sL + 16 * mb + c) * 4;
         }
-        auto load = [&](AdjRaw<NB> &w, int e) {
+        auto load = [&](AdjRaw<NE> &w, int e) {
             const int ib = nblk - 1 - e;
             if (have_T) {
 #pragma unroll
@@ -407,7 +408,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
                 w.Oc[r] = gob.f(o_or[r], os);
             }
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
+            for (int b = 0; b < NE; b++) {
                 w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
                 w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
@@ -419,16 +420,16 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         };
 
         // dS[eb]: register r = dS[16 eb + 4g + r][16 mb + c]
-        v4f dS[NB];
+        v4f dS[NE];
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) dS[eb] = zero;
-        float *gv_l = gv + seq * L * D + c * D + 16 * mb + 4 * g;       // + t0 * D
-        auto block = [&](int e, const AdjRaw<NB> &w) {
+        for (int eb = 0; eb < NE; eb++) dS[eb] = zero;
+        float *gv_l = gv + seq * L * M + c * M + 16 * mb + 4 * g;       // + t0 * M
+        auto block = [&](int e, const AdjRaw<NE> &w) {
             const int ib = nblk - 1 - e;
             LdsMat *slot = xch[ib & 1][mb];
             v4f QK = zero;
 #pragma unroll
-            for (int b = 0; b < NB; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
+            for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
             v4f Pm;
 #pragma unroll
             for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
@@ -436,7 +437,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
             if (!have_T) {
                 v4f G = zero, A, At;
 #pragma unroll
-                for (int b = 0; b < NB; b++) G = tn(w.Kt[b], w.Kt[b], G);
+                for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
@@ -446,17 +447,17 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
             }
             const v4f Ut = w.bcol * w.Dt;
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) slot[eb].put_t(p, dS[eb]);
+            for (int eb = 0; eb < NE; eb++) slot[eb].put_t(p, dS[eb]);
             v4f dU = tn(Pm, w.Oc, zero);
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) dU = tn(w.Kt[eb], dS[eb], dU);
+            for (int eb = 0; eb < NE; eb++) dU = tn(w.Kt[eb], dS[eb], dU);
             const v4f dY = tn(T, dU, zero);
             scratch[mb][0].put_t(p, dY);
             v4f ndX;
 #pragma unroll
             for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) {
+            for (int eb = 0; eb < NE; eb++) {
                 dS[eb] = tn(w.Qc[eb], w.Oc, dS[eb]);
                 dS[eb] = tn(w.Kc[eb], ndX, dS[eb]);
             }
@@ -468,7 +469,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
 #pragma unroll
             for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
             // register r = g_v[t0 + c][16 mb + 4g + r]
-            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * D) = as_float4(dXt);
+            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * M) = as_float4(dXt);
             slot[kDX].put(lane, dXt);
             const v4f M = tn(dXt, Ut, zero);       // dX U^T
             {   // share of g_beta[t0 + c]: the four 16-lane rows hold partial sums
@@ -491,30 +492,30 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
             slot[kNM].put(lane, nM);
             slot[kNMt].put_t(p, nM);
         };
-        ring_loop<PF, AdjRaw<NB>>(nblk, load, block);
+        ring_loop<PF, AdjRaw<NE>>(nblk, load, block);
         lds_barrier();        // the state waves' last block
         return;
     }
 
     // ---------------------------------------------------- state wave of key columns [16 eb, 16 eb + 16)
-    const int eb = wave - NB;
-    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * D + 4 * g) * 4;
+    const int eb = wave - NM;
+    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4;
     unsigned o_kr[4], o_qr[4], o_dr[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         o_kr[r] = (unsigned)((4 * g + r) * k.sL + 16 * eb + c) * 4;
         o_qr[r] = (unsigned)((4 * g + r) * q.sL + 16 * eb + c) * 4;
-        o_dr[r] = (unsigned)((4 * g + r) * D + c) * 4;
+        o_dr[r] = (unsigned)((4 * g + r) * M + c) * 4;
     }
-    const RowBuf cb(ckpt + seq * nchunk * D * D, (uint32_t)(nchunk * D * D * 4));
-    const unsigned o_ck = (unsigned)((16 * eb + c) * D + 4 * g) * 4;
+    const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4));
+    const unsigned o_ck = (unsigned)((16 * eb + c) * M + 4 * g) * 4;
     const ChunkOf chunk_of(chunk);
-    auto load = [&](StateRaw<NB> &w, int e) {
+    auto load = [&](StateRaw<NM> &w, int e) {
         const int ib = nblk - 1 - e;
         {   // always loaded, so that no load is left to be issued (and waited for) inside the block
-            const unsigned cs = chunk_of(ib) * (D * D * 4);
+            const unsigned cs = chunk_of(ib) * (E * M * 4);
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) w.Sck[mb] = cb.f4(o_ck + 64 * mb, cs);
+            for (int mb = 0; mb < NM; mb++) w.Sck[mb] = cb.f4(o_ck + 64 * mb, cs);
         }
         const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
                        bs = ib * b_step;
@@ -526,7 +527,7 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
             w.Qc[r] = qb.f(o_qr[r], qs);
         }
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
+        for (int b = 0; b < NM; b++) {
             w.Ot[b] = gob.f4(o_ot + 64 * b, os);
             w.Dt[b] = db.f4(o_dt + 64 * b, ds);
 #pragma unroll
@@ -535,19 +536,19 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
     };
 
     // St[mb]: register r = S[16 eb + c][16 mb + 4g + r]  (block (mb, eb) of S^T)
-    v4f St[NB];
-    float *gq_l = gq + seq * L * D + c * D + 16 * eb + 4 * g, *gk_l = gk + seq * L * D + c * D + 16 * eb + 4 * g;
+    v4f St[NM];
+    float *gq_l = gq + seq * L * E + c * E + 16 * eb + 4 * g, *gk_l = gk + seq * L * E + c * E + 16 * eb + 4 * g;
     float *gb_l = gbeta + seq * L + c;
-    auto block = [&](int e, const StateRaw<NB> &w) {
+    auto block = [&](int e, const StateRaw<NM> &w) {
         const int ib = nblk - 1 - e;
         if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) St[mb] = w.Sck[mb];
+            for (int mb = 0; mb < NM; mb++) St[mb] = w.Sck[mb];
         }
         // state at the start of the block, transposed: S0^T = S'^T - U^T K
-        v4f Ut[NB];
+        v4f Ut[NM];
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
             Ut[mb] = w.bcol * w.Dt[mb];
             v4f nU;
 #pragma unroll
@@ -556,12 +557,12 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         }
         v4f gQt = zero, gKt = zero;
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) gQt = tn(St[mb], w.Ot[mb], gQt);
+        for (int mb = 0; mb < NM; mb++) gQt = tn(St[mb], w.Ot[mb], gQt);
         // what the adjoint waves left for this block
         v4f dPm = zero, dPmt = zero, nMs = zero;
         float gb = 0.f;
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
             const LdsMat *slot = xch[ib & 1][mb];
             dPm += slot[kDPm].get(lane);
             dPmt += slot[kDPmt].get(lane);
@@ -575,43 +576,71 @@ __global__ __launch_bounds__(128 * NB) void k_delta_bwd_split(fwp_view q, fwp_vi
         gKt = tn(w.Qc, dPm, gKt);
         gKt = tn(w.Kc, nMs, gKt);
         // register r = gradient[t0 + c][16 eb + 4g + r]
-        *reinterpret_cast<float4 *>(gq_l + (int64_t)ib * kBlk * D) = as_float4(gQt);
-        *reinterpret_cast<float4 *>(gk_l + (int64_t)ib * kBlk * D) = as_float4(gKt);
+        *reinterpret_cast<float4 *>(gq_l + (int64_t)ib * kBlk * E) = as_float4(gQt);
+        *reinterpret_cast<float4 *>(gk_l + (int64_t)ib * kBlk * E) = as_float4(gKt);
         if (eb == 0 && g == 0) gb_l[ib * kBlk] = gb;
     };
 
     lds_barrier();            // the adjoint waves' first block
-    ring_loop<PF, StateRaw<NB>>(nblk, load, block);
+    ring_loop<PF, StateRaw<NM>>(nblk, load, block);
 }
 
 }  // namespace
 
+// Supported state shapes: E = 16 NE, M = 16 NM with NE in {1, 2, 4, 6}, NM in {1, 2, 4} and at most
+// eight waves (two per SIMD) in the backward workgroup.
+bool split_delta_dims(int E, int M) {
+    const int ne = E / 16, nm = M / 16;
+    return E % 16 == 0 && M % 16 == 0 && (ne == 1 || ne == 2 || ne == 4 || ne == 6) &&
+           (nm == 1 || nm == 2 || nm == 4) && ne + nm <= 8;
+}
+
 bool split_delta_supported(int L) { return L >= kBlk && L % kBlk == 0; }
 
+namespace {
+constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }
+constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
+
+template <int NE, int NM>
+void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
+                float *ckpt, float *aux, int nseq, int H, int L, int chunk, int nchunk, hipStream_t s) {
+    hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE)>), dim3(nseq), dim3(64 * (NM + 1)), 0, s, q, k, v,
+                       beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+}
+template <int NE, int NM>
+void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go, const float *ckpt,
+                const float *aux, float *gq, float *gk, float *gv, float *gbeta, int nseq, int H, int L,
+                int chunk, int nchunk, hipStream_t s) {
+    hipLaunchKernelGGL((k_delta_bwd_split<NE, NM, bwd_ring(NE)>), dim3(nseq), dim3(64 * (NE + NM)), 0, s, q, k,
+                       beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+}
+}  // namespace
+
+// the (NE, NM) pairs of split_delta_dims
+#define FWP_SPLIT_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2)
+
 int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
-                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
+                    float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
-    if (D == 16)
-        hipLaunchKernelGGL((k_delta_fwd_split<1, 4>), dim3(N * H), dim3(128), 0, s, q, k, v, beta, W,
-                           out, vdiff, ckpt, aux, H, L, chunk, nchunk);
-    else
-        hipLaunchKernelGGL((k_delta_fwd_split<2, 4>), dim3(N * H), dim3(192), 0, s, q, k, v, beta, W,
-                           out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+    float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
+#define X(ne, nm)                                                                                        \
+    if (E == 16 * ne && M == 16 * nm)                                                                    \
+        launch_fwd<ne, nm>(q, k, v, beta, W, out, vdiff, ckpt, aux, N * H, H, L, chunk, nchunk, s);
+    FWP_SPLIT_SHAPES(X)
+#undef X
     return (int)hipGetLastError();
 }
 
 int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                     const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
-                    int L, int D, int chunk, hipStream_t s) {
+                    int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    const float *aux = delta_aux_of(ckpt, N, H, L, D, chunk);
-    if (D == 16)
-        hipLaunchKernelGGL((k_delta_bwd_split<1, 3>), dim3(N * H), dim3(128), 0, s, q, k, beta, vdiff,
-                           go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
-    else
-        hipLaunchKernelGGL((k_delta_bwd_split<2, 3>), dim3(N * H), dim3(256), 0, s, q, k, beta, vdiff,
-                           go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
+    const float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
+#define X(ne, nm)                                                                                        \
+    if (E == 16 * ne && M == 16 * nm)                                                                    \
+        launch_bwd<ne, nm>(q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, N * H, H, L, chunk, nchunk, s);
+    FWP_SPLIT_SHAPES(X)
+#undef X
     return (int)hipGetLastError();
 }
 

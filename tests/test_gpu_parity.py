@@ -54,6 +54,54 @@ def test_delta(fwp, delta_kernels, N, H, L, E, M, w0):
     check("W after backward", W, ref_W)     # backward does not rewind the caller's state
 
 
+# every state shape E x M (multiples of 16) that the kernels with several waves per sequence are built for
+RECTANGULAR = [(16, 16), (16, 32), (16, 64), (32, 16), (32, 32), (32, 64), (64, 16), (64, 32), (64, 64),
+               (96, 16), (96, 32)]
+
+
+@pytest.mark.parametrize("E,M", RECTANGULAR)
+@pytest.mark.parametrize("L", [16, 80])
+def test_delta_rectangular_states(fwp, E, M, L):
+    """E != M and D = 64 (feature maps that widen the keys, values wider than keys): whole blocks go to
+    the matrix-core kernels, other lengths (checked once below) to the LDS kernels."""
+    N, H = 2, 3
+    q, k, v, beta, W0, go = delta_inputs(700 + E + M + L, N, H, L, E, M, w0=True)
+    tq, tk, tv, tb = (dev(x, True) for x in (q, k, v, beta))
+    W = dev(W0)
+    out = fwp.fast_weight_delta(tq, tk, tv, tb, W)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("q k v beta".split(), (tq, tk, tv, tb), oracle.delta_bwd(q, k, v, beta, W0, go)):
+        check("grad_" + name, t.grad, r)
+
+
+def test_delta_rectangular_states_views_and_segments(fwp):
+    # permuted views of [L,N,H,*] storage, a carried state over two segments (80 = 48 + 32), E = 96, M = 16
+    N, H, L, E, M = 2, 2, 80, 96, 16
+    q, k, v, beta, W0, go = delta_inputs(77, N, H, L, E, M, w0=True)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    ref_g = oracle.delta_bwd(q, k, v, beta, W0, go)
+    lead = [dev(np.ascontiguousarray(np.transpose(x, (2, 0, 1, 3))), True) for x in (q, k, v, beta)]
+    tq, tk, tv, tb = (t.permute(1, 2, 0, 3) for t in lead)
+    W = dev(W0)
+    outs = []
+    for a, b in ((0, 48), (48, 80)):
+        outs.append(fwp.fast_weight_delta(tq[:, :, a:b], tk[:, :, a:b], tv[:, :, a:b], tb[:, :, a:b], W))
+        W = W.clone()           # the state an earlier segment's backward reads must stay as it was
+    out = torch.cat(outs, 2)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    # gradients of the two segments on their own (the state is not differentiated through, as in the reference)
+    out.backward(dev(go))
+    first = oracle.delta_bwd(q[:, :, :48], k[:, :, :48], v[:, :, :48], beta[:, :, :48], W0, go[:, :, :48])
+    mid_W = oracle.delta_fwd(q[:, :, :48], k[:, :, :48], v[:, :, :48], beta[:, :, :48], W0)[1]
+    second = oracle.delta_bwd(q[:, :, 48:], k[:, :, 48:], v[:, :, 48:], beta[:, :, 48:], mid_W, go[:, :, 48:])
+    for name, t, a, b in zip("q k v beta".split(), lead, first, second):
+        check("grad_" + name, t.grad.permute(1, 2, 0, 3), np.concatenate((a, b), 2))
+
+
 @pytest.mark.parametrize("L", [15, 16, 17, 31, 33, 47, 48, 100])
 @pytest.mark.parametrize("D", [16, 32])
 def test_delta_block_edges(fwp, delta_kernels, L, D):
