@@ -82,7 +82,7 @@ int delta_aux_invalidate(float *ckpt, int N, int H, int L, int E, int M, int chu
 float *delta_aux_of(const float *ckpt, int N, int H, int L, int E, int M, int chunk);
 
 // The same blocks with the work of a sequence split over several waves of one workgroup (same
-// arguments, results and auxiliary buffer as mfma_delta_fwd / mfma_delta_bwd); whole blocks only.
+// arguments, results and auxiliary buffer as mfma_delta_fwd / mfma_delta_bwd).
 bool split_delta_supported(int L);
 bool split_delta_dims(int E, int M);      // E = 16 NE, M = 16 NM for the instantiated (NE, NM)
 int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,

@@ -16,8 +16,10 @@
 //       [16 eb, 16 eb + 16) of S, rewinds them and forms g_q, g_k for those columns, and g_beta.
 //
 // Hand-over is through LDS, two slots used alternately, one workgroup barrier per block: every
-// wave executes the same number of barriers whatever its role.  Sequence lengths are multiples of
-// 16 here (the host sends other lengths to the one-wave kernels), so the loops are straight-line.
+// wave executes the same number of barriers whatever its role.  A last block of fewer than 16 steps
+// needs no code of its own: every tensor is read and written through a buffer resource of exactly
+// the sequence's size, so its missing rows read as zeros (beta = 0: nothing is written to the
+// state; zero upstream gradient) and stores to them are dropped; the loops stay straight-line.
 #include "fwp_common.hpp"
 #include "fwp_wave.hpp"
 #include "fwp_mfma.hpp"
@@ -160,7 +162,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    const int nblk = L / kBlk;
+    const int nblk = (L + kBlk - 1) / kBlk;
     const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4;
     unsigned o_br[4];
 #pragma unroll
@@ -257,8 +259,9 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
         for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
     const ChunkOf chunk_of(chunk);
-    float *out_l = out + seq * L * M + c * M + 16 * mb + 4 * g;                  // + t0 * M
-    float *vd_l = vdiff ? vdiff + seq * L * M + 4 * g * M + 16 * mb + c : nullptr;   // + (t0 + r) * M
+    const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4)), db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0);
+    const unsigned o_out = (unsigned)(c * M + 16 * mb + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + 16 * mb + c) * 4;
+    const unsigned m_step = (unsigned)(kBlk * M * 4);
 
     auto block = [&](int ib, const MainRaw<NE> &cur) {
         const LdsMat *slot = xch[ib & 1];
@@ -277,12 +280,12 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         for (int eb = 0; eb < NE; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
         const v4f Rm = slot[2].get(lane);
         const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
-        *reinterpret_cast<float4 *>(out_l + (int64_t)ib * kBlk * M) = as_float4(O);
-        if (vd_l) {
+        ob.st4(O, o_out, ib * m_step);
+        if (vdiff) {
             const v4f Gu = slot[1].get(lane);
             const v4f Dd = X - tn(Gu, U, zero);
 #pragma unroll
-            for (int r = 0; r < 4; r++) vd_l[((int64_t)ib * kBlk + r) * M] = Dd[r];
+            for (int r = 0; r < 4; r++) db.st(Dd[r], o_vd + r * M * 4, ib * m_step);
         }
         if (ckpt && (chunk_of.closes(ib) || ib + 1 == nblk)) {
             float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * E * M;
@@ -368,7 +371,7 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
     v4f ident;
 #pragma unroll
     for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-    const int nblk = L / kBlk;
+    const int nblk = (L + kBlk - 1) / kBlk;
     const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
     unsigned o_br[4];
 #pragma unroll
@@ -423,7 +426,8 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
         v4f dS[NE];
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) dS[eb] = zero;
-        float *gv_l = gv + seq * L * M + c * M + 16 * mb + 4 * g;       // + t0 * M
+        const RowBuf gvb(gv + seq * L * M, (uint32_t)(L * M * 4));
+        const unsigned o_gv = (unsigned)(c * M + 16 * mb + 4 * g) * 4;
         auto block = [&](int e, const AdjRaw<NE> &w) {
             const int ib = nblk - 1 - e;
             LdsMat *slot = xch[ib & 1][mb];
@@ -469,7 +473,7 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
 #pragma unroll
             for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
             // register r = g_v[t0 + c][16 mb + 4g + r]
-            *reinterpret_cast<float4 *>(gv_l + (int64_t)ib * kBlk * M) = as_float4(dXt);
+            gvb.st4(dXt, o_gv, ib * d_step);
             slot[kDX].put(lane, dXt);
             const v4f M = tn(dXt, Ut, zero);       // dX U^T
             {   // share of g_beta[t0 + c]: the four 16-lane rows hold partial sums
@@ -537,8 +541,9 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
 
     // St[mb]: register r = S[16 eb + c][16 mb + 4g + r]  (block (mb, eb) of S^T)
     v4f St[NM];
-    float *gq_l = gq + seq * L * E + c * E + 16 * eb + 4 * g, *gk_l = gk + seq * L * E + c * E + 16 * eb + 4 * g;
-    float *gb_l = gbeta + seq * L + c;
+    const RowBuf gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
+        gbb(gbeta + seq * L, (uint32_t)(L * 4));
+    const unsigned o_g = (unsigned)(c * E + 16 * eb + 4 * g) * 4, e_step = (unsigned)(kBlk * E * 4);
     auto block = [&](int e, const StateRaw<NM> &w) {
         const int ib = nblk - 1 - e;
         if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
@@ -576,9 +581,9 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
         gKt = tn(w.Qc, dPm, gKt);
         gKt = tn(w.Kc, nMs, gKt);
         // register r = gradient[t0 + c][16 eb + 4g + r]
-        *reinterpret_cast<float4 *>(gq_l + (int64_t)ib * kBlk * E) = as_float4(gQt);
-        *reinterpret_cast<float4 *>(gk_l + (int64_t)ib * kBlk * E) = as_float4(gKt);
-        if (eb == 0 && g == 0) gb_l[ib * kBlk] = gb;
+        gqb.st4(gQt, o_g, ib * e_step);
+        gkb.st4(gKt, o_g, ib * e_step);
+        if (eb == 0 && g == 0) gbb.st(gb, c * 4, ib * kBlk * 4);
     };
 
     lds_barrier();            // the adjoint waves' first block
@@ -595,7 +600,7 @@ bool split_delta_dims(int E, int M) {
            (nm == 1 || nm == 2 || nm == 4) && ne + nm <= 8;
 }
 
-bool split_delta_supported(int L) { return L >= kBlk && L % kBlk == 0; }
+bool split_delta_supported(int L) { return L >= 1; }
 
 namespace {
 constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }

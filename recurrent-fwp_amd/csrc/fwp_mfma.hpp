@@ -55,11 +55,15 @@ struct Geo16 {
 typedef int v4i __attribute__((ext_vector_type(4)));
 __device__ float llvm_raw_buffer_load_f32(v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.f32");
 __device__ v4f llvm_raw_buffer_load_v4f32(v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.load.v4f32");
+__device__ void llvm_raw_buffer_store_f32(float x, v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.f32");
+__device__ void llvm_raw_buffer_store_v4f32(v4f x, v4i rsrc, int voffset, int soffset, int aux) __asm("llvm.amdgcn.raw.buffer.store.v4f32");
 
-// Read access to one sequence's rows of a tensor through a buffer resource: the address of a load
+// Access to one sequence's rows of a tensor through a buffer resource: the address of a load or store
 // is (descriptor base) + (32-bit byte offset per lane, VGPR) + (byte offset per block, SGPR) +
 // (immediate), so moving on to the next block costs one scalar multiply and no vector address
-// arithmetic.  All offsets stay below 2^31 (checked on the host).
+// arithmetic.  All offsets stay below 2^31 (checked on the host).  The hardware checks the sum of
+// the three offsets against the size: loads beyond it return 0 and stores beyond it are dropped,
+// which is how the rows of a last, partial block of 16 steps are dealt with.
 struct RowBuf {
     v4i rsrc;       // base address (48 bits, stride 0), size in bytes, 32-bit data format
     __device__ __forceinline__ RowBuf(const float *base, uint32_t bytes) {
@@ -71,6 +75,12 @@ struct RowBuf {
     }
     __device__ __forceinline__ v4f f4(unsigned lane_bytes, unsigned block_bytes) const {
         return llvm_raw_buffer_load_v4f32(rsrc, (int)lane_bytes, (int)block_bytes, 0);
+    }
+    __device__ __forceinline__ void st(float x, unsigned lane_bytes, unsigned block_bytes) const {
+        llvm_raw_buffer_store_f32(x, rsrc, (int)lane_bytes, (int)block_bytes, 0);
+    }
+    __device__ __forceinline__ void st4(const v4f &x, unsigned lane_bytes, unsigned block_bytes) const {
+        llvm_raw_buffer_store_v4f32(x, rsrc, (int)lane_bytes, (int)block_bytes, 0);
     }
 };
 
