@@ -149,10 +149,11 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
                 int L, int E, int M, int chunk, void *stream) {
     if (bad_view(q) || bad_view(k) || bad_view(v) || !W || !out) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
-        aligned16(ckpt) && aligned16(out)) {
-        if (delta_chunked(L))
-            return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+    if (split_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
+        aligned16(out)) {
+        // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
+        if (!reg_delta_supported(E, M) || delta_chunked(L))
+            return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
     }
     return generic_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
@@ -164,11 +165,11 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(grad_out) || !ckpt || !gq || !gk || !gv)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
+    if (split_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
-        if (delta_chunked(L))
-            return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
+        if (!reg_delta_supported(E, M) || delta_chunked(L))
+            return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
                                 (hipStream_t)stream);
         return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
                            (hipStream_t)stream);

@@ -95,9 +95,9 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
                    int L, int D, int chunk, hipStream_t s);
 
 int mfma_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
-                 int L, int D, int chunk, hipStream_t s);
+                 int L, int E, int M, int chunk, hipStream_t s);
 int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
-                 const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int D,
+                 const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E, int M,
                  int chunk, hipStream_t s);
 
 // Sum rule on the same kernels (no v_old, beta = 1).

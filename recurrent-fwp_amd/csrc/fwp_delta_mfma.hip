@@ -632,28 +632,28 @@ struct BothWays {
     }
 };
 
-template <int NB>
+template <int NE, int NM>   // state E = 16 NE by M = 16 NM
 __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
                                                      float *__restrict__ W, float *__restrict__ out,
                                                      float *__restrict__ ckpt, int H, int L, int chunk,
                                                      int nchunk) {
-    constexpr int D = 16 * NB;
+    constexpr int E = 16 * NE, M = 16 * NM;
     const Geo16 p(threadIdx.x);
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
     const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f S[NB][NB];
+    v4f S[NE][NM];
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++)
+        for (int mb = 0; mb < NM; mb++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                S[eb][mb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+                S[eb][mb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
 
-    struct Raw { BothWays<NB> K, Q, V; };
+    struct Raw { BothWays<NE> K, Q; BothWays<NM> V; };
     auto load = [&](Raw &w, int t0) {
         w.K.load(kb, k.sL, t0, L, p, true);       // zero rows beyond L: they then write nothing
         w.Q.load(qb, q.sL, t0, L, p, false);
@@ -668,52 +668,52 @@ __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp
         __builtin_amdgcn_sched_barrier(0);
         v4f R = zero;
 #pragma unroll
-        for (int b = 0; b < NB; b++) R = tn(cur.K.t[b], cur.Q.t[b], R);      // K Q^T [s][t]
+        for (int b = 0; b < NE; b++) R = tn(cur.K.t[b], cur.Q.t[b], R);      // K Q^T [s][t]
 #pragma unroll
         for (int r = 0; r < 4; r++) R[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;   // lower(Q K^T)^T
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
             v4f Ot = tn(cur.V.c[mb], R, zero);
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) Ot = tn(S[eb][mb], cur.Q.t[eb], Ot);
+            for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb][mb], cur.Q.t[eb], Ot);
             if (t0 + c < L)
-                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * M + 16 * mb + 4 * g) =
                     make_float4(Ot[0], Ot[1], Ot[2], Ot[3]);
         }
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++)
+        for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) S[eb][mb] = tn(cur.K.c[eb], cur.V.c[mb], S[eb][mb]);
+            for (int mb = 0; mb < NM; mb++) S[eb][mb] = tn(cur.K.c[eb], cur.V.c[mb], S[eb][mb]);
         const int t_end = min(t0 + kBlk, L);
         if (ckpt && (t_end % chunk == 0 || t_end == L)) {
-            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * E * M;
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++)
+            for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-                for (int mb = 0; mb < NB; mb++)
+                for (int mb = 0; mb < NM; mb++)
 #pragma unroll
                     for (int r = 0; r < 4; r++)
-                        dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+                        dst[(16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
         }
         cur = nxt;
     }
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++)
+        for (int mb = 0; mb < NM; mb++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+                W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
 }
 
-template <int NB>
+template <int NE, int NM>   // state E = 16 NE by M = 16 NM
 __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp_view v, fwp_view go,
                                                      const float *__restrict__ ckpt,
                                                      const float *__restrict__ W_init,
                                                      float *__restrict__ gq, float *__restrict__ gk,
                                                      float *__restrict__ gv, int H, int L, int chunk,
                                                      int nchunk) {
-    constexpr int D = 16 * NB;
+    constexpr int E = 16 * NE, M = 16 * NM;
     const Geo16 p(threadIdx.x);
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
@@ -725,17 +725,17 @@ __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp
 #pragma unroll
     for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
 
-    struct Raw { BothWays<NB> K, Q, V, O; v4f Sck[NB][NB]; };
+    struct Raw { BothWays<NE> K, Q; BothWays<NM> V, O; v4f Sck[NM][NE]; };
     auto load = [&](Raw &w, int t0) {
-        const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * D * D;
+        const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * E * M;
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++)
+        for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) {     // block (mb, eb) of S^T, minus the carried-in state if asked
-                const int64_t o = (16 * eb + c) * D + 16 * mb + 4 * g;
+            for (int eb = 0; eb < NE; eb++) {     // block (mb, eb) of S^T, minus the carried-in state if asked
+                const int64_t o = (16 * eb + c) * M + 16 * mb + 4 * g;
                 float4 x = *reinterpret_cast<const float4 *>(src + o);
                 if (W_init) {
-                    const float4 y = *reinterpret_cast<const float4 *>(W_init + seq * D * D + o);
+                    const float4 y = *reinterpret_cast<const float4 *>(W_init + seq * E * M + o);
                     x = make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w);
                 }
                 w.Sck[mb][eb] = v4f{x.x, x.y, x.z, x.w};
@@ -746,11 +746,11 @@ __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp
         w.O.load(gob, go.sL, t0, L, p, true);     // and carry no gradient
     };
 
-    v4f St[NB][NB], dS[NB][NB];
+    v4f St[NM][NE], dS[NE][NM];
 #pragma unroll
-    for (int a = 0; a < NB; a++)
+    for (int a = 0; a < NE; a++)
 #pragma unroll
-        for (int b = 0; b < NB; b++) dS[a][b] = zero;
+        for (int b = 0; b < NM; b++) dS[a][b] = zero;
 
     const int nblk = (L + kBlk - 1) / kBlk;
     Raw cur, nxt;
@@ -762,21 +762,22 @@ __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp
         const int t_end = min(t0 + kBlk, L);
         if (t_end % chunk == 0 || t_end == L) {
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++)
+            for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-                for (int eb = 0; eb < NB; eb++) St[mb][eb] = cur.Sck[mb][eb];
+                for (int eb = 0; eb < NE; eb++) St[mb][eb] = cur.Sck[mb][eb];
         }
         // state before the block, transposed: S0^T = S'^T - V^T K
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
             const v4f nV = -cur.V.c[mb];
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) St[mb][eb] = tn(nV, cur.K.c[eb], St[mb][eb]);
+            for (int eb = 0; eb < NE; eb++) St[mb][eb] = tn(nV, cur.K.c[eb], St[mb][eb]);
         }
         v4f QK = zero, Z = zero, Zt = zero;
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            QK = tn(cur.Q.t[b], cur.K.t[b], QK);          // Q K^T   [t][s]
+        for (int b = 0; b < NE; b++) QK = tn(cur.Q.t[b], cur.K.t[b], QK);          // Q K^T   [t][s]
+#pragma unroll
+        for (int b = 0; b < NM; b++) {
             Z = tn(cur.O.t[b], cur.V.t[b], Z);            // dO V^T  [t][s]
             Zt = tn(cur.V.t[b], cur.O.t[b], Zt);
         }
@@ -790,33 +791,33 @@ __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp
         }
         const bool col_ok = t0 + c < L;
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {        // g_v^T = dS^T K^T + dO^T Pm
+        for (int mb = 0; mb < NM; mb++) {        // g_v^T = dS^T K^T + dO^T Pm
             v4f gVt = tn(cur.O.c[mb], Pm, zero);
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) gVt = tn(dS[eb][mb], cur.K.t[eb], gVt);
+            for (int eb = 0; eb < NE; eb++) gVt = tn(dS[eb][mb], cur.K.t[eb], gVt);
             if (col_ok)
-                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
+                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * M + 16 * mb + 4 * g) =
                     make_float4(gVt[0], gVt[1], gVt[2], gVt[3]);
         }
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) {
+        for (int eb = 0; eb < NE; eb++) {
             v4f gQt = tn(cur.K.c[eb], dPmt, zero);
             v4f gKt = tn(cur.Q.c[eb], dPm, zero);
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) {
+            for (int mb = 0; mb < NM; mb++) {
                 gQt = tn(St[mb][eb], cur.O.t[mb], gQt);
                 gKt = tn(tn(dS[eb][mb], ident, zero), cur.V.t[mb], gKt);      // dS V^T
             }
             if (col_ok) {
-                const int64_t o = (seq * L + t0 + c) * D + 16 * eb + 4 * g;
+                const int64_t o = (seq * L + t0 + c) * E + 16 * eb + 4 * g;
                 *reinterpret_cast<float4 *>(gq + o) = make_float4(gQt[0], gQt[1], gQt[2], gQt[3]);
                 *reinterpret_cast<float4 *>(gk + o) = make_float4(gKt[0], gKt[1], gKt[2], gKt[3]);
             }
         }
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++)
+        for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) dS[eb][mb] = tn(cur.Q.c[eb], cur.O.c[mb], dS[eb][mb]);
+            for (int mb = 0; mb < NM; mb++) dS[eb][mb] = tn(cur.Q.c[eb], cur.O.c[mb], dS[eb][mb]);
         cur = nxt;
     }
 }
@@ -878,28 +879,31 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
     return (int)hipGetLastError();
 }
 
+// the state shapes the blocked sum-rule kernels are instantiated for (those of the split delta kernels)
+#define FWP_SUM_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2)
+
 int mfma_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
-                 int L, int D, int chunk, hipStream_t s) {
+                 int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    if (D == 16)
-        hipLaunchKernelGGL(k_sum_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, W, out, ckpt, H, L,
+#define X(ne, nm)                                                                                          \
+    if (E == 16 * ne && M == 16 * nm)                                                                      \
+        hipLaunchKernelGGL((k_sum_fwd_mfma<ne, nm>), dim3(N * H), dim3(64), 0, s, q, k, v, W, out, ckpt, H, L, \
                            chunk, nchunk);
-    else
-        hipLaunchKernelGGL(k_sum_fwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, W, out, ckpt, H, L,
-                           chunk, nchunk);
+    FWP_SUM_SHAPES(X)
+#undef X
     return (int)hipGetLastError();
 }
 
 int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
-                 const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int D,
+                 const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E, int M,
                  int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
-    if (D == 16)
-        hipLaunchKernelGGL(k_sum_bwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, go, ckpt, W_init, gq,
-                           gk, gv, H, L, chunk, nchunk);
-    else
-        hipLaunchKernelGGL(k_sum_bwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, go, ckpt, W_init, gq,
-                           gk, gv, H, L, chunk, nchunk);
+#define X(ne, nm)                                                                                          \
+    if (E == 16 * ne && M == 16 * nm)                                                                      \
+        hipLaunchKernelGGL((k_sum_bwd_mfma<ne, nm>), dim3(N * H), dim3(64), 0, s, q, k, v, go, ckpt, W_init, \
+                           gq, gk, gv, H, L, chunk, nchunk);
+    FWP_SUM_SHAPES(X)
+#undef X
     return (int)hipGetLastError();
 }
 

@@ -43,6 +43,16 @@ SHAPES = [
     (2, 2, 40, 32, 128, True),    # fast-net layers: d_head x fast_ff_d_head and back
     (2, 2, 40, 128, 32, False),
     (1, 1, 20, 5, 3, True),
+    # rectangular and larger states on the matrix cores (feature maps that widen the keys; d_head 64)
+    (2, 2, 40, 96, 16, True),
+    (1, 2, 48, 64, 64, True),
+    (2, 1, 37, 16, 64, False),
+    (1, 2, 64, 64, 32, True),
+    (1, 1, 33, 32, 64, True),
+    (1, 2, 20, 96, 32, False),
+    (1, 2, 50, 64, 16, True),
+    (1, 1, 17, 16, 32, True),
+    (1, 1, 31, 32, 16, False),
 ]
 
 
