@@ -31,8 +31,9 @@ bool delta_chunked(int L) {
     return g_delta_kernels >= FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
 }
 
-// Several waves per sequence pay off while they find SIMDs of their own: measured on MI355X
-// (1024 SIMDs) the split kernels win up to about two waves per SIMD and lose beyond.
+// Several waves per sequence: measured on MI355X (1024 SIMDs) the split kernels win or tie at every
+// sequence count for D = 16 (768 sequences: 23 + 28 us against 29 + 40 us; 4096: 112 + 145 against
+// 124 + 145) and up to about a thousand sequences for D = 32 (beyond, their backward is 5-10 % slower).
 // Shapes that have no other fast kernel (E != M, E or M above 32) always take them.
 bool delta_split(int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
                  const fwp_view &beta) {
@@ -47,7 +48,7 @@ bool delta_split(int N, int H, int L, int E, int M, std::initializer_list<fwp_vi
     if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
     if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
-    return L >= 32 && (int64_t)N * H * (E / 8) <= 2048;
+    return L >= 32 && (E == 16 || (int64_t)N * H <= 1024);
 }
 
 }  // namespace
