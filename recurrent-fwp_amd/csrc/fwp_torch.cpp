@@ -1,10 +1,13 @@
-// The delta-rule and sum-rule operators as C++ autograd functions over the C ABI of libfwp_hip.so.
+// The delta-rule, sum-rule, Delta RNN and Recurrent Delta Net operators as C++ autograd functions over
+// the C ABI of libfwp_hip.so.
 //
-// Same operators, arguments, results and errors as DeltaFastWeight in fast_weight.py and FastWeightSum
-// in fast_transformers.py (the reference's algorithmic/fast_weight/__init__.py:26-96 and
-// algorithmic/fast_transformers/__init__.py:25-84); they exist because a forward + backward pair of the
-// benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter time through a Python
-// autograd.Function.  Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
+// Same operators, arguments, results and errors as the Python autograd.Functions of this package
+// (fast_weight.py, fast_transformers.py, fast_weight_rnn_v2.py, rec_update_fwm_tanh.py; the reference's
+// algorithmic/fast_weight/__init__.py:26-96, fast_transformers/__init__.py:25-84,
+// fast_weight_rnn_v2/__init__.py:29-121, rec_update_fwm_tanh/__init__.py:31-139).  They exist because a
+// forward + backward pair of the benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter
+// time through a Python autograd.Function, and a single inference step even less GPU time.
+// Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
 
 #include <c10/core/DeviceGuard.h>
@@ -27,6 +30,20 @@ struct fwp_failure : std::runtime_error {
 PyObject *g_error_class = nullptr;
 
 [[noreturn]] void fail(const std::string &what) { throw fwp_failure(what); }
+
+// The reference checks shapes with assert; so do the Python Functions, and so does this.
+struct fwp_assertion : std::runtime_error {
+    using std::runtime_error::runtime_error;
+};
+void require(bool ok, const char *what) {
+    if (!ok) throw fwp_assertion(what);
+}
+
+bool same_shape(const at::Tensor &t, std::initializer_list<int64_t> shape) { return t.sizes() == at::IntArrayRef(shape); }
+
+void require_state(const at::Tensor &t, const char *name) {
+    if (!t.is_contiguous() || t.scalar_type() != at::kFloat) fail(std::string(name) + " must be a contiguous fp32 tensor");
+}
 
 void check(int rc, const char *what) {
     if (rc != 0)
@@ -219,6 +236,181 @@ struct SumFn : torch::autograd::Function<SumFn> {
     }
 };
 
+struct LaunchGuard {      // makes the tensors' GPU current for a launch when it is not
+    c10::OptionalDeviceGuard guard;
+    explicit LaunchGuard(const at::Tensor &t) {
+        if (t.get_device() != c10::hip::current_device()) guard.reset_device(t.device());
+    }
+};
+
+struct RnnFn : torch::autograd::Function<RnnFn> {
+    static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Z_in, const at::Tensor &K_in,
+                              const at::Tensor &V_in, const at::Tensor &W, const at::Tensor &beta_in,
+                              const at::Tensor &h0, bool need_grad) {
+        require_device(Z_in);
+        require(Z_in.dim() == 4 && V_in.dim() == 4, "expected 4-D [N,H,L,D] tensors");
+        const int64_t N = Z_in.size(0), H = Z_in.size(1), L = Z_in.size(2), D = V_in.size(3);
+        require(same_shape(Z_in, {N, H, L, D}) && same_shape(K_in, {N, H, L, D}) && same_shape(V_in, {N, H, L, D}),
+                "Z, K, V must be [N,H,L,D]");
+        require(same_shape(beta_in, {N, H, L, 1}), "beta must be [N,H,L,1]");
+        require(same_shape(h0, {N, H, 1, D}), "h0 must be [N,H,1,D]");
+        require(same_shape(W, {N, H, D, D}), "W must be [N,H,D,D]");
+        require_state(W, "W");
+        require_state(h0, "h0");
+        fwp_view zv, kv, vv, bv;
+        const at::Tensor Z = rows(Z_in, zv), K = rows(K_in, kv), V = rows(V_in, vv), beta = rows(beta_in, bv);
+        const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
+        const auto opts = Z.options();
+        at::Tensor out = at::empty({N, H, L, D}, opts), vdiff, ckpt, h_init;
+        if (need_grad) {
+            h_init = h0.detach().clone();
+            vdiff = at::empty({N, H, L, D}, opts);
+            ckpt = at::empty({N, H, (L + chunk - 1) / chunk, D, D}, opts);
+        }
+        {
+            LaunchGuard guard(Z);
+            check(fwp_rnn_fwd(zv, kv, vv, bv, W.data_ptr<float>(), h0.data_ptr<float>(), out.data_ptr<float>(),
+                              need_grad ? vdiff.data_ptr<float>() : nullptr,
+                              need_grad ? ckpt.data_ptr<float>() : nullptr, (int)N, (int)H, (int)L, (int)D, chunk,
+                              stream_of(Z)),
+                  "fwp_rnn_fwd");
+        }
+        if (need_grad) {
+            ctx->save_for_backward({K, beta, vdiff, out, h_init, ckpt});
+            ctx->saved_data["chunk"] = (int64_t)chunk;
+        }
+        ctx->set_materialize_grads(false);
+        return out;
+    }
+
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
+                                                 torch::autograd::tensor_list grads) {
+        const at::Tensor none;
+        if (!grads[0].defined()) return {none, none, none, none, none, none, none};
+        const auto saved = ctx->get_saved_variables();
+        if (saved.size() != 6) fail("backward of a forward pass that kept nothing for it");
+        const at::Tensor &K = saved[0], &beta = saved[1], &vdiff = saved[2], &out = saved[3], &h_init = saved[4],
+                         &ckpt = saved[5];
+        const int64_t N = K.size(0), H = K.size(1), L = K.size(2), D = K.size(3);
+        const int chunk = (int)ctx->saved_data["chunk"].toInt();
+        fwp_view kv, bv, gv_;
+        rows(K, kv);
+        rows(beta, bv);
+        const at::Tensor go = rows(grads[0], gv_);
+        const auto opts = K.options();
+        at::Tensor gz = at::empty({N, H, L, D}, opts), gk = at::empty({N, H, L, D}, opts),
+                   gv = at::empty({N, H, L, D}, opts), gb = at::empty({N, H, L, 1}, opts);
+        {
+            LaunchGuard guard(K);
+            check(fwp_rnn_bwd(kv, bv, vdiff.data_ptr<float>(), out.data_ptr<float>(), h_init.data_ptr<float>(), gv_,
+                              ckpt.data_ptr<float>(), gz.data_ptr<float>(), gk.data_ptr<float>(),
+                              gv.data_ptr<float>(), gb.data_ptr<float>(), (int)N, (int)H, (int)L, (int)D, chunk,
+                              stream_of(K)),
+                  "fwp_rnn_bwd");
+        }
+        return {gz, gk, gv, none, gb, none, none};
+    }
+};
+
+at::Tensor fast_rnn_v2(const at::Tensor &Z, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
+                       const at::Tensor &beta, const at::Tensor &h0) {
+    const bool need_grad = at::GradMode::is_enabled() && (Z.requires_grad() || K.requires_grad() || V.requires_grad() ||
+                                                          W.requires_grad() || beta.requires_grad() || h0.requires_grad());
+    return RnnFn::apply(Z, K, V, W, beta, h0, need_grad);
+}
+
+struct RecFn : torch::autograd::Function<RecFn> {
+    static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &qx_in, const at::Tensor &kx_in,
+                              const at::Tensor &vx_in, const at::Tensor &bx_in, const at::Tensor &R_q,
+                              const at::Tensor &R_k, const at::Tensor &R_v, const at::Tensor &r_b, const at::Tensor &W,
+                              const at::Tensor &h0, bool need_grad) {
+        require_device(qx_in);
+        require(qx_in.dim() == 4 && vx_in.dim() == 4, "expected 4-D [N,H,L,D] tensors");
+        const int64_t N = qx_in.size(0), H = qx_in.size(1), L = qx_in.size(2), E = qx_in.size(3), M = vx_in.size(3);
+        require(E == M, "Current kernel only support this case.");
+        require(same_shape(R_q, {1, H, M, M}) && same_shape(R_k, {1, H, M, M}) && same_shape(R_v, {1, H, M, M}) &&
+                    same_shape(r_b, {1, H, 1, M}),
+                "Reshape/unsqueeze if needed.");
+        require(same_shape(kx_in, {N, H, L, M}) && same_shape(vx_in, {N, H, L, M}) && same_shape(bx_in, {N, H, L, 1}),
+                "kx, vx must be [N,H,L,D] and bx [N,H,L,1]");
+        require(same_shape(W, {N, H, M, M}) && same_shape(h0, {N, H, 1, M}), "W must be [N,H,D,D] and h0 [N,H,1,D]");
+        require_state(W, "W");
+        require_state(h0, "h0");
+        const int64_t D = M;
+        fwp_view qv, kv, vv, bv;
+        const at::Tensor qx = rows(qx_in, qv), kx = rows(kx_in, kv), vx = rows(vx_in, vv), bx = rows(bx_in, bv);
+        const at::Tensor Rq = R_q.detach().contiguous().to(at::kFloat), Rk = R_k.detach().contiguous().to(at::kFloat),
+                         Rv = R_v.detach().contiguous().to(at::kFloat), rb = r_b.detach().contiguous().to(at::kFloat);
+        const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
+        const auto opts = qx.options();
+        at::Tensor out = at::empty({N, H, L, D}, opts), h_init, q_act, k_act, beta_act, vdiff, ckpt;
+        if (need_grad) {
+            h_init = h0.detach().clone();
+            q_act = at::empty({N, H, L, D}, opts);          // q after softmax
+            k_act = at::empty({N, H, L, D}, opts);          // k after softmax
+            beta_act = at::empty({N, H, L}, opts);          // beta after sigmoid
+            vdiff = at::empty({N, H, L, D}, opts);          // v - v_old
+            ckpt = at::empty({N, H, (L + chunk - 1) / chunk, D, D}, opts);
+        }
+        const auto p = [&](const at::Tensor &t) { return need_grad ? t.data_ptr<float>() : nullptr; };
+        {
+            LaunchGuard guard(qx);
+            check(fwp_rec_fwd(qv, kv, vv, bv, Rq.data_ptr<float>(), Rk.data_ptr<float>(), Rv.data_ptr<float>(),
+                              rb.data_ptr<float>(), W.data_ptr<float>(), h0.data_ptr<float>(), out.data_ptr<float>(),
+                              p(q_act), p(k_act), p(beta_act), p(vdiff), p(ckpt), (int)N, (int)H, (int)L, (int)D,
+                              chunk, stream_of(qx)),
+                  "fwp_rec_fwd");
+        }
+        if (need_grad) {
+            ctx->save_for_backward({out, h_init, Rq, Rk, Rv, rb, q_act, k_act, beta_act, vdiff, ckpt});
+            ctx->saved_data["chunk"] = (int64_t)chunk;
+        }
+        ctx->set_materialize_grads(false);
+        return out;
+    }
+
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
+                                                 torch::autograd::tensor_list grads) {
+        const at::Tensor none;
+        if (!grads[0].defined()) return {none, none, none, none, none, none, none, none, none, none, none};
+        const auto saved = ctx->get_saved_variables();
+        if (saved.size() != 11) fail("backward of a forward pass that kept nothing for it");
+        const at::Tensor &out = saved[0], &h_init = saved[1], &Rq = saved[2], &Rk = saved[3], &Rv = saved[4],
+                         &rb = saved[5], &q_act = saved[6], &k_act = saved[7], &beta_act = saved[8],
+                         &vdiff = saved[9], &ckpt = saved[10];
+        const int64_t N = out.size(0), H = out.size(1), L = out.size(2), D = out.size(3);
+        const int chunk = (int)ctx->saved_data["chunk"].toInt();
+        fwp_view gv_;
+        const at::Tensor go = rows(grads[0], gv_);
+        const auto opts = out.options();
+        at::Tensor gqx = at::empty({N, H, L, D}, opts), gkx = at::empty({N, H, L, D}, opts),
+                   gvx = at::empty({N, H, L, D}, opts), gbx = at::empty({N, H, L, 1}, opts),
+                   gRq = at::empty({1, H, D, D}, opts), gRk = at::empty({1, H, D, D}, opts),
+                   gRv = at::empty({1, H, D, D}, opts), grb = at::empty({1, H, 1, D}, opts),
+                   workspace = at::empty({N, H, 3 * D * D + D}, opts);
+        {
+            LaunchGuard guard(out);
+            check(fwp_rec_bwd(q_act.data_ptr<float>(), k_act.data_ptr<float>(), beta_act.data_ptr<float>(),
+                              vdiff.data_ptr<float>(), out.data_ptr<float>(), h_init.data_ptr<float>(), gv_,
+                              Rq.data_ptr<float>(), Rk.data_ptr<float>(), Rv.data_ptr<float>(), rb.data_ptr<float>(),
+                              ckpt.data_ptr<float>(), gqx.data_ptr<float>(), gkx.data_ptr<float>(),
+                              gvx.data_ptr<float>(), gbx.data_ptr<float>(), gRq.data_ptr<float>(),
+                              gRk.data_ptr<float>(), gRv.data_ptr<float>(), grb.data_ptr<float>(),
+                              workspace.data_ptr<float>(), (int)N, (int)H, (int)L, (int)D, chunk, stream_of(out)),
+                  "fwp_rec_bwd");
+        }
+        return {gqx, gkx, gvx, gbx, gRq, gRk, gRv, grb, none, none, none};
+    }
+};
+
+at::Tensor rec_update_fwm_tanh(const at::Tensor &qx, const at::Tensor &kx, const at::Tensor &vx, const at::Tensor &bx,
+                               const at::Tensor &R_q, const at::Tensor &R_k, const at::Tensor &R_v,
+                               const at::Tensor &r_b, const at::Tensor &W, const at::Tensor &h0) {
+    bool any = false;
+    for (const at::Tensor *t : {&qx, &kx, &vx, &bx, &R_q, &R_k, &R_v, &r_b, &W, &h0}) any = any || t->requires_grad();
+    return RecFn::apply(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0, at::GradMode::is_enabled() && any);
+}
+
 at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
                            bool exact) {
     const bool need_grad = at::GradMode::is_enabled() && (Q.requires_grad() || K.requires_grad() || V.requires_grad());
@@ -246,11 +438,18 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             if (p) std::rethrow_exception(p);
         } catch (const fwp_failure &e) {
             PyErr_SetString(g_error_class ? g_error_class : PyExc_RuntimeError, e.what());
+        } catch (const fwp_assertion &e) {
+            PyErr_SetString(PyExc_AssertionError, e.what());
         }
     });
     m.def("fast_weight_delta", &fast_weight_delta,
           "out = fast_weight_delta(Q, K, V, beta, W): delta-rule fast weight memory; W is updated in place");
     m.def("fast_weight_sum", &fast_weight_sum,
           "out = fast_weight_sum(Q, K, V, W, exact): sum-rule fast weight memory; W is updated in place");
+    m.def("fast_rnn_v2", &fast_rnn_v2,
+          "rnn_out = fast_rnn_v2(Z, K, V, W, beta, h0): Delta RNN; W and h0 are updated in place");
+    m.def("rec_update_fwm_tanh", &rec_update_fwm_tanh,
+          "out = rec_update_fwm_tanh(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0): Recurrent Delta Net; W and h0 "
+          "are updated in place");
     m.def("set_error_class", &set_error_class, "exception class raised for rejected calls");
 }

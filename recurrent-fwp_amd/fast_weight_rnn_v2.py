@@ -3,7 +3,7 @@
 import torch
 
 from . import _lib
-from .fast_weight import _nchunk
+from .fast_weight import _fwp_torch, _nchunk
 
 
 class FastRNNv2(torch.autograd.Function):
@@ -77,4 +77,5 @@ class FastRNNv2(torch.autograd.Function):
         return grad_Z, grad_K, grad_V, None, grad_beta, None
 
 
-fast_rnn_v2 = FastRNNv2.apply
+# the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
+fast_rnn_v2 = _fwp_torch.fast_rnn_v2 if _fwp_torch is not None else FastRNNv2.apply

@@ -3,7 +3,7 @@
 import torch
 
 from . import _lib
-from .fast_weight import _nchunk
+from .fast_weight import _fwp_torch, _nchunk
 
 
 class FastWeightRecUpdateTanh(torch.autograd.Function):
@@ -92,4 +92,5 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
                 grad_R_q, grad_R_k, grad_R_v, grad_r_b, None, None)
 
 
-rec_update_fwm_tanh = FastWeightRecUpdateTanh.apply
+# the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
+rec_update_fwm_tanh = _fwp_torch.rec_update_fwm_tanh if _fwp_torch is not None else FastWeightRecUpdateTanh.apply

@@ -88,3 +88,40 @@ def test_sum_rule_same_as_python_function(fwp, mode, N, H, L, E, M):
             fwp.fast_weight_sum(q, k, v, W0.clone())
     finally:
         fwp.FastWeightSum.state_gradient = "reference"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,L,D", [(2, 2, 64, 32), (1, 3, 37, 16), (2, 1, 1, 32), (1, 2, 20, 24)])
+def test_delta_rnn_same_as_python_function(fwp, N, H, L, D):
+    from helpers import rnn_inputs
+    z, k, v, W0, beta, h0, go = (torch.from_numpy(a).cuda() for a in rnn_inputs(21, N, H, L, D, dtype=np.float32, w0=True))
+    assert fwp.fast_rnn_v2 is native(fwp).fast_rnn_v2
+    results = []
+    for f in (fwp.fast_rnn_v2, fwp.FastRNNv2.apply):
+        ins = [t.clone().requires_grad_(True) for t in (z, k, v, beta)]
+        W, h = W0.clone(), h0.clone()
+        out = f(ins[0], ins[1], ins[2], W, ins[3], h)
+        results.append([out, W, h, *torch.autograd.grad(out, ins, go)])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    with pytest.raises(AssertionError):
+        fwp.fast_rnn_v2(z, k[:, :, :-1], v, W0.clone(), beta, h0.clone())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,L,D", [(2, 2, 64, 32), (1, 3, 37, 16), (2, 1, 1, 32), (1, 2, 20, 24)])
+def test_recurrent_delta_net_same_as_python_function(fwp, N, H, L, D):
+    from helpers import rec_inputs
+    arrays = [torch.from_numpy(a).cuda() for a in rec_inputs(22, N, H, L, D, dtype=np.float32, w0=True)]
+    diff, W0, h0, go = arrays[:8], arrays[8], arrays[9], arrays[10]
+    assert fwp.rec_update_fwm_tanh is native(fwp).rec_update_fwm_tanh
+    results = []
+    for f in (fwp.rec_update_fwm_tanh, fwp.FastWeightRecUpdateTanh.apply):
+        ins = [t.clone().requires_grad_(True) for t in diff]
+        W, h = W0.clone(), h0.clone()
+        out = f(*ins, W, h)
+        results.append([out, W, h, *torch.autograd.grad(out, ins, go)])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    with pytest.raises(AssertionError, match="Reshape"):
+        fwp.rec_update_fwm_tanh(*diff[:4], diff[4][0], *diff[5:], W0.clone(), h0.clone())
