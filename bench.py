@@ -427,12 +427,54 @@ def lm_cpu_baseline(pkg):
                       f"median of 2 runs after a warm-up ({med:.1f} s each)"}
 
 
+def run_single_steps(args, pkg):
+    """Stepwise inference: one call per time step (T = 1, no gradient, state carried in W and h), as an
+    actor or a decoder makes them.  Launch- and host-bound; reported per operator, through the package's
+    default entry point and through the Python autograd.Function."""
+    import numpy as np
+    import torch
+    from helpers import delta_inputs, rec_inputs, rnn_inputs
+    B, H, D = 32, 8, 32
+    dev = lambda arrays: [torch.from_numpy(a).to("cuda:0") for a in arrays]
+    q, k, v, beta, W0, _ = dev(delta_inputs(0, B, H, 1, D, D, dtype=np.float32))
+    z, rk, rv, rW0, rbeta, rh0, _ = dev(rnn_inputs(0, B, H, 1, D, dtype=np.float32))
+    rec = dev(rec_inputs(0, B, H, 1, D, dtype=np.float32))
+    W, h = W0.clone(), rh0.clone()
+    calls = {
+        "fast_weight_delta": (lambda f: f(q, k, v, beta, W), pkg.fast_weight_delta, pkg.DeltaFastWeight.apply),
+        "fast_rnn_v2": (lambda f: f(z, rk, rv, W, rbeta, h), pkg.fast_rnn_v2, pkg.FastRNNv2.apply),
+        "rec_update_fwm_tanh": (lambda f: f(*rec[:8], W, h), pkg.rec_update_fwm_tanh,
+                                pkg.FastWeightRecUpdateTanh.apply),
+    }
+    n = max(args.steps, 1) * 10
+    out = {}
+    with torch.no_grad():
+        for name, (call, default, python) in calls.items():
+            for label, f in (("default", default), ("python_function", python)):
+                for _ in range(args.warmup):
+                    call(f)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n):
+                    call(f)
+                torch.cuda.synchronize()
+                out.setdefault(name, {})[label + "_us"] = (time.perf_counter() - t0) / n * 1e6
+    lat = out["fast_weight_delta"]["default_us"] * 1e-6
+    return {"metric": "stepwise inference tokens/s (one forward call per time step, no gradient), 1 GPU",
+            "value": B / lat, "unit": "tokens/s", "n_gpus": 1, "steps": n, "warmup": args.warmup,
+            "ms_per_step": lat * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f32", "data": "synthetic",
+            "config": {"workload": "single steps: fast_weight_delta forward, B=32 H=8 T=1 D=32, state carried",
+                       "B": B, "H": H, "T": 1, "D": D},
+            "roofline": None, "cpu_baseline": None, "latency_us_per_call": out}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["lm"], default="delta")
+    ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["lm", "step"], default="delta")
     ap.add_argument("--cpu-reps", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--delta-kernels", choices=["auto", "scan", "chunked", "split"], default="auto",
@@ -465,6 +507,9 @@ def main():
     name = args.workload
     if name == "lm":
         print(json.dumps(run_lm(args, pkg)))
+        return
+    if name == "step":
+        print(json.dumps(run_single_steps(args, pkg)))
         return
     w = WORKLOADS[name]
     arrays = make_inputs(name, w)
