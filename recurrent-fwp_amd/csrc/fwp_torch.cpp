@@ -1,10 +1,11 @@
-// The delta-rule, sum-rule, Delta RNN and Recurrent Delta Net operators as C++ autograd functions over
-// the C ABI of libfwp_hip.so.
+// The delta-rule, sum-rule, Delta RNN, Recurrent Delta Net and Delta LSTM operators as C++ autograd
+// functions over the C ABI of libfwp_hip.so.
 //
 // Same operators, arguments, results and errors as the Python autograd.Functions of this package
-// (fast_weight.py, fast_transformers.py, fast_weight_rnn_v2.py, rec_update_fwm_tanh.py; the reference's
+// (fast_weight.py, fast_transformers.py, fast_weight_rnn_v2.py, rec_update_fwm_tanh.py, fast_lstm_v4.py; the reference's
 // algorithmic/fast_weight/__init__.py:26-96, fast_transformers/__init__.py:25-84,
-// fast_weight_rnn_v2/__init__.py:29-121, rec_update_fwm_tanh/__init__.py:31-139).  They exist because a
+// fast_weight_rnn_v2/__init__.py:29-121, rec_update_fwm_tanh/__init__.py:31-139,
+// language_modeling/src/utils/fast_lstm_v4/__init__.py:36-208).  They exist because a
 // forward + backward pair of the benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter
 // time through a Python autograd.Function, and a single inference step even less GPU time.
 // Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
@@ -17,6 +18,7 @@
 #include <mutex>
 #include <stdexcept>
 #include <string>
+#include <tuple>
 #include <unordered_map>
 
 #include "fwp_hip.h"
@@ -411,6 +413,119 @@ at::Tensor rec_update_fwm_tanh(const at::Tensor &qx, const at::Tensor &kx, const
     return RecFn::apply(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0, at::GradMode::is_enabled() && any);
 }
 
+struct LstmFn : torch::autograd::Function<LstmFn> {
+    // gates in the order i (input gate), u (update), o (output gate); per gate Z, K, V, beta, W
+    static torch::autograd::variable_list forward(
+        torch::autograd::AutogradContext *ctx, const at::Tensor &Zi, const at::Tensor &Ki, const at::Tensor &Vi,
+        const at::Tensor &bi, const at::Tensor &Wi, const at::Tensor &Zu, const at::Tensor &Ku, const at::Tensor &Vu,
+        const at::Tensor &bu, const at::Tensor &Wu, const at::Tensor &Zo, const at::Tensor &Ko, const at::Tensor &Vo,
+        const at::Tensor &bo, const at::Tensor &Wo, const at::Tensor &h0, const at::Tensor &c0, bool need_grad) {
+        require_device(Zi);
+        if (Zi.dim() != 4 || Vi.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
+        const int64_t N = Zi.size(0), H = Zi.size(1), L = Zi.size(2), D = Vi.size(3);
+        const at::Tensor *Zs[3] = {&Zi, &Zu, &Zo}, *Ks[3] = {&Ki, &Ku, &Ko}, *Vs[3] = {&Vi, &Vu, &Vo},
+                         *Bs[3] = {&bi, &bu, &bo}, *Ws[3] = {&Wi, &Wu, &Wo};
+        for (int a = 0; a < 3; a++)
+            if (!(same_shape(*Zs[a], {N, H, L, D}) && same_shape(*Ks[a], {N, H, L, D}) &&
+                  same_shape(*Vs[a], {N, H, L, D}) && same_shape(*Bs[a], {N, H, L, 1}) &&
+                  same_shape(*Ws[a], {N, H, D, D})))
+                fail("shape mismatch between the gates' Z, K, V [N,H,L,D], beta [N,H,L,1] and W [N,H,D,D]");
+        if (!same_shape(h0, {N, H, 1, D}) || !same_shape(c0, {N, H, 1, D})) fail("h0 and c0 must be [N,H,1,D]");
+        require_state(Wi, "Wi");
+        require_state(Wu, "Wu");
+        require_state(Wo, "Wo");
+        require_state(h0, "h0");
+        require_state(c0, "c0");
+        fwp_view zv[3], kv[3], vv[3], bv[3];
+        at::Tensor Zr[3], Kr[3], Vr[3], Br[3];
+        float *Wp[3];
+        for (int a = 0; a < 3; a++) {
+            Zr[a] = rows(*Zs[a], zv[a]);
+            Kr[a] = rows(*Ks[a], kv[a]);
+            Vr[a] = rows(*Vs[a], vv[a]);
+            Br[a] = rows(*Bs[a], bv[a]);
+            Wp[a] = Ws[a]->data_ptr<float>();
+        }
+        const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
+        const auto opts = Zr[0].options();
+        at::Tensor out = at::empty({N, H, L, D}, opts), cell = at::empty({N, H, L, D}, opts), gates, vdiff, ckpt,
+                   h_init, c_init;
+        if (need_grad) {
+            h_init = h0.detach().clone();
+            c_init = c0.detach().clone();
+            gates = at::empty({3, N, H, L, D}, opts);
+            vdiff = at::empty({3, N, H, L, D}, opts);
+            ckpt = at::empty({3, N, H, (L + chunk - 1) / chunk, D, D}, opts);
+        }
+        const auto p = [&](const at::Tensor &t) { return need_grad ? t.data_ptr<float>() : nullptr; };
+        {
+            LaunchGuard guard(Zr[0]);
+            check(fwp_lstm_fwd(zv, kv, vv, bv, Wp, h0.data_ptr<float>(), c0.data_ptr<float>(), out.data_ptr<float>(),
+                               cell.data_ptr<float>(), p(gates), p(vdiff), p(ckpt), (int)N, (int)H, (int)L, (int)D,
+                               chunk, stream_of(Zr[0])),
+                  "fwp_lstm_fwd");
+        }
+        if (need_grad) {
+            ctx->save_for_backward({Kr[0], Kr[1], Kr[2], Br[0], Br[1], Br[2], vdiff, gates, out, cell, h_init, c_init, ckpt});
+            ctx->saved_data["chunk"] = (int64_t)chunk;
+        }
+        ctx->mark_non_differentiable({cell});
+        ctx->set_materialize_grads(false);
+        return {out, cell};
+    }
+
+    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
+                                                 torch::autograd::tensor_list grads) {
+        const at::Tensor none;
+        torch::autograd::tensor_list res(18, none);
+        if (!grads[0].defined()) return res;
+        const auto saved = ctx->get_saved_variables();
+        if (saved.size() != 13) fail("backward of a forward pass that kept nothing for it");
+        const at::Tensor &vdiff = saved[6], &gates = saved[7], &out = saved[8], &cell = saved[9], &h_init = saved[10],
+                         &c_init = saved[11], &ckpt = saved[12];
+        const int64_t N = out.size(0), H = out.size(1), L = out.size(2), D = out.size(3);
+        const int chunk = (int)ctx->saved_data["chunk"].toInt();
+        fwp_view kv[3], bv[3], gov;
+        for (int a = 0; a < 3; a++) {
+            rows(saved[a], kv[a]);
+            rows(saved[3 + a], bv[a]);
+        }
+        const at::Tensor go = rows(grads[0], gov);
+        const auto opts = out.options();
+        at::Tensor gz = at::empty({3, N, H, L, D}, opts), gk = at::empty({3, N, H, L, D}, opts),
+                   gv = at::empty({3, N, H, L, D}, opts), gb = at::empty({3, N, H, L, 1}, opts);
+        {
+            LaunchGuard guard(out);
+            check(fwp_lstm_bwd(kv, bv, vdiff.data_ptr<float>(), gates.data_ptr<float>(), out.data_ptr<float>(),
+                               cell.data_ptr<float>(), h_init.data_ptr<float>(), c_init.data_ptr<float>(), gov,
+                               ckpt.data_ptr<float>(), gz.data_ptr<float>(), gk.data_ptr<float>(),
+                               gv.data_ptr<float>(), gb.data_ptr<float>(), (int)N, (int)H, (int)L, (int)D, chunk,
+                               stream_of(out)),
+                  "fwp_lstm_bwd");
+        }
+        for (int a = 0; a < 3; a++) {
+            res[5 * a + 0] = gz[a];
+            res[5 * a + 1] = gk[a];
+            res[5 * a + 2] = gv[a];
+            res[5 * a + 3] = gb[a];
+        }
+        return res;
+    }
+};
+
+std::tuple<at::Tensor, at::Tensor> fast_lstm_v4(
+    const at::Tensor &Zi, const at::Tensor &Ki, const at::Tensor &Vi, const at::Tensor &bi, const at::Tensor &Wi,
+    const at::Tensor &Zu, const at::Tensor &Ku, const at::Tensor &Vu, const at::Tensor &bu, const at::Tensor &Wu,
+    const at::Tensor &Zo, const at::Tensor &Ko, const at::Tensor &Vo, const at::Tensor &bo, const at::Tensor &Wo,
+    const at::Tensor &h0, const at::Tensor &c0) {
+    bool any = false;
+    for (const at::Tensor *t : {&Zi, &Ki, &Vi, &bi, &Wi, &Zu, &Ku, &Vu, &bu, &Wu, &Zo, &Ko, &Vo, &bo, &Wo, &h0, &c0})
+        any = any || t->requires_grad();
+    const auto r = LstmFn::apply(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0,
+                                 at::GradMode::is_enabled() && any);
+    return {r[0], r[1]};
+}
+
 at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
                            bool exact) {
     const bool need_grad = at::GradMode::is_enabled() && (Q.requires_grad() || K.requires_grad() || V.requires_grad());
@@ -451,5 +566,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("rec_update_fwm_tanh", &rec_update_fwm_tanh,
           "out = rec_update_fwm_tanh(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0): Recurrent Delta Net; W and h0 "
           "are updated in place");
+    m.def("fast_lstm_v4", &fast_lstm_v4,
+          "rnn_out, cell_out = fast_lstm_v4(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0): "
+          "Delta LSTM; the W, h0 and c0 are updated in place");
     m.def("set_error_class", &set_error_class, "exception class raised for rejected calls");
 }

@@ -5,7 +5,7 @@ import ctypes
 import torch
 
 from . import _lib
-from .fast_weight import _nchunk
+from .fast_weight import _fwp_torch, _nchunk
 
 
 def _views(ts):
@@ -95,4 +95,5 @@ class FastLSTMv4(torch.autograd.Function):
         return (*res, None, None)
 
 
-fast_lstm_v4 = FastLSTMv4.apply
+# the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
+fast_lstm_v4 = _fwp_torch.fast_lstm_v4 if _fwp_torch is not None else FastLSTMv4.apply

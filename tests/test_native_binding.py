@@ -125,3 +125,29 @@ def test_recurrent_delta_net_same_as_python_function(fwp, N, H, L, D):
         assert torch.equal(a, b)
     with pytest.raises(AssertionError, match="Reshape"):
         fwp.rec_update_fwm_tanh(*diff[:4], diff[4][0], *diff[5:], W0.clone(), h0.clone())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,L,D", [(2, 2, 64, 32), (1, 2, 24, 16), (2, 1, 1, 32), (1, 2, 11, 18)])
+def test_delta_lstm_same_as_python_function(fwp, N, H, L, D):
+    from helpers import lstm_inputs
+    Zs, Ks, Vs, Bs, Ws, h0, c0, go = lstm_inputs(23, N, H, L, D, dtype=np.float32, w0=True)
+    cu = lambda a: torch.from_numpy(a).cuda()
+    assert fwp.fast_lstm_v4 is native(fwp).fast_lstm_v4
+    results = []
+    for f in (fwp.fast_lstm_v4, fwp.FastLSTMv4.apply):
+        ins, args, states = [], [], []
+        for g in range(3):
+            quad = [cu(x[g]).requires_grad_(True) for x in (Zs, Ks, Vs, Bs)]
+            W = cu(Ws[g]).clone()
+            ins += quad
+            states.append(W)
+            args += [*quad, W]
+        h, c = cu(h0).clone(), cu(c0).clone()
+        out, cell = f(*args, h, c)
+        assert not cell.requires_grad
+        results.append([out, cell, h, c, *states, *torch.autograd.grad(out, ins, cu(go))])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    with pytest.raises(fwp._lib.FwpError, match="h0 and c0"):
+        fwp.fast_lstm_v4(*args, h[:, :, 0], c)
