@@ -34,6 +34,13 @@ bool delta_chunked(int L) {
 // Several waves per sequence: measured on MI355X (1024 SIMDs) the split kernels win or tie at every
 // sequence count for D = 16 (768 sequences: 23 + 28 us against 29 + 40 us; 4096: 112 + 145 against
 // 124 + 145) and up to about a thousand sequences for D = 32 (beyond, their backward is 5-10 % slower).
+// The kernels that read through buffer resources address a sequence with 32-bit byte offsets.
+bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
+    for (const fwp_view &v : views)
+        if (v.sL < 0 || ((int64_t)L * v.sL + (E > M ? E : M)) * 4 >= (int64_t(1) << 31)) return false;
+    return true;
+}
+
 // Shapes that have no other fast kernel (E != M, E or M above 32) always take them.
 bool delta_split(int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
                  const fwp_view &beta) {
@@ -153,9 +160,11 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
     if (split_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
         aligned16(out)) {
         // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
-        if (!reg_delta_supported(E, M) || delta_chunked(L))
+        const bool blocked = in_range32(L, E, M, {q, k, v}) && (!reg_delta_supported(E, M) || delta_chunked(L));
+        if (blocked)
             return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
-        return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+        if (reg_delta_supported(E, M))
+            return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
     }
     return generic_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
 }
@@ -169,10 +178,13 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (split_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
-        if (!reg_delta_supported(E, M) || delta_chunked(L))
+        const bool blocked =
+            in_range32(L, E, M, {q, k, v, grad_out}) && (!reg_delta_supported(E, M) || delta_chunked(L));
+        if (blocked)
             return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
                                 (hipStream_t)stream);
-        return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
+        if (reg_delta_supported(E, M))
+            return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,
                            (hipStream_t)stream);
     }
     return generic_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,

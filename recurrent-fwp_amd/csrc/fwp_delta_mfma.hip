@@ -607,29 +607,18 @@ __global__ __launch_bounds__(64) void k_delta_bwd_mfma(fwp_view q, fwp_view k, f
 //
 // The same blocks without the triangular system: O = Q S + lower(Q K^T) V, S' = S + K^T V, and in
 // reverse g_v = K dS + lower(Q K^T)^T dO, g_q = dO S0^T + lower(dO V^T) K,
-// g_k = V dS^T + lower(dO V^T)^T Q, dS += Q^T dO.
+// g_k = V dS^T + lower(dO V^T)^T Q, dS += Q^T dO.  One wave per sequence; the state is E x M,
+// NE = E/16 by NM = M/16 tiles.  Every tensor is read and written through a buffer resource of
+// exactly the sequence's size: the missing rows of a last partial block read as zeros (they then
+// write nothing to the state and carry no gradient) and stores to them are dropped.  The operands
+// of the coming blocks wait in a ring of registers; matrices needed transposed go through LDS.
 
-// Loads of one 16-step block of a [.., L, D] tensor in both orientations.  Rows beyond L: clamped
-// loads, zeroed if `zero_tail`.
-template <int NB>
-struct BothWays {
-    v4f t[NB], c[NB];   // t: register r = X[t0 + c][16b + 4g + r];  c: register r = X[t0 + 4g + r][16b + c]
-    __device__ __forceinline__ void load(const float *base, int64_t sL, int t0, int L, const Geo16 &p,
-                                         bool zero_tail) {
-        const int64_t tc = min(t0 + p.c, L - 1);
-        const bool col_ok = !zero_tail || t0 + p.c < L;
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const float4 x = *reinterpret_cast<const float4 *>(base + tc * sL + 16 * b + 4 * p.g);
-            t[b] = col_ok ? v4f{x.x, x.y, x.z, x.w} : v4f{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const int64_t tr = min(t0 + 4 * p.g + r, L - 1);
-                const float y = base[tr * sL + 16 * b + p.c];
-                c[b][r] = (!zero_tail || t0 + 4 * p.g + r < L) ? y : 0.f;
-            }
-        }
-    }
+constexpr int sum_ring(int ne, int nm) { return (ne + nm) <= 3 ? 3 : (ne + nm) <= 6 ? 2 : 1; }
+
+// Kt[b], Qt[b]: register r = K[t0 + c][16b + 4g + r];  Kc[b], Vc[b]: register r = K[t0 + 4g + r][16b + c]
+template <int NE, int NM>
+struct SumFwdRaw {
+    v4f Kt[NE], Qt[NE], Kc[NE], Vc[NM];
 };
 
 template <int NE, int NM>   // state E = 16 NE by M = 16 NM
@@ -637,13 +626,29 @@ __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp
                                                      float *__restrict__ W, float *__restrict__ out,
                                                      float *__restrict__ ckpt, int H, int L, int chunk,
                                                      int nchunk) {
-    constexpr int E = 16 * NE, M = 16 * NM;
+    constexpr int E = 16 * NE, M = 16 * NM, PF = sum_ring(NE, NM);
     const Geo16 p(threadIdx.x);
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0);
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)), ob(out + seq * L * M, (uint32_t)(L * M * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   v_step = (unsigned)(kBlk * v.sL * 4), m_step = (unsigned)(kBlk * M * 4);
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                   o_out = (unsigned)(c * M + 4 * g) * 4;
+    unsigned o_kr[4], o_vr[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+        o_vr[r] = (unsigned)((4 * g + r) * v.sL + c) * 4;
+    }
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    const int nblk = (L + kBlk - 1) / kBlk;
+    const ChunkOf chunk_of(chunk);
+
+    // S[eb][mb]: register r holds S[16 eb + 4g + r][16 mb + c]
     v4f S[NE][NM];
 #pragma unroll
     for (int eb = 0; eb < NE; eb++)
@@ -653,40 +658,40 @@ __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp
             for (int r = 0; r < 4; r++)
                 S[eb][mb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
 
-    struct Raw { BothWays<NE> K, Q; BothWays<NM> V; };
-    auto load = [&](Raw &w, int t0) {
-        w.K.load(kb, k.sL, t0, L, p, true);       // zero rows beyond L: they then write nothing
-        w.Q.load(qb, q.sL, t0, L, p, false);
-        w.V.load(vb, v.sL, t0, L, p, false);
+    using Raw = SumFwdRaw<NE, NM>;
+    auto load = [&](Raw &w, int ib) {
+        const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step;
+#pragma unroll
+        for (int b = 0; b < NE; b++) {
+            w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+        }
+#pragma unroll
+        for (int b = 0; b < NM; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) w.Vc[b][r] = vb.f(o_vr[r] + 64 * b, vs);
     };
-    const int nblk = (L + kBlk - 1) / kBlk;
-    Raw cur, nxt;
-    load(cur, 0);
-    for (int ib = 0; ib < nblk; ib++) {
-        const int t0 = ib * kBlk;
-        load(nxt, min(ib + 1, nblk - 1) * kBlk);
-        __builtin_amdgcn_sched_barrier(0);
+    auto block = [&](int ib, const Raw &w) {
         v4f R = zero;
 #pragma unroll
-        for (int b = 0; b < NE; b++) R = tn(cur.K.t[b], cur.Q.t[b], R);      // K Q^T [s][t]
+        for (int b = 0; b < NE; b++) R = tn(w.Kt[b], w.Qt[b], R);      // K Q^T [s][t]
 #pragma unroll
         for (int r = 0; r < 4; r++) R[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;   // lower(Q K^T)^T
 #pragma unroll
         for (int mb = 0; mb < NM; mb++) {
-            v4f Ot = tn(cur.V.c[mb], R, zero);
+            v4f Ot = tn(w.Vc[mb], R, zero);
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb][mb], cur.Q.t[eb], Ot);
-            if (t0 + c < L)
-                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * M + 16 * mb + 4 * g) =
-                    make_float4(Ot[0], Ot[1], Ot[2], Ot[3]);
+            for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb][mb], w.Qt[eb], Ot);
+            ob.st4(Ot, o_out + 64 * mb, ib * m_step);        // register r = O[t0 + c][16 mb + 4g + r]
         }
 #pragma unroll
         for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-            for (int mb = 0; mb < NM; mb++) S[eb][mb] = tn(cur.K.c[eb], cur.V.c[mb], S[eb][mb]);
-        const int t_end = min(t0 + kBlk, L);
-        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
-            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * E * M;
+            for (int mb = 0; mb < NM; mb++) S[eb][mb] = tn(w.Kc[eb], w.Vc[mb], S[eb][mb]);
+        if (ckpt && (chunk_of.closes(ib) || ib + 1 == nblk)) {
+            float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * E * M;
 #pragma unroll
             for (int eb = 0; eb < NE; eb++)
 #pragma unroll
@@ -695,8 +700,8 @@ __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp
                     for (int r = 0; r < 4; r++)
                         dst[(16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
         }
-        cur = nxt;
-    }
+    };
+    ring_loop<PF, Raw, false>(nblk, load, block);
 #pragma unroll
     for (int eb = 0; eb < NE; eb++)
 #pragma unroll
@@ -706,120 +711,155 @@ __global__ __launch_bounds__(64) void k_sum_fwd_mfma(fwp_view q, fwp_view k, fwp
                 W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
 }
 
-template <int NE, int NM>   // state E = 16 NE by M = 16 NM
+// O: upstream gradient.  Sck: block (mb, eb) of S^T as checkpointed at the end of the block's chunk,
+// minus the carried-in state if asked.
+template <int NE, int NM>
+struct SumBwdRaw {
+    v4f Kt[NE], Kc[NE], Qt[NE], Qc[NE], Vt[NM], Vc[NM], Ot[NM], Oc[NM];
+    v4f Sck[NM][NE];
+};
+
+template <int NE, int NM>
 __global__ __launch_bounds__(64) void k_sum_bwd_mfma(fwp_view q, fwp_view k, fwp_view v, fwp_view go,
                                                      const float *__restrict__ ckpt,
                                                      const float *__restrict__ W_init,
                                                      float *__restrict__ gq, float *__restrict__ gk,
                                                      float *__restrict__ gv, int H, int L, int chunk,
                                                      int nchunk) {
-    constexpr int E = 16 * NE, M = 16 * NM;
-    const Geo16 p(threadIdx.x);
+    constexpr int E = 16 * NE, M = 16 * NM, PF = sum_ring(NE, NM) > 1 ? sum_ring(NE, NM) - 1 : 1;
+    __shared__ LdsMat scratch[4];
+    const int lane = threadIdx.x;
+    const Geo16 p(lane);
     const int g = p.g, c = p.c;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / H), h = (int)(seq % H);
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
-                *gob = row(go, n, h, 0);
-    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f ident;
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
+        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + M) * 4)),
+        cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
+        wb(W_init ? W_init + seq * E * M : nullptr, W_init ? (uint32_t)(E * M * 4) : 0),
+        gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
+        gvb(gv + seq * L * M, (uint32_t)(L * M * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   v_step = (unsigned)(kBlk * v.sL * 4), o_step = (unsigned)(kBlk * go.sL * 4),
+                   e_step = (unsigned)(kBlk * E * 4), m_step = (unsigned)(kBlk * M * 4);
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                   o_vt = (unsigned)(c * v.sL + 4 * g) * 4, o_ot = (unsigned)(c * go.sL + 4 * g) * 4,
+                   o_ge = (unsigned)(c * E + 4 * g) * 4, o_gm = (unsigned)(c * M + 4 * g) * 4,
+                   o_ck = (unsigned)(c * M + 4 * g) * 4;
+    unsigned o_kr[4], o_qr[4], o_vr[4], o_or[4];
 #pragma unroll
-    for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+    for (int r = 0; r < 4; r++) {
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
+        o_vr[r] = (unsigned)((4 * g + r) * v.sL + c) * 4;
+        o_or[r] = (unsigned)((4 * g + r) * go.sL + c) * 4;
+    }
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    const int nblk = (L + kBlk - 1) / kBlk;
+    const ChunkOf chunk_of(chunk);
 
-    struct Raw { BothWays<NE> K, Q; BothWays<NM> V, O; v4f Sck[NM][NE]; };
-    auto load = [&](Raw &w, int t0) {
-        const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * E * M;
+    using Raw = SumBwdRaw<NE, NM>;
+    auto load = [&](Raw &w, int e) {
+        const int ib = nblk - 1 - e;
+        const unsigned cs = chunk_of(ib) * (E * M * 4);
 #pragma unroll
         for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) {     // block (mb, eb) of S^T, minus the carried-in state if asked
-                const int64_t o = (16 * eb + c) * M + 16 * mb + 4 * g;
-                float4 x = *reinterpret_cast<const float4 *>(src + o);
-                if (W_init) {
-                    const float4 y = *reinterpret_cast<const float4 *>(W_init + seq * E * M + o);
-                    x = make_float4(x.x - y.x, x.y - y.y, x.z - y.z, x.w - y.w);
-                }
-                w.Sck[mb][eb] = v4f{x.x, x.y, x.z, x.w};
+            for (int eb = 0; eb < NE; eb++) {
+                const unsigned o = o_ck + (unsigned)(16 * eb * M + 16 * mb) * 4;
+                w.Sck[mb][eb] = cb.f4(o, cs);
+                if (W_init) w.Sck[mb][eb] -= wb.f4(o, 0);
             }
-        w.K.load(kb, k.sL, t0, L, p, false);
-        w.Q.load(qb, q.sL, t0, L, p, false);
-        w.V.load(vb, v.sL, t0, L, p, true);       // rows beyond L wrote nothing
-        w.O.load(gob, go.sL, t0, L, p, true);     // and carry no gradient
+        const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step, os = ib * o_step;
+#pragma unroll
+        for (int b = 0; b < NE; b++) {
+            w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+                w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NM; b++) {
+            w.Vt[b] = vb.f4(o_vt + 64 * b, vs);
+            w.Ot[b] = gob.f4(o_ot + 64 * b, os);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Vc[b][r] = vb.f(o_vr[r] + 64 * b, vs);
+                w.Oc[b][r] = gob.f(o_or[r] + 64 * b, os);
+            }
+        }
     };
 
+    // St[mb][eb]: register r = S[16 eb + c][16 mb + 4g + r];  dS[eb][mb]: register r = dS[16 eb + 4g + r][16 mb + c]
     v4f St[NM][NE], dS[NE][NM];
 #pragma unroll
     for (int a = 0; a < NE; a++)
 #pragma unroll
         for (int b = 0; b < NM; b++) dS[a][b] = zero;
 
-    const int nblk = (L + kBlk - 1) / kBlk;
-    Raw cur, nxt;
-    load(cur, (nblk - 1) * kBlk);
-    for (int ib = nblk - 1; ib >= 0; ib--) {
-        const int t0 = ib * kBlk;
-        load(nxt, max(ib - 1, 0) * kBlk);
-        __builtin_amdgcn_sched_barrier(0);
-        const int t_end = min(t0 + kBlk, L);
-        if (t_end % chunk == 0 || t_end == L) {
+    auto block = [&](int e, const Raw &w) {
+        const int ib = nblk - 1 - e;
+        if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
 #pragma unroll
             for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-                for (int eb = 0; eb < NE; eb++) St[mb][eb] = cur.Sck[mb][eb];
+                for (int eb = 0; eb < NE; eb++) St[mb][eb] = w.Sck[mb][eb];
         }
         // state before the block, transposed: S0^T = S'^T - V^T K
 #pragma unroll
         for (int mb = 0; mb < NM; mb++) {
-            const v4f nV = -cur.V.c[mb];
+            const v4f nV = -w.Vc[mb];
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) St[mb][eb] = tn(nV, cur.K.c[eb], St[mb][eb]);
+            for (int eb = 0; eb < NE; eb++) St[mb][eb] = tn(nV, w.Kc[eb], St[mb][eb]);
         }
-        v4f QK = zero, Z = zero, Zt = zero;
+        v4f QK = zero, Z = zero;
 #pragma unroll
-        for (int b = 0; b < NE; b++) QK = tn(cur.Q.t[b], cur.K.t[b], QK);          // Q K^T   [t][s]
+        for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);          // Q K^T   [t][s]
 #pragma unroll
-        for (int b = 0; b < NM; b++) {
-            Z = tn(cur.O.t[b], cur.V.t[b], Z);            // dO V^T  [t][s]
-            Zt = tn(cur.V.t[b], cur.O.t[b], Zt);
-        }
-        v4f Pm, dPm, dPmt;
+        for (int b = 0; b < NM; b++) Z = tn(w.Ot[b], w.Vt[b], Z);            // dO V^T  [t][s]
+        v4f Pm, dPm;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const bool low = p.lo[r] || p.di[r], upp = p.up[r] || p.di[r];
+            const bool low = p.lo[r] || p.di[r];
             Pm[r] = low ? QK[r] : 0.f;
             dPm[r] = low ? Z[r] : 0.f;
-            dPmt[r] = upp ? Zt[r] : 0.f;
         }
-        const bool col_ok = t0 + c < L;
+        scratch[0].put_t(p, dPm);
 #pragma unroll
         for (int mb = 0; mb < NM; mb++) {        // g_v^T = dS^T K^T + dO^T Pm
-            v4f gVt = tn(cur.O.c[mb], Pm, zero);
+            v4f gVt = tn(w.Oc[mb], Pm, zero);
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) gVt = tn(dS[eb][mb], cur.K.t[eb], gVt);
-            if (col_ok)
-                *reinterpret_cast<float4 *>(gv + (seq * L + t0 + c) * M + 16 * mb + 4 * g) =
-                    make_float4(gVt[0], gVt[1], gVt[2], gVt[3]);
+            for (int eb = 0; eb < NE; eb++) gVt = tn(dS[eb][mb], w.Kt[eb], gVt);
+            gvb.st4(gVt, o_gm + 64 * mb, ib * m_step);
         }
+        __builtin_amdgcn_wave_barrier();
+        const v4f dPmt = scratch[0].get(lane);        // lower(dO V^T)^T
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) {
-            v4f gQt = tn(cur.K.c[eb], dPmt, zero);
-            v4f gKt = tn(cur.Q.c[eb], dPm, zero);
+            v4f gQt = tn(w.Kc[eb], dPmt, zero);
+            v4f gKt = tn(w.Qc[eb], dPm, zero);
 #pragma unroll
             for (int mb = 0; mb < NM; mb++) {
-                gQt = tn(St[mb][eb], cur.O.t[mb], gQt);
-                gKt = tn(tn(dS[eb][mb], ident, zero), cur.V.t[mb], gKt);      // dS V^T
+                LdsMat &tr = scratch[1 + (eb * NM + mb) % 3];
+                tr.put_t(p, dS[eb][mb]);
+                gQt = tn(St[mb][eb], w.Ot[mb], gQt);
+                __builtin_amdgcn_wave_barrier();
+                gKt = tn(tr.get(lane), w.Vt[mb], gKt);      // dS V^T
             }
-            if (col_ok) {
-                const int64_t o = (seq * L + t0 + c) * E + 16 * eb + 4 * g;
-                *reinterpret_cast<float4 *>(gq + o) = make_float4(gQt[0], gQt[1], gQt[2], gQt[3]);
-                *reinterpret_cast<float4 *>(gk + o) = make_float4(gKt[0], gKt[1], gKt[2], gKt[3]);
-            }
+            gqb.st4(gQt, o_ge + 64 * eb, ib * e_step);
+            gkb.st4(gKt, o_ge + 64 * eb, ib * e_step);
         }
 #pragma unroll
         for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-            for (int mb = 0; mb < NM; mb++) dS[eb][mb] = tn(cur.Q.c[eb], cur.O.c[mb], dS[eb][mb]);
-        cur = nxt;
-    }
+            for (int mb = 0; mb < NM; mb++) dS[eb][mb] = tn(w.Qc[eb], w.Oc[mb], dS[eb][mb]);
+    };
+    ring_loop<PF, Raw, false>(nblk, load, block);
 }
 
 }  // namespace

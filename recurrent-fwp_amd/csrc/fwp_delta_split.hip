@@ -27,97 +27,6 @@
 namespace fwp {
 namespace {
 
-// Workgroup barrier that orders the LDS hand-over only.  __syncthreads() also waits for every
-// global load and store of the wave, the prefetches of the coming blocks included.
-__device__ __forceinline__ void lds_barrier() {
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-}
-
-__device__ __forceinline__ v4f as_v4f(const float *ptr) {
-    const float4 x = *reinterpret_cast<const float4 *>(ptr);
-    return v4f{x.x, x.y, x.z, x.w};
-}
-__device__ __forceinline__ float4 as_float4(const v4f &x) { return make_float4(x[0], x[1], x[2], x[3]); }
-__device__ __forceinline__ v4f from_float4(const float4 &x) { return v4f{x.x, x.y, x.z, x.w}; }
-
-// A 16x16 matrix in LDS as the 64 lanes' register quadruples (1 KB).  put() followed by get() hands a
-// matrix over as it is; put_t() followed by get() hands over its transpose: lane (g, c) holds
-// X[4g + r][c], which the reader of the transpose wants in lane (c / 4, 4g + r) as register c % 4.
-// A transpose costs four scattered LDS writes instead of the four MFMAs of a product with the
-// identity.  Within one wave LDS operations execute in order, so a wave may read back what it
-// has just written without a barrier.
-struct LdsMat {
-    float4 q[64];
-    __device__ __forceinline__ void put(int lane, const v4f &x) { q[lane] = as_float4(x); }
-    __device__ __forceinline__ void put_t(const Geo16 &p, const v4f &x) {
-        float *f = reinterpret_cast<float *>(q) + 64 * (p.c / 4) + 16 * p.g + p.c % 4;
-#pragma unroll
-        for (int r = 0; r < 4; r++) f[4 * r] = x[r];
-    }
-    __device__ __forceinline__ v4f get(int lane) const { return from_float4(q[lane]); }
-};
-
-// (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At:
-// (I - At)(I + At^2)(I + At^4)(I + At^8) with the transposes of the squares taken through LDS
-// (`scratch`: two matrices owned by the calling wave), 6 products.
-__device__ __forceinline__ v4f inv_unit_triangular_lds(v4f A, v4f At, v4f identity, LdsMat *scratch,
-                                                       const Geo16 &p, int lane) {
-    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f T = identity - At;
-    const v4f A2 = tn(At, A, zero);
-    scratch[0].put_t(p, A2);
-    T = tn(A2, T, T);
-    __builtin_amdgcn_wave_barrier();
-    const v4f At2 = scratch[0].get(lane);
-    const v4f A4 = tn(At2, A2, zero);
-    scratch[1].put_t(p, A4);
-    T = tn(A4, T, T);
-    __builtin_amdgcn_wave_barrier();
-    const v4f At4 = scratch[1].get(lane);
-    const v4f A8 = tn(At4, A4, zero);
-    return tn(A8, T, T);
-}
-
-// Index of the checkpoint chunk a block lies in: block / blocks_per_chunk as a multiplication
-// (exact while block * blocks_per_chunk < 2^32), the remainder alongside.
-struct ChunkOf {
-    unsigned bpc, magic;
-    __device__ explicit ChunkOf(int chunk) : bpc(chunk / kBlk), magic(0xFFFFFFFFu / bpc + 1) {}
-    __device__ __forceinline__ unsigned operator()(unsigned block) const { return __umulhi(block, magic); }
-    // is `block` the last one of its chunk?
-    __device__ __forceinline__ bool closes(unsigned block) const {
-        return (block + 1) - (*this)(block + 1) * bpc == 0;
-    }
-};
-
-// The per-block loop of one wave: `step(e, raw)` for e = 0 .. n-1 with the data of the coming PF
-// blocks in flight in a ring of registers, one barrier per block.  `load(raw, e)` is asked for
-// e <= n - 1 only (past the end the last block is loaded again and not used).  Memory latency is
-// several block times here, so one block ahead is not enough.
-template <int PF, class Raw, class Load, class Step>
-__device__ __forceinline__ void ring_loop(int n, Load load, Step step) {
-    Raw ring[PF];
-#pragma unroll
-    for (int j = 0; j < PF; j++) load(ring[j], min(j, n - 1));
-    int e = 0;
-    for (; e + PF <= n; e += PF) {
-#pragma unroll
-        for (int j = 0; j < PF; j++) {
-            step(e + j, ring[j]);
-            load(ring[j], min(e + j + PF, n - 1));
-            __builtin_amdgcn_sched_barrier(0);     // the loads are issued here, not next to their use
-            lds_barrier();
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < PF; j++) {
-        if (e + j < n) {
-            step(e + j, ring[j]);
-            lds_barrier();
-        }
-    }
-}
-
 // ------------------------------------------------------------------ forward
 
 // What the preparing wave reads of a block.
