@@ -31,31 +31,34 @@ bool delta_chunked(int L) {
     return g_delta_kernels >= FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
 }
 
-// Several waves per sequence: measured on MI355X (1024 SIMDs) the split kernels win or tie at every
-// sequence count for D = 16 (768 sequences: 23 + 28 us against 29 + 40 us; 4096: 112 + 145 against
-// 124 + 145) and up to about a thousand sequences for D = 32 (beyond, their backward is 5-10 % slower).
-// The kernels that read through buffer resources address a sequence with 32-bit byte offsets.
+// Several waves per sequence or one, measured on MI355X (1024 SIMDs).  Backward: the split kernel
+// wins or ties at every sequence count for D = 16 (768 sequences: 28 us against 40 us; 2048: 76
+// against 77) and up to about a thousand sequences for D = 32 (beyond, it is 5-10 % slower).
+// Forward, where the one-wave kernel does not invert on the matrix cores: D = 16, the split kernel up
+// to 384 sequences (256: 14.7 us against 17.5 us), one wave beyond (512: 19.1 against 20.8; 768: 20.2
+// against 22.7; 2048: 42 against 49); D = 32 as for backward (256 sequences of 1024 steps: 64 us
+// against 117 us; 2048 of 256 steps: 129 against 108).
+// The kernels that read through buffer resources address a sequence with 32-bit byte offsets, and
+// may ask for rows up to two blocks past its end (which must not wrap around to rows that exist).
 bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
     for (const fwp_view &v : views)
-        if (v.sL < 0 || ((int64_t)L * v.sL + (E > M ? E : M)) * 4 >= (int64_t(1) << 31)) return false;
+        if (v.sL < 0 || ((int64_t)(L + 32) * v.sL + (E > M ? E : M)) * 4 >= (int64_t(1) << 31)) return false;
     return true;
 }
 
 // Shapes that have no other fast kernel (E != M, E or M above 32) always take them.
-bool delta_split(int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
+bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
                  const fwp_view &beta) {
     if (!split_delta_supported(L) || !split_delta_dims(E, M)) return false;
-    // a sequence is addressed with 32-bit byte offsets
-    const auto in_range = [&](const fwp_view &v) {
-        return v.sL >= 0 && ((int64_t)L * v.sL + (E > M ? E : M)) * 4 < (int64_t(1) << 31);
-    };
-    if (!in_range(beta)) return false;
+    if (!in_range32(L, E, M, {beta}) || !in_range32(L, E, M, views)) return false;
     for (const fwp_view &v : views)      // rows read 16 bytes at a time
-        if (!reg_view_ok(v) || !in_range(v)) return false;
+        if (!reg_view_ok(v)) return false;
     if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
     if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
-    return L >= 32 && (E == 16 || (int64_t)N * H <= 1024);
+    if (L < 32) return false;
+    if (E == 16) return !forward || (int64_t)N * H <= 384;
+    return (int64_t)N * H <= 1024;
 }
 
 }  // namespace
@@ -117,10 +120,10 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(out);
-    if (aligned && delta_split(N, H, L, E, M, {q, k, v}, beta))
+    if (aligned && delta_split(true, N, H, L, E, M, {q, k, v}, beta))
         return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned) {
-        if (delta_chunked(L))
+        if (delta_chunked(L) && in_range32(L, E, M, {q, k, v, beta}))
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
                                   (hipStream_t)stream);
         return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
@@ -139,7 +142,7 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv);
-    if (aligned && delta_split(N, H, L, E, M, {q, k, grad_out}, beta))
+    if (aligned && delta_split(false, N, H, L, E, M, {q, k, grad_out}, beta))
         return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
                                (hipStream_t)stream);
     if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) && aligned) {

@@ -24,282 +24,251 @@
 namespace fwp {
 namespace {
 
-// Per-lane element offsets inside a block (32-bit: a block spans 16 rows).
-struct LaneOffs {
-    unsigned kt, qt, bc;            // row c:       K^T and Q^T loads (+ 4g), beta
-    unsigned kr[4], vr[4], br[4];   // row 4g + r:  K, V rows (+ c), beta
+// One block of 16 steps as the forward wave reads it, one 16-byte load per lane and tile:
+// Kt[b], Qt[b], Vt[b]: register r = K[t0 + c][16b + 4g + r]   (K^T, Q^T, V^T)
+// The tiles of K and V it needs the other way round it transposes through LDS: that takes as
+// many instructions as reading them so from memory (four dwords per lane), but the wave may have 63
+// memory instructions in flight and no more, and those would be most of them.
+template <int NE, int NM>
+struct FwdRaw {
+    v4f Kt[NE], Qt[NE], Vt[NM];
 };
 
-// One block of 16 steps as loaded from memory.
-// Kt[b], Qt[b]: register r = K[t0 + c][16b + 4g + r]   (K^T, Q^T: one 16-byte load per lane)
-// Kc[b], Vc[b]: register r = K[t0 + 4g + r][16b + c]
-// bcol = beta[t0 + c], brow[r] = beta[t0 + 4g + r]
-template <int NB>
-struct RawBlock {
-    v4f Kt[NB], Qt[NB], Kc[NB], Vc[NB];
-    float bcol, brow[4];
-    // Whole block inside the sequence: uniform block base + constant lane offsets.
-    __device__ __forceinline__ void load_full(const fwp_view &q, const fwp_view &k, const fwp_view &v,
-                                              const fwp_view &beta, const float *qb, const float *kb,
-                                              const float *vb, const float *bb, const LaneOffs &o,
-                                              int t0) {
-        const float *kblk = kb + (int64_t)t0 * k.sL, *qblk = qb + (int64_t)t0 * q.sL,
-                    *vblk = vb + (int64_t)t0 * v.sL, *bblk = bb + (int64_t)t0 * beta.sL;
-        bcol = bblk[o.bc];
-#pragma unroll
-        for (int r = 0; r < 4; r++) brow[r] = bblk[o.br[r]];
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const float4 kk = *reinterpret_cast<const float4 *>(kblk + (o.kt + 16 * b));
-            const float4 qq = *reinterpret_cast<const float4 *>(qblk + (o.qt + 16 * b));
-            Kt[b] = v4f{kk.x, kk.y, kk.z, kk.w};
-            Qt[b] = v4f{qq.x, qq.y, qq.z, qq.w};
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                Kc[b][r] = kblk[o.kr[r] + 16 * b];
-                Vc[b][r] = vblk[o.vr[r] + 16 * b];
-            }
-        }
-    }
-    // Ragged last block, or a prefetch past the end: rows beyond L get loads clamped to the last
-    // row and beta = 0, so they neither write to the state nor are stored.
-    __device__ __forceinline__ void load_clamped(const fwp_view &q, const fwp_view &k,
-                                                 const fwp_view &v, const fwp_view &beta,
-                                                 const float *qb, const float *kb, const float *vb,
-                                                 const float *bb, int t0, int L, const Geo16 &p) {
-        const int64_t tc = min(t0 + p.c, L - 1);
-        bcol = t0 + p.c < L ? bb[tc * beta.sL] : 0.f;
-        int64_t tr[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            tr[r] = min(t0 + 4 * p.g + r, L - 1);
-            brow[r] = t0 + 4 * p.g + r < L ? bb[tr[r] * beta.sL] : 0.f;
-        }
-#pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const float4 kk = *reinterpret_cast<const float4 *>(kb + tc * k.sL + 16 * b + 4 * p.g);
-            const float4 qq = *reinterpret_cast<const float4 *>(qb + tc * q.sL + 16 * b + 4 * p.g);
-            Kt[b] = v4f{kk.x, kk.y, kk.z, kk.w};
-            Qt[b] = v4f{qq.x, qq.y, qq.z, qq.w};
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                Kc[b][r] = kb[tr[r] * k.sL + 16 * b + p.c];
-                Vc[b][r] = vb[tr[r] * v.sL + 16 * b + p.c];
-            }
-        }
-    }
+constexpr int kGrp = 4;     // blocks whose triangular systems are solved together, one per 16 lanes
+
+// What the solve of a group of blocks reads: K^T of each block and beta[t0 + c].
+template <int NE>
+struct SolveRaw {
+    v4f Kt[kGrp][NE];
+    float bcol[kGrp];
 };
 
-// What a block contributes that does not depend on the state.
-struct PreBlock {
-    v4f Tt;   // (I + A)^-T
-    v4f Gu;   // strict_lower(K K^T)^T
-    v4f Rm;   // lower(Q K^T)^T
-};
+// Forward, one wave per sequence.  The inverses T = (I + A)^-1 are not multiplied out on the matrix
+// cores (six products per block): T (I + A) = I is solved by substitution, column by column from
+// the right, T[c][j] = [c == j] - sum_{i > j} T[c][i] b_i G[i][j] with G = K K^T, 120 multiply-adds
+// per row.  Lane 16 jb + c does row c of block jb of a group of four blocks, reading G and beta
+// from LDS (the 16 lanes of a block read the same address).  What is left for the matrix cores
+// per block: G, lower(Q K^T) and the five products that involve the state.
+//
+// Four sequences per workgroup, one wave each: the waves of a 256-thread workgroup are placed on
+// the four SIMDs of a CU, one each, whereas one-wave workgroups sometimes land two on one SIMD
+// while another SIMD of the CU stays empty (and which, depends on what ran before).
+constexpr int kSeqPerWg = 4;
 
-template <int NB>   // NB = D / 16
-__global__ __launch_bounds__(64) void k_delta_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
+template <int NE, int NM>   // state E = 16 NE by M = 16 NM
+__global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
                                                        fwp_view beta, float *__restrict__ W,
                                                        float *__restrict__ out,
                                                        float *__restrict__ vdiff,
                                                        float *__restrict__ ckpt,
-                                                       float *__restrict__ aux, int H, int L,
-                                                       int chunk, int nchunk) {
-    constexpr int D = 16 * NB;
-    const Geo16 p(threadIdx.x);
+                                                       float *__restrict__ aux, int nseq, int H,
+                                                       int L, int chunk, int nchunk) {
+    constexpr int E = 16 * NE, M = 16 * NM;
+    // per wave: K K^T per block of the group in the accumulator layout, 64 lanes + 4 of padding so
+    // that the four blocks' reads fall on different banks; beta likewise
+    __shared__ float4 gm_[kSeqPerWg][kGrp][68];
+    __shared__ float bl_[kSeqPerWg][kGrp][20];
+    __shared__ LdsMat tm_[kSeqPerWg][kGrp];         // (I + A)^-T per block of the group
+    __shared__ LdsMat tr_[kSeqPerWg][3];            // for transposes
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    auto &gm = gm_[wave];
+    auto &bl = bl_[wave];
+    auto &tm = tm_[wave];
+    auto &tr = tr_[wave];
+    const int lane = threadIdx.x % 64;
+    const Geo16 p(lane);
     const int g = p.g, c = p.c;
-    const int64_t seq = blockIdx.x;
+    const int64_t seq = (int64_t)blockIdx.x * kSeqPerWg + wave;
+    if (seq >= nseq) return;
     const int n = (int)(seq / H), h = (int)(seq % H);
+    const int nblk = (L + kBlk - 1) / kBlk, ngrp = (nblk + kGrp - 1) / kGrp;
     // aux (with ckpt): a header whose first float says that the per-block matrices T = (I + A)^-1
-    // follow, row-major, [sequence][block][16][16]; backward then does not invert again.
-    if (aux && seq == 0 && threadIdx.x == 0) aux[0] = 1.f;
-    float *aux_T = aux ? aux + kAuxHeader + seq * ((L + kBlk - 1) / kBlk) * 256 + c * 16 + 4 * g : nullptr;
-    auto save_T = [&](int ib, const v4f &Tt) {   // register r = T[c][4g + r]
-        if (aux_T) *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = make_float4(Tt[0], Tt[1], Tt[2], Tt[3]);
-    };
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *vb = row(v, n, h, 0),
-                *bb = row(beta, n, h, 0);
+    // follow, row-major, [sequence][block][16][16]; backward then does not invert.
+    if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
+        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
+        ob(out + seq * L * M, (uint32_t)(L * M * 4)),
+        db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0),
+        tb(aux ? aux + kAuxHeader + seq * nblk * 256 : nullptr, aux ? (uint32_t)(nblk * 1024) : 0);
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
+                   m_step = (unsigned)(kBlk * M * 4);
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                   o_bc = (unsigned)(c * beta.sL) * 4;
+    const unsigned o_vt = (unsigned)(c * v.sL + 4 * g) * 4, o_out = (unsigned)(c * M + 4 * g) * 4;
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    LaneOffs lo;
-    lo.kt = (unsigned)(c * k.sL + 4 * g);
-    lo.qt = (unsigned)(c * q.sL + 4 * g);
-    lo.bc = (unsigned)(c * beta.sL);
+    // A block past the end is read at index nblk: every row beyond the buffers, all zeros.
+    auto load = [&](FwdRaw<NE, NM> &w, int ib) {
+        ib = min(ib, nblk);
+        const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step;
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        lo.kr[r] = (unsigned)((4 * g + r) * k.sL + c);
-        lo.vr[r] = (unsigned)((4 * g + r) * v.sL + c);
-        lo.br[r] = (unsigned)((4 * g + r) * beta.sL);
-    }
-    auto load_block = [&](RawBlock<NB> &raw, int t0) {
-        if (t0 + kBlk <= L) raw.load_full(q, k, v, beta, qb, kb, vb, bb, lo, t0);
-        else raw.load_clamped(q, k, v, beta, qb, kb, vb, bb, t0, L, p);
+        for (int b = 0; b < NE; b++) {
+            w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+        }
+#pragma unroll
+        for (int b = 0; b < NM; b++) w.Vt[b] = vb.f4(o_vt + 64 * b, vs);
+    };
+    auto load_group = [&](SolveRaw<NE> &w, int m) {
+#pragma unroll
+        for (int j = 0; j < kGrp; j++) {
+            const int ib = min(kGrp * m + j, nblk);
+            w.bcol[j] = bb.f(o_bc, ib * b_step);
+#pragma unroll
+            for (int b = 0; b < NE; b++) w.Kt[j][b] = kb.f4(o_kt + 64 * b, ib * k_step);
+        }
+    };
+    // group m: G of its blocks to LDS, the solve, (I + A)^-T to LDS
+    auto solve = [&](const SolveRaw<NE> &w, int m) {
+#pragma unroll
+        for (int j = 0; j < kGrp; j++) {
+            v4f G = zero;
+#pragma unroll
+            for (int b = 0; b < NE; b++) G = tn(w.Kt[j][b], w.Kt[j][b], G);
+            gm[j][lane] = as_float4(G);
+            if (g == 0) bl[j][c] = w.bcol[j];
+        }
+        __builtin_amdgcn_wave_barrier();
+        const float4 *gq = gm[g];
+        float be[16], T[16], Wn[16];
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const float4 b4 = *reinterpret_cast<const float4 *>(&bl[g][4 * a]);
+            be[4 * a] = b4.x, be[4 * a + 1] = b4.y, be[4 * a + 2] = b4.z, be[4 * a + 3] = b4.w;
+        }
+#pragma unroll
+        for (int jj = 15; jj >= 0; jj--) {
+            float acc = c == jj ? 1.f : 0.f;
+#pragma unroll
+            for (int a = (jj + 1) / 4; a < 4; a++) {
+                const float4 g4 = gq[16 * a + jj];          // G[4a .. 4a + 3][jj]
+                const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+                for (int x = 0; x < 4; x++)
+                    if (4 * a + x > jj) acc = fmaf(Wn[4 * a + x], gg[x], acc);
+            }
+            T[jj] = acc;
+            Wn[jj] = -(acc * be[jj]);
+        }
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const v4f t4 = {T[4 * a], T[4 * a + 1], T[4 * a + 2], T[4 * a + 3]};
+            tm[g].at(16 * a + c) = as_float4(t4);          // read back as register r = T[c][4g' + r] by lane (g', c)
+        }
+        __builtin_amdgcn_wave_barrier();
     };
 
     // state block [eb][mb]: register r holds S[16*eb + 4g + r][16*mb + c]
-    v4f S[NB][NB];
+    v4f S[NE][NM];
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++)
+        for (int mb = 0; mb < NM; mb++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                S[eb][mb][r] = W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c];
+                S[eb][mb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
+    const ChunkOf chunk_of(chunk);
 
-    // The state-independent products of a block, in four stages so that the caller can place the
-    // sequential products of the previous block between them (the matrix pipe runs in order; two
-    // independent chains interleaved keep it busy while each waits for its own results).
-    v4f G, R, N, Nt, N2, Nt2, N4, Nt4;
-    auto pre_stage = [&](int stage, const RawBlock<NB> &raw, PreBlock &pre) {
-        if (stage == 0) {
-            G = zero;
-            R = zero;
+    // block ib, the j-th of its group
+    auto block = [&](int ib, const FwdRaw<NE, NM> &w, int j) {
+        v4f R = zero, Rm;
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
-                G = tn(raw.Kt[b], raw.Kt[b], G);       // K K^T
-                R = tn(raw.Kt[b], raw.Qt[b], R);       // K Q^T  [s][t]
-            }
-        } else if (stage == 1) {
+        for (int eb = 0; eb < NE; eb++) R = tn(w.Kt[eb], w.Qt[eb], R);      // K Q^T  [s][t]
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                N[r] = p.lo[r] ? raw.brow[r] * G[r] : 0.f;        // A
-                Nt[r] = p.up[r] ? raw.bcol * G[r] : 0.f;          // A^T
-                pre.Gu[r] = p.up[r] ? G[r] : 0.f;
-                pre.Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
-                pre.Tt[r] = (p.di[r] ? 1.f : 0.f) - Nt[r];        // I - A^T
-            }
-            N2 = tn(Nt, N, zero);                                 // A^2
-            Nt2 = tn(N, Nt, zero);                                // (A^T)^2
-        } else if (stage == 2) {
-            pre.Tt = tn(N2, pre.Tt, pre.Tt);                      // (I + (A^T)^2)(I - A^T)
-            N4 = tn(Nt2, N2, zero);
-            Nt4 = tn(N2, Nt2, zero);
-        } else {
-            pre.Tt = tn(N4, pre.Tt, pre.Tt);
-            const v4f N8 = tn(Nt4, N4, zero);
-            pre.Tt = tn(N8, pre.Tt, pre.Tt);                      // (I + A)^-T
-        }
-    };
-
-    const int nblk = (L + kBlk - 1) / kBlk;
-
-    // One block: the sequential products of block ib (raw data `cur`, state-independent part
-    // `pre_cur`) interleaved with the stages of block ib + 1 (`nxt` -> `pre_nxt`), while the loads of
-    // block ib + 2 (`fut`) are in flight.  Everything past the end is clamped and its results unused,
-    // so the body is one basic block for the scheduler.
-    // Results of a block are kept in registers and stored at the top of the next block, right
-    // after its prefetch loads: the memory counter is shared by loads and stores and waits on it
-    // come out as "everything outstanding", so a store must be a block old by the time the next
-    // wait comes or that wait pays the store's latency.
-    v4f pend_O[NB], pend_D[NB], pend_T;
-    auto flush = [&](auto full_tag, int ib) {        // stores of block ib; S still is the state after it
-        constexpr bool FULL = decltype(full_tag)::value;
-        const int t0 = ib * kBlk;
+        for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+        // register r = K[t0 + 4g + r][16 eb + c], V likewise
+        v4f Kc[NE], Vc[NM];
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
-            if (FULL || t0 + c < L)         // register r = O[t0 + c][16mb + 4g + r]
-                *reinterpret_cast<float4 *>(out + (seq * L + t0 + c) * D + 16 * mb + 4 * g) =
-                    make_float4(pend_O[mb][0], pend_O[mb][1], pend_O[mb][2], pend_O[mb][3]);
-            if (vdiff) {
-#pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (FULL || t0 + 4 * g + r < L)
-                        vdiff[(seq * L + t0 + 4 * g + r) * D + 16 * mb + c] = pend_D[mb][r];
-            }
-        }
-        if (t0 + kBlk < L) save_T(ib + 1, pend_T);
-        const int t_end = min(t0 + kBlk, L);
-        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
-            float *dst = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
-#pragma unroll
-            for (int eb = 0; eb < NB; eb++)
-#pragma unroll
-                for (int mb = 0; mb < NB; mb++)
-#pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        dst[(16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
-        }
-    };
-
-    auto block = [&](auto full_tag, int ib, const RawBlock<NB> &cur, const RawBlock<NB> &nxt,
-                     RawBlock<NB> &fut, const PreBlock &pre_cur, PreBlock &pre_nxt) {
-        constexpr bool FULL = decltype(full_tag)::value;   // blocks ib .. ib+2 lie inside the sequence
-        const int t0 = ib * kBlk;
-        if constexpr (FULL) fut.load_full(q, k, v, beta, qb, kb, vb, bb, lo, t0 + 2 * kBlk);
-        else fut.load_clamped(q, k, v, beta, qb, kb, vb, bb, t0 + 2 * kBlk, L, p);
-        if (ib > 0) flush(std::true_type(), ib - 1);
-        // loads and stores stay here, a whole block ahead of the next wait
-        __builtin_amdgcn_sched_barrier(0);
-
-        v4f X[NB], U[NB], Ot[NB];
-#pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
-            v4f KS = zero;
-#pragma unroll
-            for (int eb = 0; eb < NB; eb++) KS = tn(cur.Kt[eb], S[eb][mb], KS);
-            X[mb] = cur.Vc[mb] - KS;
-        }
-        pre_stage(0, nxt, pre_nxt);
-#pragma unroll
-        for (int mb = 0; mb < NB; mb++) {                 // O^T, state part (old state)
-            Ot[mb] = zero;
-#pragma unroll
-            for (int eb = 0; eb < NB; eb++) Ot[mb] = tn(S[eb][mb], cur.Qt[eb], Ot[mb]);
+        for (int eb = 0; eb < NE; eb++) {
+            tr[eb % 2].put_t(p, w.Kt[eb]);
+            Kc[eb] = tr[eb % 2].get(lane);
         }
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
+            tr[(NE + mb) % 2].put_t(p, w.Vt[mb]);
+            Vc[mb] = tr[(NE + mb) % 2].get(lane);
+        }
+        const v4f Tt = tm[j].get(lane);
+        tb.st4(Tt, (unsigned)(c * 16 + 4 * g) * 4, (unsigned)ib * 1024);      // whole rows of T per instruction
+        const v4f brow = from_float4(*reinterpret_cast<const float4 *>(&bl[j][4 * g]));   // beta[t0 + 4g + r]
+        const bool beta_nonzero =
+            __builtin_amdgcn_ballot_w64(brow[0] == 0.f || brow[1] == 0.f || brow[2] == 0.f || brow[3] == 0.f) == 0;
+#pragma unroll
+        for (int mb = 0; mb < NM; mb++) {
+            v4f KS = zero, Ot = zero;
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) KS = tn(w.Kt[eb], S[eb][mb], KS);
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb][mb], w.Qt[eb], Ot);    // O^T, state part (old state)
+            const v4f X = Vc[mb] - KS;
             v4f Y;
 #pragma unroll
-            for (int r = 0; r < 4; r++) Y[r] = cur.brow[r] * X[mb][r];
-            U[mb] = tn(pre_cur.Tt, Y, zero);
+            for (int r = 0; r < 4; r++) Y[r] = brow[r] * X[r];
+            const v4f U = tn(Tt, Y, zero);
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) S[eb][mb] = tn(Kc[eb], U, S[eb][mb]);
+            const v4f O = tn(U, Rm, Ot);          // register r = O[t0 + c][16 mb + 4g + r]
+            ob.st4(O, o_out + 64 * mb, ib * m_step);
+            if (vdiff) {
+                // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division
+                // where no beta of the block is zero (rows past the end read beta = 0)
+                v4f Dd;
+                if (beta_nonzero) {
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Dd[r] = U[r] * __builtin_amdgcn_rcpf(brow[r]);
+                } else {
+                    const v4f G = from_float4(gm[j][lane]);
+                    v4f Gu;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Gu[r] = p.up[r] ? G[r] : 0.f;
+                    Dd = X - tn(Gu, U, zero);
+                }
+                tr[2].put_t(p, Dd);        // leaves like O
+                db.st4(tr[2].get(lane), o_out + 64 * mb, ib * m_step);
+            }
         }
-        pre_stage(1, nxt, pre_nxt);
+        if (ckpt && ib < nblk && (chunk_of.closes(ib) || ib + 1 == nblk)) {
+            float *dst = ckpt + (seq * nchunk + chunk_of(ib)) * E * M;
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++)
+            for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) S[eb][mb] = tn(cur.Kc[eb], U[mb], S[eb][mb]);
-        pre_stage(2, nxt, pre_nxt);
+                for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
-            pend_O[mb] = tn(U[mb], pre_cur.Rm, Ot[mb]);
-        }
-        pre_stage(3, nxt, pre_nxt);
-        pend_T = pre_nxt.Tt;
-        if (vdiff) {
-#pragma unroll
-            for (int mb = 0; mb < NB; mb++) pend_D[mb] = X[mb] - tn(pre_cur.Gu, U[mb], zero);
+                    for (int r = 0; r < 4; r++) dst[(16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
         }
     };
 
-    // Main loop: the blocks whose prefetch (two blocks on) still lies inside the sequence; the last
-    // blocks take the clamped variant.
-    RawBlock<NB> cur, nxt, fut;
-    PreBlock pre_cur, pre_nxt;
-    load_block(cur, 0);
-    load_block(nxt, kBlk);
+    // Blocks in groups of four, the last group filled up with empty blocks; the rows of the next
+    // four blocks and the K^T of the next group are in flight while a group is worked on.
+    SolveRaw<NE> sr;
+    FwdRaw<NE, NM> ring[kGrp];
+    load_group(sr, 0);
 #pragma unroll
-    for (int st = 0; st < 4; st++) pre_stage(st, cur, pre_cur);
-    save_T(0, pre_cur.Tt);
-    int ib = 0;
-    for (; (ib + 3) * kBlk <= L; ib++) {
-        block(std::true_type(), ib, cur, nxt, fut, pre_cur, pre_nxt);
-        cur = nxt;
-        nxt = fut;
-        pre_cur = pre_nxt;
+    for (int j = 0; j < kGrp; j++) load(ring[j], j);
+    solve(sr, 0);
+    load_group(sr, 1);
+    for (int m = 0; m < ngrp; m++) {
+#pragma unroll
+        for (int j = 0; j < kGrp; j++) {
+            block(kGrp * m + j, ring[j], j);
+            load(ring[j], kGrp * (m + 1) + j);
+            __builtin_amdgcn_sched_barrier(0);     // the loads are issued here, not next to their use
+        }
+        if (m + 1 < ngrp) {
+            solve(sr, m + 1);
+            load_group(sr, m + 2);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
-    for (; ib < nblk; ib++) {
-        block(std::false_type(), ib, cur, nxt, fut, pre_cur, pre_nxt);
-        cur = nxt;
-        nxt = fut;
-        pre_cur = pre_nxt;
-    }
-    flush(std::false_type(), nblk - 1);
 #pragma unroll
-    for (int eb = 0; eb < NB; eb++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++)
+        for (int mb = 0; mb < NM; mb++)
 #pragma unroll
             for (int r = 0; r < 4; r++)
-                W[(seq * D + 16 * eb + 4 * g + r) * D + 16 * mb + c] = S[eb][mb][r];
+                W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c] = S[eb][mb][r];
 }
 
 // ----------------------------------------------------------------- backward
@@ -897,11 +866,13 @@ int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, 
     const int nchunk = (L + chunk - 1) / chunk;
     float *aux = delta_aux_of(ckpt, N, H, L, D, D, chunk);
     if (D == 16)
-        hipLaunchKernelGGL(k_delta_fwd_mfma<1>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
-                           vdiff, ckpt, aux, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_fwd_mfma<1, 1>), dim3((N * H + kSeqPerWg - 1) / kSeqPerWg),
+                           dim3(64 * kSeqPerWg), 0, s, q, k, v, beta, W, out, vdiff, ckpt, aux, N * H, H, L, chunk,
+                           nchunk);
     else
-        hipLaunchKernelGGL(k_delta_fwd_mfma<2>, dim3(N * H), dim3(64), 0, s, q, k, v, beta, W, out,
-                           vdiff, ckpt, aux, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_fwd_mfma<2, 2>), dim3((N * H + kSeqPerWg - 1) / kSeqPerWg),
+                           dim3(64 * kSeqPerWg), 0, s, q, k, v, beta, W, out, vdiff, ckpt, aux, N * H, H, L, chunk,
+                           nchunk);
     return (int)hipGetLastError();
 }
 

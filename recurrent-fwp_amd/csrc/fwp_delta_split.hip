@@ -54,6 +54,9 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
                                                                   float *__restrict__ aux, int H, int L,
                                                                   int chunk, int nchunk) {
     constexpr int E = 16 * NE, M = 16 * NM;
+    // lower(Q K^T)^T: with one state wave that wave forms it itself (the preparing wave is the
+    // busier one), with several the preparing wave does it once for all
+    constexpr bool kPrepQK = NM > 1;
     // slot, matrix (0: (I + A)^-T, 1: strict_lower(K K^T)^T, 2: lower(Q K^T)^T), lane
     __shared__ LdsMat xch[2][3];
     __shared__ LdsMat scratch[2];       // the preparing wave's
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
             for (int b = 0; b < NE; b++) {
                 w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
-                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+                if constexpr (kPrepQK) w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
             }
         };
         auto prepare = [&](const PrepRaw<NE> &w, int ib) {
@@ -104,7 +107,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
             for (int b = 0; b < NE; b++) {
                 G = tn(w.Kt[b], w.Kt[b], G);       // K K^T
-                R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
+                if constexpr (kPrepQK) R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
             }
             v4f A, At, Gu, Rm;
 #pragma unroll
@@ -118,7 +121,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
             LdsMat *slot = xch[ib & 1];
             slot[0].put(lane, Tt);
             slot[1].put(lane, Gu);
-            slot[2].put(lane, Rm);
+            if constexpr (kPrepQK) slot[2].put(lane, Rm);
             if (aux_T)       // register r = T[c][4g + r]
                 *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = as_float4(Tt);
         };
@@ -187,12 +190,30 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         const v4f U = tn(Tt, Y, zero);
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
-        const v4f Rm = slot[2].get(lane);
+        v4f Rm;
+        if constexpr (kPrepQK) {
+            Rm = slot[2].get(lane);
+        } else {
+            v4f R = zero;
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) R = tn(cur.Kt[eb], cur.Qt[eb], R);
+#pragma unroll
+            for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+        }
         const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
         ob.st4(O, o_out, ib * m_step);
         if (vdiff) {
-            const v4f Gu = slot[1].get(lane);
-            const v4f Dd = X - tn(Gu, U, zero);
+            // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division where no
+            // beta of the block is zero (rows past the end of the sequence read beta = 0)
+            v4f Dd;
+            if (__builtin_amdgcn_ballot_w64(cur.brow[0] == 0.f || cur.brow[1] == 0.f || cur.brow[2] == 0.f ||
+                                            cur.brow[3] == 0.f) == 0) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) Dd[r] = U[r] * __builtin_amdgcn_rcpf(cur.brow[r]);
+            } else {
+                const v4f Gu = slot[1].get(lane);
+                Dd = X - tn(Gu, U, zero);
+            }
 #pragma unroll
             for (int r = 0; r < 4; r++) db.st(Dd[r], o_vd + r * M * 4, ib * m_step);
         }

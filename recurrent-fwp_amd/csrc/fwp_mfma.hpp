@@ -93,21 +93,25 @@ __device__ __forceinline__ void lds_barrier() {
 __device__ __forceinline__ float4 as_float4(const v4f &x) { return make_float4(x[0], x[1], x[2], x[3]); }
 __device__ __forceinline__ v4f from_float4(const float4 &x) { return v4f{x.x, x.y, x.z, x.w}; }
 
-// A 16x16 matrix in LDS as the 64 lanes' register quadruples (1 KB).  put() followed by get() hands a
+// A 16x16 matrix in LDS as the 64 lanes' register quadruples.  put() followed by get() hands a
 // matrix over as it is; put_t() followed by get() hands over its transpose: lane (g, c) holds
 // X[4g + r][c], which the reader of the transpose wants in lane (c / 4, 4g + r) as register c % 4.
 // A transpose costs four scattered LDS writes instead of the four MFMAs of a product with the
-// identity.  Within one wave LDS operations execute in order, so a wave may read back what it
-// has just written without a barrier.
+// identity; each group of 16 lanes is followed by 16 bytes of padding, which spreads those
+// writes over all banks.  Within one wave LDS operations execute in order, so a wave may read
+// back what it has just written without a barrier.
 struct LdsMat {
-    float4 q[64];
-    __device__ __forceinline__ void put(int lane, const v4f &x) { q[lane] = as_float4(x); }
+    float4 q[68];
+    // where lane `l` keeps its quadruple
+    __device__ __forceinline__ float4 &at(int l) { return q[l + l / 16]; }
+    __device__ __forceinline__ const float4 &at(int l) const { return q[l + l / 16]; }
+    __device__ __forceinline__ void put(int lane, const v4f &x) { at(lane) = as_float4(x); }
     __device__ __forceinline__ void put_t(const Geo16 &p, const v4f &x) {
-        float *f = reinterpret_cast<float *>(q) + 64 * (p.c / 4) + 16 * p.g + p.c % 4;
+        float *f = reinterpret_cast<float *>(q) + 68 * (p.c / 4) + 16 * p.g + p.c % 4;
 #pragma unroll
         for (int r = 0; r < 4; r++) f[4 * r] = x[r];
     }
-    __device__ __forceinline__ v4f get(int lane) const { return from_float4(q[lane]); }
+    __device__ __forceinline__ v4f get(int lane) const { return from_float4(at(lane)); }
 };
 
 // (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At:
