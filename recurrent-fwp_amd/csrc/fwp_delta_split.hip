@@ -277,10 +277,14 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
                                                              int chunk, int nchunk) {
     constexpr int E = 16 * NE, M = 16 * NM;
     constexpr int kDX = NE, kDPm = NE + 1, kDPmt = NE + 2, kNM = NE + 3, kNMt = NE + 4;
+    // lower(dO U^T): with one state wave that wave forms it itself from rows it reads anyway (the
+    // adjoint waves are the busier ones), with several the adjoint waves do it once for all
+    constexpr bool kStateDPm = NE == 1;
     // slot, adjoint wave, matrix: blocks eb = 0..NE-1 of dS^T, then dX^T, dPm, dPm^T,
     // -strict_lower(dX U^T) and its transpose
     __shared__ LdsMat xch[2][NM][NE + 5];
     __shared__ LdsMat scratch[NM][2];       // the adjoint waves'
+    __shared__ LdsMat own_[NE];             // the state waves'
     __shared__ float gbx[2][NM][16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
@@ -395,7 +399,8 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
                 dS[eb] = tn(w.Qc[eb], w.Oc, dS[eb]);
                 dS[eb] = tn(w.Kc[eb], ndX, dS[eb]);
             }
-            const v4f Z = tn(w.Ot, Ut, zero);      // dO U^T
+            v4f Z = zero;
+            if constexpr (!kStateDPm) Z = tn(w.Ot, Ut, zero);      // dO U^T
             __builtin_amdgcn_wave_barrier();
             const v4f dYt = scratch[mb][0].get(lane);
             const v4f dXt = w.bcol * dYt;
@@ -421,8 +426,10 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
                 dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
                 nM[r] = p.lo[r] ? -M[r] : 0.f;
             }
-            slot[kDPm].put(lane, dPm);
-            slot[kDPmt].put_t(p, dPm);
+            if constexpr (!kStateDPm) {
+                slot[kDPm].put(lane, dPm);
+                slot[kDPmt].put_t(p, dPm);
+            }
             slot[kNM].put(lane, nM);
             slot[kNMt].put_t(p, nM);
         };
@@ -433,6 +440,7 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
 
     // ---------------------------------------------------- state wave of key columns [16 eb, 16 eb + 16)
     const int eb = wave - NM;
+    LdsMat *own = &own_[eb];
     const unsigned o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4;
     unsigned o_kr[4], o_qr[4], o_dr[4];
 #pragma unroll
@@ -496,11 +504,22 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
         // what the adjoint waves left for this block
         v4f dPm = zero, dPmt = zero, nMs = zero;
         float gb = 0.f;
+        if constexpr (kStateDPm) {
+            v4f Z = zero;
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) Z = tn(w.Ot[mb], Ut[mb], Z);      // dO U^T
+#pragma unroll
+            for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
+            own[0].put_t(p, dPm);
+            dPmt = own[0].get(lane);
+        }
 #pragma unroll
         for (int mb = 0; mb < NM; mb++) {
             const LdsMat *slot = xch[ib & 1][mb];
-            dPm += slot[kDPm].get(lane);
-            dPmt += slot[kDPmt].get(lane);
+            if constexpr (!kStateDPm) {
+                dPm += slot[kDPm].get(lane);
+                dPmt += slot[kDPmt].get(lane);
+            }
             nMs += slot[kNM].get(lane) + slot[kNMt].get(lane);
             gb += gbx[ib & 1][mb][c];
             const v4f dSt = slot[eb].get(lane), dXt = slot[kDX].get(lane);     // dSt: block (mb, eb) of dS^T
