@@ -472,8 +472,11 @@ def run_single_steps(args, pkg):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps (default 2000; 200 for the language model)")
+    ap.add_argument("--warmup", type=int, default=None,
+                    help="untimed steps before them (default a tenth of --steps: a step takes ~50 us and "
+                         "the first milliseconds on a cold GPU run 10 %% slower)")
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["lm", "step"], default="delta")
     ap.add_argument("--cpu-reps", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -486,6 +489,10 @@ def main():
                     help="only run five device-to-device copies of 2 GiB (a kernel of known traffic for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
+    if args.steps is None:
+        args.steps = 200 if args.workload == "lm" else 2000
+    if args.warmup is None:
+        args.warmup = max(args.steps // 10, 1)
     if args.copy_calibration:
         import torch
         src = torch.ones(512 * 1024 * 1024, device="cuda:0")      # 2 GiB: far beyond every cache level

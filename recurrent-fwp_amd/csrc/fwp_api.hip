@@ -31,13 +31,15 @@ bool delta_chunked(int L) {
     return g_delta_kernels >= FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
 }
 
-// Several waves per sequence or one, measured on MI355X (1024 SIMDs).  Backward: the split kernel
-// wins or ties at every sequence count for D = 16 (768 sequences: 28 us against 40 us; 2048: 76
-// against 77) and up to about a thousand sequences for D = 32 (beyond, it is 5-10 % slower).
-// Forward, where the one-wave kernel does not invert on the matrix cores: D = 16, the split kernel up
-// to 384 sequences (256: 14.7 us against 17.5 us), one wave beyond (512: 19.1 against 20.8; 768: 20.2
-// against 22.7; 2048: 42 against 49); D = 32 as for backward (256 sequences of 1024 steps: 64 us
-// against 117 us; 2048 of 256 steps: 129 against 108).
+// Several waves per sequence or one, measured on MI355X (1024 SIMDs) as the time of a training step
+// (what runs before a kernel changes where its waves land, so kernels timed alone mislead).
+// Backward: the split kernel wins or ties at every sequence count for D = 16 (768 sequences: 28 us
+// against 40 us; 2048: 76 against 77) and up to about a thousand sequences for D = 32 (beyond, it is
+// 5-10 % slower).  Forward: the split kernel up to about a thousand sequences (D = 16, step of forward
+// + backward at 512 / 768 / 1024 sequences of 256 steps: 41.4 / 43.5 / 49.6 us against 44.3 / 46.7 /
+// 50.8 us with the one-wave forward; D = 32, 256 sequences of 1024 steps: 64 us against 117 us), one
+// wave beyond (D = 16, 2048 sequences: 113 us against 123 us; D = 32, 2048 of 256 steps: 108 against
+// 129).
 // The kernels that read through buffer resources address a sequence with 32-bit byte offsets, and
 // may ask for rows up to two blocks past its end (which must not wrap around to rows that exist).
 bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
@@ -57,7 +59,7 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
     if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
     if (L < 32) return false;
-    if (E == 16) return !forward || (int64_t)N * H <= 384;
+    if (E == 16 && !forward) return true;
     return (int64_t)N * H <= 1024;
 }
 

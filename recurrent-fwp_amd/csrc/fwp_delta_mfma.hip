@@ -34,8 +34,6 @@ struct FwdRaw {
     v4f Kt[NE], Qt[NE], Vt[NM];
 };
 
-constexpr int kGrp = 4;     // blocks whose triangular systems are solved together, one per 16 lanes
-
 // What the solve of a group of blocks reads: K^T of each block and beta[t0 + c].
 template <int NE>
 struct SolveRaw {
@@ -44,30 +42,24 @@ struct SolveRaw {
 };
 
 // Forward, one wave per sequence.  The inverses T = (I + A)^-1 are not multiplied out on the matrix
-// cores (six products per block): T (I + A) = I is solved by substitution, column by column from
-// the right, T[c][j] = [c == j] - sum_{i > j} T[c][i] b_i G[i][j] with G = K K^T, 120 multiply-adds
-// per row.  Lane 16 jb + c does row c of block jb of a group of four blocks, reading G and beta
-// from LDS (the 16 lanes of a block read the same address).  What is left for the matrix cores
-// per block: G, lower(Q K^T) and the five products that involve the state.
+// cores: the triangular systems of four blocks at a time are solved by substitution (SolveRow).
+// What is left for the matrix cores per block: G = K K^T, lower(Q K^T) and the five products that
+// involve the state.
 //
 // Up to four sequences per workgroup, one wave each (blockDim.x / 64 of them): the waves of a
 // workgroup are placed on different SIMDs of a CU, whereas one-wave workgroups sometimes land two
 // on one SIMD while another SIMD of the CU stays empty (and which, depends on what ran before).
-// The host picks the smallest number that needs no more workgroups than there are CUs.
 constexpr int kSeqPerWg = 4;
 constexpr int kCUs = 256;
+// the smallest number that needs no more workgroups than there are CUs
 inline int seq_per_wg(int nseq) { return nseq >= kSeqPerWg * kCUs ? kSeqPerWg : (nseq + kCUs - 1) / kCUs; }
 
 // LDS of one wave of the forward kernel
 struct FwdLds {
-    // K K^T per block of the group in the accumulator layout, 64 lanes + 4 of padding so that the
-    // four blocks' reads fall on different banks; beta likewise
-    float4 gm[kGrp][68];
-    float bl[kGrp][20];
+    SolveLds solve;
     LdsMat tm[kGrp];         // (I + A)^-T per block of the group
     LdsMat tr[3];            // for transposes
 };
-
 template <int NE, int NM>   // state E = 16 NE by M = 16 NM
 __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
                                                        fwp_view beta, float *__restrict__ W,
@@ -80,8 +72,8 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
     extern __shared__ __align__(16) unsigned char dyn_lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     FwdLds &lds = reinterpret_cast<FwdLds *>(dyn_lds)[wave];
-    auto &gm = lds.gm;
-    auto &bl = lds.bl;
+    auto &gm = lds.solve.gm;
+    auto &bl = lds.solve.bl;
     auto &tm = lds.tm;
     auto &tr = lds.tr;
     const int lane = threadIdx.x % 64;
@@ -136,36 +128,13 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
             v4f G = zero;
 #pragma unroll
             for (int b = 0; b < NE; b++) G = tn(w.Kt[j][b], w.Kt[j][b], G);
-            gm[j][lane] = as_float4(G);
-            if (g == 0) bl[j][c] = w.bcol[j];
+            lds.solve.put(j, lane, p, G, w.bcol[j]);
         }
         __builtin_amdgcn_wave_barrier();
-        const float4 *gq = gm[g];
-        float be[16], T[16], Wn[16];
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-            const float4 b4 = *reinterpret_cast<const float4 *>(&bl[g][4 * a]);
-            be[4 * a] = b4.x, be[4 * a + 1] = b4.y, be[4 * a + 2] = b4.z, be[4 * a + 3] = b4.w;
-        }
-#pragma unroll
-        for (int jj = 15; jj >= 0; jj--) {
-            float acc = c == jj ? 1.f : 0.f;
-#pragma unroll
-            for (int a = (jj + 1) / 4; a < 4; a++) {
-                const float4 g4 = gq[16 * a + jj];          // G[4a .. 4a + 3][jj]
-                const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
-#pragma unroll
-                for (int x = 0; x < 4; x++)
-                    if (4 * a + x > jj) acc = fmaf(Wn[4 * a + x], gg[x], acc);
-            }
-            T[jj] = acc;
-            Wn[jj] = -(acc * be[jj]);
-        }
-#pragma unroll
-        for (int a = 0; a < 4; a++) {
-            const v4f t4 = {T[4 * a], T[4 * a + 1], T[4 * a + 2], T[4 * a + 3]};
-            tm[g].at(16 * a + c) = as_float4(t4);          // read back as register r = T[c][4g' + r] by lane (g', c)
-        }
+        SolveRow x;
+        x.begin(lds.solve, p);
+        x.template columns<15, 0>(lds.solve, p);
+        x.store(tm[g], p);
         __builtin_amdgcn_wave_barrier();
     };
 

@@ -29,12 +29,12 @@ namespace {
 
 // ------------------------------------------------------------------ forward
 
-// What the preparing wave reads of a block.
-// Kt[b], Qt[b]: register r = K[t0 + c][16b + 4g + r];  bcol = beta[t0 + c], brow[r] = beta[t0 + 4g + r]
-template <int NE>
+// What the preparing wave reads of a group of four blocks.
+// Kt[j][b], Qt[j][b]: register r = K[t0 + c][16b + 4g + r] of block j;  bcol[j] = beta[t0 + c]
+template <int NE, bool QK>
 struct PrepRaw {
-    v4f Kt[NE], Qt[NE];
-    float bcol, brow[4];
+    v4f Kt[kGrp][NE], Qt[QK ? kGrp : 1][QK ? NE : 1];
+    float bcol[kGrp];
 };
 
 // What a state wave reads of a block: K and Q whole, its own 16 columns of V.
@@ -54,12 +54,13 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
                                                                   float *__restrict__ aux, int H, int L,
                                                                   int chunk, int nchunk) {
     constexpr int E = 16 * NE, M = 16 * NM;
-    // lower(Q K^T)^T: with one state wave that wave forms it itself (the preparing wave is the
-    // busier one), with several the preparing wave does it once for all
+    // lower(Q K^T)^T: with one state wave that wave forms it itself, with several the preparing
+    // wave does it once for all
     constexpr bool kPrepQK = NM > 1;
-    // slot, matrix (0: (I + A)^-T, 1: strict_lower(K K^T)^T, 2: lower(Q K^T)^T), lane
-    __shared__ LdsMat xch[2][3];
-    __shared__ LdsMat scratch[2];       // the preparing wave's
+    // What the preparing wave hands over, per block of a group of four, two groups alternately:
+    // (I + A)^-T and (with several state waves) lower(Q K^T)^T
+    __shared__ LdsMat tmat[2][kGrp], rmat[kPrepQK ? 2 : 1][kPrepQK ? kGrp : 1];
+    __shared__ SolveLds solve_lds;       // the preparing wave's
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -74,7 +75,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    const int nblk = (L + kBlk - 1) / kBlk;
+    const int nblk = (L + kBlk - 1) / kBlk, ngrp = (nblk + kGrp - 1) / kGrp;
     const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4;
     unsigned o_br[4];
 #pragma unroll
@@ -82,61 +83,83 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 
     if (wave == NM) {
         // ------------------------------------------------ preparing wave
+        // While the state waves do the four blocks of group m (one block per round, a barrier
+        // after each), it prepares group m + 1 in four steps, one per round: K K^T of the four
+        // blocks; the first columns of the substitution (SolveRow); the rest of it and
+        // (I + A)^-T to LDS; lower(Q K^T)^T of the four blocks.
         // aux (with ckpt): a header whose first float says that the per-block matrices
-        // T = (I + A)^-1 follow, row-major, [sequence][block][16][16]; backward then does not
-        // invert again.
+        // T = (I + A)^-1 follow, row-major, [sequence][block][16][16] (written by the first state
+        // wave); backward then does not invert.
         if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
-        float *aux_T = aux ? aux + kAuxHeader + seq * nblk * 256 + c * 16 + 4 * g : nullptr;
         const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
-        v4f ident;
+        using Raw = PrepRaw<NE, kPrepQK>;
+        // a block past the end is read at index nblk: every row beyond the buffers, all zeros
+        auto load = [&](Raw &w, int m) {
 #pragma unroll
-        for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-        auto load = [&](PrepRaw<NE> &w, int ib) {
-            const unsigned ks = ib * k_step, qs = ib * q_step, bs = ib * b_step;
-            w.bcol = bb.f(o_bc, bs);
+            for (int j = 0; j < kGrp; j++) {
+                const int ib = min(kGrp * m + j, nblk);
+                w.bcol[j] = bb.f(o_bc, ib * b_step);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
-#pragma unroll
-            for (int b = 0; b < NE; b++) {
-                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
-                if constexpr (kPrepQK) w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+                for (int b = 0; b < NE; b++) {
+                    w.Kt[j][b] = kb.f4(o_kt + 64 * b, ib * k_step);
+                    if constexpr (kPrepQK) w.Qt[j][b] = qb.f4(o_qt + 64 * b, ib * q_step);
+                }
             }
         };
-        auto prepare = [&](const PrepRaw<NE> &w, int ib) {
-            v4f G = zero, R = zero;
+        SolveRow x;
+        auto step = [&](int ph, const Raw &w, int m) {        // step ph of group m
+            if (ph == 0) {
 #pragma unroll
-            for (int b = 0; b < NE; b++) {
-                G = tn(w.Kt[b], w.Kt[b], G);       // K K^T
-                if constexpr (kPrepQK) R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
-            }
-            v4f A, At, Gu, Rm;
+                for (int j = 0; j < kGrp; j++) {
+                    v4f G = zero;
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
-                At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
-                Gu[r] = p.up[r] ? G[r] : 0.f;
-                Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+                    for (int b = 0; b < NE; b++) G = tn(w.Kt[j][b], w.Kt[j][b], G);       // K K^T
+                    solve_lds.put(j, lane, p, G, w.bcol[j]);
+                }
+            } else if (ph == 1) {
+                x.begin(solve_lds, p);
+                x.template columns<15, 5>(solve_lds, p);
+            } else if (ph == 2) {
+                x.template columns<4, 0>(solve_lds, p);
+                x.store(tmat[m & 1][g], p);
+            } else if constexpr (kPrepQK) {
+#pragma unroll
+                for (int j = 0; j < kGrp; j++) {
+                    v4f R = zero, Rm;
+#pragma unroll
+                    for (int b = 0; b < NE; b++) R = tn(w.Kt[j][b], w.Qt[j][b], R);       // K Q^T  [s][t]
+#pragma unroll
+                    for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+                    rmat[m & 1][j].put(lane, Rm);
+                }
             }
-            const v4f Tt = inv_unit_triangular_lds(A, At, ident, scratch, p, lane);     // (I + A)^-T
-            LdsMat *slot = xch[ib & 1];
-            slot[0].put(lane, Tt);
-            slot[1].put(lane, Gu);
-            if constexpr (kPrepQK) slot[2].put(lane, Rm);
-            if (aux_T)       // register r = T[c][4g + r]
-                *reinterpret_cast<float4 *>(aux_T + (int64_t)ib * 256) = as_float4(Tt);
         };
-        {
-            PrepRaw<NE> first;
-            load(first, 0);
-            prepare(first, 0);
-        }
+        // rounds 4m .. 4m + 3, as far as there are blocks: group m + 1
+        auto rounds = [&](int m, const Raw &w) {
+#pragma unroll
+            for (int ph = 0; ph < kGrp; ph++) {
+                if (kGrp * m + ph >= nblk) return;
+                if (m + 1 < ngrp) step(ph, w, m + 1);
+                lds_barrier();
+            }
+        };
+        Raw even, odd;        // the groups of even and of odd index
+        load(even, 0);
+        load(odd, 1);
+#pragma unroll
+        for (int ph = 0; ph < kGrp; ph++) step(ph, even, 0);
+        load(even, 2);
+        __builtin_amdgcn_sched_barrier(0);
         lds_barrier();
-        // while the state waves do block e: block e + 1 (nothing in the last round)
-        ring_loop<PF, PrepRaw<NE>>(
-            nblk, [&](PrepRaw<NE> &w, int e) { load(w, min(e + 1, nblk - 1)); },
-            [&](int e, const PrepRaw<NE> &w) {
-                if (e + 1 < nblk) prepare(w, e + 1);
-            });
+        for (int m = 0; kGrp * m < nblk; m += 2) {
+            rounds(m, odd);
+            load(odd, m + 3);
+            __builtin_amdgcn_sched_barrier(0);
+            if (kGrp * (m + 1) >= nblk) break;
+            rounds(m + 1, even);
+            load(even, m + 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         return;
     }
 
@@ -175,14 +198,17 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     const unsigned o_out = (unsigned)(c * M + 16 * mb + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + 16 * mb + c) * 4;
     const unsigned m_step = (unsigned)(kBlk * M * 4);
 
+    const RowBuf tb(aux && mb == 0 ? aux + kAuxHeader + seq * nblk * 256 : nullptr,
+                    aux && mb == 0 ? (uint32_t)(nblk * 1024) : 0);
     auto block = [&](int ib, const MainRaw<NE> &cur) {
-        const LdsMat *slot = xch[ib & 1];
+        const int grp = (ib / kGrp) & 1, j = ib % kGrp;
         v4f KS = zero, Ot = zero;
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
-        const v4f Tt = slot[0].get(lane);
+        const v4f Tt = tmat[grp][j].get(lane);
+        tb.st4(Tt, (unsigned)(c * 16 + 4 * g) * 4, (unsigned)ib * 1024);      // register r = T[c][4g + r]
         const v4f X = cur.Vc - KS;
         v4f Y;
 #pragma unroll
@@ -192,7 +218,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         for (int eb = 0; eb < NE; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
         v4f Rm;
         if constexpr (kPrepQK) {
-            Rm = slot[2].get(lane);
+            Rm = rmat[grp][j].get(lane);
         } else {
             v4f R = zero;
 #pragma unroll
@@ -211,7 +237,11 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
                 for (int r = 0; r < 4; r++) Dd[r] = U[r] * __builtin_amdgcn_rcpf(cur.brow[r]);
             } else {
-                const v4f Gu = slot[1].get(lane);
+                v4f G = zero, Gu;
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) G = tn(cur.Kt[eb], cur.Kt[eb], G);
+#pragma unroll
+                for (int r = 0; r < 4; r++) Gu[r] = p.up[r] ? G[r] : 0.f;
                 Dd = X - tn(Gu, U, zero);
             }
 #pragma unroll

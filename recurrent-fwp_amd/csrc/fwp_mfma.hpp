@@ -79,8 +79,13 @@ struct RowBuf {
     __device__ __forceinline__ void st(float x, unsigned lane_bytes, unsigned block_bytes) const {
         llvm_raw_buffer_store_f32(x, rsrc, (int)lane_bytes, (int)block_bytes, 0);
     }
+    // A 16-byte store takes the whole offset in the VGPR.  With the block offset in an SGPR the
+    // compiler sees no hazard between the store and a vector instruction that overwrites the data
+    // registers right behind it, and the hardware has one: the store then writes the new value for
+    // some lanes (seen as zeros in the first dword of the last four lanes of each row, and only
+    // with several waves per SIMD).  Without the SGPR the compiler leaves the wait state.
     __device__ __forceinline__ void st4(const v4f &x, unsigned lane_bytes, unsigned block_bytes) const {
-        llvm_raw_buffer_store_v4f32(x, rsrc, (int)lane_bytes, (int)block_bytes, 0);
+        llvm_raw_buffer_store_v4f32(x, rsrc, (int)(lane_bytes + block_bytes), 0, 0);
     }
 };
 
@@ -134,6 +139,62 @@ __device__ __forceinline__ v4f inv_unit_triangular_lds(v4f A, v4f At, v4f identi
     const v4f A8 = tn(At4, A4, zero);
     return tn(A8, T, T);
 }
+
+// T = (I + A)^-1 for A = strict_lower(diag(b) G), G = K K^T, without multiplying it out on the matrix
+// cores (six products per block): T (I + A) = I is solved by substitution, column by column from the
+// right, T[c][j] = [c == j] - sum_{i > j} T[c][i] b_i G[i][j], 120 multiply-adds per row.  A wave
+// does a group of four blocks at once: lane 16 jb + c computes row c of block jb, reading G and b
+// from LDS (the 16 lanes of a block read the same address).
+constexpr int kGrp = 4;     // blocks per group
+
+// G per block of the group in the accumulator layout, 64 lanes + 4 of padding so that the four
+// blocks' reads fall on different banks; b likewise
+struct SolveLds {
+    float4 gm[kGrp][68];
+    float bl[kGrp][20];
+    // by the whole wave, for block j of the group: G in the accumulator layout, bcol = b[t0 + c]
+    __device__ __forceinline__ void put(int j, int lane, const Geo16 &p, const v4f &G, float bcol) {
+        gm[j][lane] = as_float4(G);
+        if (p.g == 0) bl[j][p.c] = bcol;
+    }
+};
+
+// A lane's row of T and what it carries between the steps of the substitution.
+struct SolveRow {
+    float be[16], T[16], Wn[16];
+    __device__ __forceinline__ void begin(const SolveLds &s, const Geo16 &p) {
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            const float4 b4 = *reinterpret_cast<const float4 *>(&s.bl[p.g][4 * a]);
+            be[4 * a] = b4.x, be[4 * a + 1] = b4.y, be[4 * a + 2] = b4.z, be[4 * a + 3] = b4.w;
+        }
+    }
+    // columns HI down to LO of the row (the columns above HI done before)
+    template <int HI, int LO>
+    __device__ __forceinline__ void columns(const SolveLds &s, const Geo16 &p) {
+        const float4 *gq = s.gm[p.g];
+#pragma unroll
+        for (int jj = HI; jj >= LO; jj--) {
+            float acc = p.c == jj ? 1.f : 0.f;
+#pragma unroll
+            for (int a = (jj + 1) / 4; a < 4; a++) {
+                const float4 g4 = gq[16 * a + jj];          // G[4a .. 4a + 3][jj]
+                const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+                for (int x = 0; x < 4; x++)
+                    if (4 * a + x > jj) acc = fmaf(Wn[4 * a + x], gg[x], acc);
+            }
+            T[jj] = acc;
+            Wn[jj] = -(acc * be[jj]);
+        }
+    }
+    // (I + A)^-T of the lane's block as the accumulator layout wants it: lane (g', c) then reads
+    // register r = T[c][4g' + r]
+    __device__ __forceinline__ void store(LdsMat &m, const Geo16 &p) const {
+#pragma unroll
+        for (int a = 0; a < 4; a++) m.at(16 * a + p.c) = make_float4(T[4 * a], T[4 * a + 1], T[4 * a + 2], T[4 * a + 3]);
+    }
+};
 
 // Index of the checkpoint chunk a block lies in: block / blocks_per_chunk as a multiplication
 // (exact while block * blocks_per_chunk < 2^32), the remainder alongside.

@@ -59,6 +59,35 @@ def test_delta_full_size_properties(fwp):
     assert torch.allclose(g3[2], 2 * g1[2], atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(96, 8, 256, 16), (32, 8, 1024, 32), (160, 8, 250, 16)])
+@pytest.mark.parametrize("op", ["delta", "sum"])
+def test_blocked_kernels_against_scan_kernels_at_full_occupancy(fwp, op, shape):
+    """The blocked kernels (matrix cores, buffer-resource loads and stores) against the step-by-step
+    kernels (another code path altogether) at sizes that put several waves on every SIMD: what only
+    goes wrong when waves share a SIMD or the memory pipeline is busy shows here, not at the sizes
+    the oracle is run at.  Tolerance as for the oracle parity: |a - b| <= 1e-4 + 1e-3 |b|."""
+    B, H, T, D = shape
+    q, k, v, beta, W0, go = (dev(a) for a in delta_inputs(1, B, H, T, D, D, dtype=np.float32))
+    L_ = fwp._lib
+    res = {}
+    try:
+        for kind in ("scan", "chunked", "split", "auto"):
+            L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED,
+                                             "split": L_.DELTA_SPLIT, "auto": L_.DELTA_AUTO}[kind])
+            W = W0.clone()
+            if op == "delta":
+                out, g = grads_of(lambda t: fwp.fast_weight_delta(*t, W), [q, k, v, beta], go)
+            else:
+                out, g = grads_of(lambda t: fwp.fast_weight_sum(*t, W), [q, k, v], go)
+            res[kind] = (out, W, *g)
+    finally:
+        L_.config(L_.CFG_DELTA_KERNELS, L_.DELTA_AUTO)
+    for kind in ("chunked", "split", "auto"):
+        for i, (x, y) in enumerate(zip(res[kind], res["scan"])):
+            assert torch.isfinite(x).all()
+            assert torch.allclose(x, y, atol=1e-4, rtol=1e-3), (kind, i, float((x - y).abs().max()))
+
+
 def test_rnn_full_size_properties(fwp):
     z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(1, 64, 8, 256, 32, dtype=np.float32))
 
