@@ -29,12 +29,16 @@ namespace {
 
 // ------------------------------------------------------------------ forward
 
-// What the preparing wave reads of a group of four blocks.
-// Kt[j][b], Qt[j][b]: register r = K[t0 + c][16b + 4g + r] of block j;  bcol[j] = beta[t0 + c]
-template <int NE, bool QK>
+// What the preparing wave reads: of two blocks for K K^T, of one block for lower(Q K^T).
+// Kt[j][b], Qt[b]: register r = K[t0 + c][16b + 4g + r];  bcol[j] = beta[t0 + c]
+template <int NE>
 struct PrepRaw {
-    v4f Kt[kGrp][NE], Qt[QK ? kGrp : 1][QK ? NE : 1];
-    float bcol[kGrp];
+    v4f Kt[2][NE];
+    float bcol[2];
+};
+template <int NE>
+struct PrepQk {
+    v4f Kt[NE], Qt[NE];
 };
 
 // What a state wave reads of a block: K and Q whole, its own 16 columns of V.
@@ -84,81 +88,93 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     if (wave == NM) {
         // ------------------------------------------------ preparing wave
         // While the state waves do the four blocks of group m (one block per round, a barrier
-        // after each), it prepares group m + 1 in four steps, one per round: K K^T of the four
-        // blocks; the first columns of the substitution (SolveRow); the rest of it and
-        // (I + A)^-T to LDS; lower(Q K^T)^T of the four blocks.
+        // after each), it prepares group m + 1 in four steps, one per round: K K^T of two blocks,
+        // of the other two, the first columns of the substitution (SolveRow), the rest of it and
+        // (I + A)^-T to LDS; with several state waves also lower(Q K^T)^T of one block per step.
         // aux (with ckpt): a header whose first float says that the per-block matrices
         // T = (I + A)^-1 follow, row-major, [sequence][block][16][16] (written by the first state
         // wave); backward then does not invert.
         if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
         const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
-        using Raw = PrepRaw<NE, kPrepQK>;
+        using Raw = PrepRaw<NE>;
         // a block past the end is read at index nblk: every row beyond the buffers, all zeros
-        auto load = [&](Raw &w, int m) {
+        auto load = [&](Raw &w, int ib0) {            // blocks ib0, ib0 + 1
 #pragma unroll
-            for (int j = 0; j < kGrp; j++) {
-                const int ib = min(kGrp * m + j, nblk);
+            for (int j = 0; j < 2; j++) {
+                const int ib = min(ib0 + j, nblk);
                 w.bcol[j] = bb.f(o_bc, ib * b_step);
 #pragma unroll
+                for (int b = 0; b < NE; b++) w.Kt[j][b] = kb.f4(o_kt + 64 * b, ib * k_step);
+            }
+        };
+        auto load_qk = [&](PrepQk<NE> &w, int ib) {
+            if constexpr (kPrepQK) {
+                ib = min(ib, nblk);
+#pragma unroll
                 for (int b = 0; b < NE; b++) {
-                    w.Kt[j][b] = kb.f4(o_kt + 64 * b, ib * k_step);
-                    if constexpr (kPrepQK) w.Qt[j][b] = qb.f4(o_qt + 64 * b, ib * q_step);
+                    w.Kt[b] = kb.f4(o_kt + 64 * b, ib * k_step);
+                    w.Qt[b] = qb.f4(o_qt + 64 * b, ib * q_step);
                 }
             }
         };
         SolveRow x;
-        auto step = [&](int ph, const Raw &w, int m) {        // step ph of group m
+        auto gram = [&](const Raw &w, int j0) {        // K K^T of blocks j0, j0 + 1 of the group
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                v4f G = zero;
+#pragma unroll
+                for (int b = 0; b < NE; b++) G = tn(w.Kt[j][b], w.Kt[j][b], G);
+                solve_lds.put(j0 + j, lane, p, G, w.bcol[j]);
+            }
+        };
+        auto qk = [&](const PrepQk<NE> &w, int m, int j) {   // lower(Q K^T)^T of block j of group m
+            if constexpr (kPrepQK) {
+                v4f R = zero, Rm;
+#pragma unroll
+                for (int b = 0; b < NE; b++) R = tn(w.Kt[b], w.Qt[b], R);       // K Q^T  [s][t]
+#pragma unroll
+                for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+                rmat[m & 1][j].put(lane, Rm);
+            }
+        };
+        // The rows of K for K K^T are read four rounds before they are used (two blocks each in
+        // `lo` and `hi`), those for lower(Q K^T) one round before (`one`, alternately).
+        Raw lo, hi;
+        PrepQk<NE> one[2];
+        // step ph of group m: K K^T of two blocks each in the first two steps, the substitution in
+        // the last two, one lower(Q K^T) in each; then the reads for what comes
+        auto step = [&](int ph, int m) {
             if (ph == 0) {
-#pragma unroll
-                for (int j = 0; j < kGrp; j++) {
-                    v4f G = zero;
-#pragma unroll
-                    for (int b = 0; b < NE; b++) G = tn(w.Kt[j][b], w.Kt[j][b], G);       // K K^T
-                    solve_lds.put(j, lane, p, G, w.bcol[j]);
-                }
+                gram(lo, 0);
+                load(lo, kGrp * (m + 1));
             } else if (ph == 1) {
+                gram(hi, 2);
+                load(hi, kGrp * (m + 1) + 2);
+            } else if (ph == 2) {
                 x.begin(solve_lds, p);
                 x.template columns<15, 5>(solve_lds, p);
-            } else if (ph == 2) {
+            } else {
                 x.template columns<4, 0>(solve_lds, p);
                 x.store(tmat[m & 1][g], p);
-            } else if constexpr (kPrepQK) {
-#pragma unroll
-                for (int j = 0; j < kGrp; j++) {
-                    v4f R = zero, Rm;
-#pragma unroll
-                    for (int b = 0; b < NE; b++) R = tn(w.Kt[j][b], w.Qt[j][b], R);       // K Q^T  [s][t]
-#pragma unroll
-                    for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
-                    rmat[m & 1][j].put(lane, Rm);
-                }
             }
+            qk(one[ph % 2], m, ph);
+            load_qk(one[(ph + 1) % 2], kGrp * m + ph + 1);
+            __builtin_amdgcn_sched_barrier(0);
         };
+        load(lo, 0);
+        load(hi, 2);
+        load_qk(one[0], 0);
+#pragma unroll
+        for (int ph = 0; ph < kGrp; ph++) step(ph, 0);
+        lds_barrier();
         // rounds 4m .. 4m + 3, as far as there are blocks: group m + 1
-        auto rounds = [&](int m, const Raw &w) {
+        for (int m = 0; kGrp * m < nblk; m++) {
 #pragma unroll
             for (int ph = 0; ph < kGrp; ph++) {
-                if (kGrp * m + ph >= nblk) return;
-                if (m + 1 < ngrp) step(ph, w, m + 1);
+                if (kGrp * m + ph >= nblk) break;
+                if (m + 1 < ngrp) step(ph, m + 1);
                 lds_barrier();
             }
-        };
-        Raw even, odd;        // the groups of even and of odd index
-        load(even, 0);
-        load(odd, 1);
-#pragma unroll
-        for (int ph = 0; ph < kGrp; ph++) step(ph, even, 0);
-        load(even, 2);
-        __builtin_amdgcn_sched_barrier(0);
-        lds_barrier();
-        for (int m = 0; kGrp * m < nblk; m += 2) {
-            rounds(m, odd);
-            load(odd, m + 3);
-            __builtin_amdgcn_sched_barrier(0);
-            if (kGrp * (m + 1) >= nblk) break;
-            rounds(m + 1, even);
-            load(even, m + 4);
-            __builtin_amdgcn_sched_barrier(0);
         }
         return;
     }
