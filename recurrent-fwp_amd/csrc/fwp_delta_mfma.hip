@@ -171,8 +171,7 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
         const v4f Tt = tm[j].get(lane);
         tb.st4(Tt, (unsigned)(c * 16 + 4 * g) * 4, (unsigned)ib * 1024);      // whole rows of T per instruction
         const v4f brow = from_float4(*reinterpret_cast<const float4 *>(&bl[j][4 * g]));   // beta[t0 + 4g + r]
-        const bool beta_nonzero =
-            __builtin_amdgcn_ballot_w64(brow[0] == 0.f || brow[1] == 0.f || brow[2] == 0.f || brow[3] == 0.f) == 0;
+        const bool beta_nonzero = betas_divide(brow);
 #pragma unroll
         for (int mb = 0; mb < NM; mb++) {
             v4f KS = zero, Ot = zero;
@@ -191,7 +190,7 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
             ob.st4(O, o_out + 64 * mb, ib * m_step);
             if (vdiff) {
                 // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division
-                // where no beta of the block is zero (rows past the end read beta = 0)
+                // where the block's betas allow it
                 v4f Dd;
                 if (beta_nonzero) {
 #pragma unroll

@@ -245,11 +245,10 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
         ob.st4(O, o_out, ib * m_step);
         if (vdiff) {
-            // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division where no
-            // beta of the block is zero (rows past the end of the sequence read beta = 0)
+            // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division where
+            // the block's betas allow it
             v4f Dd;
-            if (__builtin_amdgcn_ballot_w64(cur.brow[0] == 0.f || cur.brow[1] == 0.f || cur.brow[2] == 0.f ||
-                                            cur.brow[3] == 0.f) == 0) {
+            if (betas_divide(v4f{cur.brow[0], cur.brow[1], cur.brow[2], cur.brow[3]})) {
 #pragma unroll
                 for (int r = 0; r < 4; r++) Dd[r] = U[r] * __builtin_amdgcn_rcpf(cur.brow[r]);
             } else {

@@ -196,6 +196,15 @@ struct SolveRow {
     }
 };
 
+// v - v_old can be had from U = diag(beta)(v - v_old) by a division only where every beta of the
+// block is large enough for its reciprocal to be finite and exact enough (rows past the end of the
+// sequence read beta = 0; zeros and denormals may also come from the caller).
+__device__ __forceinline__ bool betas_divide(const v4f &brow) {
+    constexpr float kMin = 1e-30f;
+    return __builtin_amdgcn_ballot_w64(!(fabsf(brow[0]) >= kMin) || !(fabsf(brow[1]) >= kMin) ||
+                                       !(fabsf(brow[2]) >= kMin) || !(fabsf(brow[3]) >= kMin)) == 0;
+}
+
 // Index of the checkpoint chunk a block lies in: block / blocks_per_chunk as a multiplication
 // (exact while block * blocks_per_chunk < 2^32), the remainder alongside.
 struct ChunkOf {

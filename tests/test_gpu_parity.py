@@ -118,6 +118,31 @@ def test_delta_block_edges(fwp, delta_kernels, L, D):
         check("grad_" + name, t.grad, r)
 
 
+@pytest.mark.parametrize("D", [16, 32])
+def test_delta_write_strengths_zero_tiny_negative_and_above_one(fwp, delta_kernels, D):
+    # write strengths as the operator admits them (any real number, not only sigmoid outputs): exact
+    # zeros (the step writes nothing, v - v_old still is saved for backward), denormals, tiny values,
+    # negative values and values above one, spread so that some blocks of 16 steps have none of them
+    q, k, v, beta, W0, go = delta_inputs(900 + D, 2, 3, 100, D, D, w0=True)
+    beta = beta.copy()
+    beta[:, :, 5] = 0.0
+    beta[:, :, 17:20] = 0.0
+    beta[0, :, 40] = 1e-42          # denormal
+    beta[1, :, 41] = 1e-33
+    beta[:, :, 50] = -0.7
+    beta[:, :, 66] = 1.9
+    beta[:, :, 99] = 0.0            # in the last, partial block
+    tq, tk, tv, tb = (dev(x, True) for x in (q, k, v, beta))
+    W = dev(W0)
+    out = fwp.fast_weight_delta(tq, tk, tv, tb, W)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("q k v beta".split(), (tq, tk, tv, tb), oracle.delta_bwd(q, k, v, beta, W0, go)):
+        check("grad_" + name, t.grad, r)
+
+
 def test_delta_strided_views_and_segments(fwp, delta_kernels):
     # inputs as the layers pass them: [L,N,H,*] storage permuted to [N,H,L,*], and a carried state
     N, H, L, D = 2, 3, 48, 16
