@@ -43,14 +43,22 @@ struct PrepQk {
 
 // What a state wave reads of a block: K and Q whole, its own 16 columns of V.
 // Kc[b], Vc: register r = K[t0 + 4g + r][16b + c]
-template <int NE>
+template <int NE, bool WITH_Q>
 struct MainRaw {
-    v4f Kt[NE], Qt[NE], Kc[NE], Vc;
+    v4f Kt[NE], Qt[WITH_Q ? NE : 1], Kc[NE], Vc;
     float brow[4];
 };
 
-template <int NE, int NM, int PF>   // E = 16 NE, M = 16 NM, PF = blocks in flight
-__global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
+// What the output wave reads of a block: Q whole, K too where it forms lower(Q K^T) itself.
+template <int NE, bool WITH_K>
+struct OutRaw {
+    v4f Qt[NE], Kt[WITH_K ? NE : 1];
+};
+
+// OUT: one more wave takes the products that only feed the output (S^T Q^T, lower(Q K^T), O), one
+// block behind the state waves, which hand it their columns of the state and of U.
+template <int NE, int NM, int PF, bool OUT>   // E = 16 NE, M = 16 NM, PF = blocks in flight
+__global__ __launch_bounds__(64 * (NM + 1 + OUT)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
                                                                   fwp_view beta, float *__restrict__ W,
                                                                   float *__restrict__ out,
                                                                   float *__restrict__ vdiff,
@@ -65,6 +73,9 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     // (I + A)^-T and (with several state waves) lower(Q K^T)^T
     __shared__ LdsMat tmat[2][kGrp], rmat[kPrepQK ? 2 : 1][kPrepQK ? kGrp : 1];
     __shared__ SolveLds solve_lds;       // the preparing wave's
+    // state wave mb to the output wave, blocks of even and odd index alternately: its columns of
+    // the state before the block (NE tiles) and of U
+    __shared__ LdsMat hx[OUT ? 2 : 1][OUT ? NM : 1][OUT ? NE + 1 : 1];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -176,6 +187,48 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
                 lds_barrier();
             }
         }
+        if constexpr (OUT) lds_barrier();      // the output wave's last block
+        return;
+    }
+
+    const unsigned m_step = (unsigned)(kBlk * M * 4);
+    if (OUT && wave == NM + 1) {
+        // ------------------------------------------------ output wave, one block behind
+        using Raw = OutRaw<NE, !kPrepQK>;
+        const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4));
+        const unsigned o_out = (unsigned)(c * M + 4 * g) * 4;
+        auto load = [&](Raw &w, int ib) {
+            const unsigned ks = ib * k_step, qs = ib * q_step;
+#pragma unroll
+            for (int b = 0; b < NE; b++) {
+                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+                if constexpr (!kPrepQK) w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            }
+        };
+        auto block = [&](int ib, const Raw &w) {
+            v4f Rm;
+            if constexpr (kPrepQK) {
+                Rm = rmat[(ib / kGrp) & 1][ib % kGrp].get(lane);
+            } else {
+                v4f R = zero;
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) R = tn(w.Kt[eb], w.Qt[eb], R);
+#pragma unroll
+                for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+            }
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) {
+                const LdsMat *from = hx[OUT ? ib & 1 : 0][OUT ? mb : 0];
+                v4f Ot = zero;
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) Ot = tn(from[eb].get(lane), w.Qt[eb], Ot);   // O^T, state part
+                const v4f O = tn(from[OUT ? NE : 0].get(lane), Rm, Ot);   // register r = O[t0 + c][16 mb + 4g + r]
+                ob.st4(O, o_out + 64 * mb, ib * m_step);
+            }
+        };
+        lds_barrier();      // the preparing wave's block 0
+        lds_barrier();      // the state waves' block 0
+        ring_loop<PF, Raw>(nblk, load, block);
         return;
     }
 
@@ -187,7 +240,8 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
         o_vr[r] = (unsigned)((4 * g + r) * v.sL + 16 * mb + c) * 4;
     }
-    auto load = [&](MainRaw<NE> &w, int ib) {
+    using StateRaw = MainRaw<NE, !OUT>;
+    auto load = [&](StateRaw &w, int ib) {
         const unsigned ks = ib * k_step, qs = ib * q_step, vs = ib * v_step, bs = ib * b_step;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -197,7 +251,7 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
 #pragma unroll
         for (int b = 0; b < NE; b++) {
             w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
-            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+            if constexpr (!OUT) w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
             for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
         }
@@ -212,17 +266,20 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     const ChunkOf chunk_of(chunk);
     const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4)), db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0);
     const unsigned o_out = (unsigned)(c * M + 16 * mb + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + 16 * mb + c) * 4;
-    const unsigned m_step = (unsigned)(kBlk * M * 4);
-
     const RowBuf tb(aux && mb == 0 ? aux + kAuxHeader + seq * nblk * 256 : nullptr,
                     aux && mb == 0 ? (uint32_t)(nblk * 1024) : 0);
-    auto block = [&](int ib, const MainRaw<NE> &cur) {
+    auto block = [&](int ib, const StateRaw &cur) {
         const int grp = (ib / kGrp) & 1, j = ib % kGrp;
         v4f KS = zero, Ot = zero;
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) KS = tn(cur.Kt[eb], S[eb], KS);
+        if constexpr (OUT) {
 #pragma unroll
-        for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
+            for (int eb = 0; eb < NE; eb++) hx[ib & 1][mb][eb].put(lane, S[eb]);
+        } else {
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) Ot = tn(S[eb], cur.Qt[eb], Ot);      // O^T, state part (old state)
+        }
         const v4f Tt = tmat[grp][j].get(lane);
         tb.st4(Tt, (unsigned)(c * 16 + 4 * g) * 4, (unsigned)ib * 1024);      // register r = T[c][4g + r]
         const v4f X = cur.Vc - KS;
@@ -232,18 +289,22 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
         const v4f U = tn(Tt, Y, zero);
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) S[eb] = tn(cur.Kc[eb], U, S[eb]);
-        v4f Rm;
-        if constexpr (kPrepQK) {
-            Rm = rmat[grp][j].get(lane);
+        if constexpr (OUT) {
+            hx[ib & 1][mb][NE].put(lane, U);
         } else {
-            v4f R = zero;
+            v4f Rm;
+            if constexpr (kPrepQK) {
+                Rm = rmat[grp][j].get(lane);
+            } else {
+                v4f R = zero;
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) R = tn(cur.Kt[eb], cur.Qt[eb], R);
+                for (int eb = 0; eb < NE; eb++) R = tn(cur.Kt[eb], cur.Qt[eb], R);
 #pragma unroll
-            for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+                for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+            }
+            const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
+            ob.st4(O, o_out, ib * m_step);
         }
-        const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
-        ob.st4(O, o_out, ib * m_step);
         if (vdiff) {
             // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division where
             // the block's betas allow it
@@ -272,7 +333,8 @@ __global__ __launch_bounds__(64 * (NM + 1)) void k_delta_fwd_split(fwp_view q, f
     };
 
     lds_barrier();      // the preparing wave's block 0
-    ring_loop<PF, MainRaw<NE>>(nblk, load, block);
+    ring_loop<PF, StateRaw>(nblk, load, block);
+    if constexpr (OUT) lds_barrier();      // the output wave's last block
 #pragma unroll
     for (int eb = 0; eb < NE; eb++)
 #pragma unroll
@@ -600,11 +662,21 @@ namespace {
 constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }
 constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
 
+// The output wave is built for the two square shapes and used up to one and a half waves per SIMD
+// (D = 16, forward at 256 / 512 / 768 sequences of 256 steps: 12.5 / 15.2 / 18.4 us with it,
+// 14.8 / 17.4 / 18.1 us without; D = 32, 256 sequences of 1024 steps: 54 against 62 us).
 template <int NE, int NM>
 void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
                 float *ckpt, float *aux, int nseq, int H, int L, int chunk, int nchunk, hipStream_t s) {
-    hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE)>), dim3(nseq), dim3(64 * (NM + 1)), 0, s, q, k, v,
-                       beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+    if constexpr (NE == NM && NE <= 2) {
+        if ((int64_t)nseq * (NM + 2) <= 1536) {
+            hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), true>), dim3(nseq), dim3(64 * (NM + 2)), 0,
+                               s, q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+            return;
+        }
+    }
+    hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), false>), dim3(nseq), dim3(64 * (NM + 1)), 0, s, q,
+                       k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
 }
 template <int NE, int NM>
 void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go, const float *ckpt,
