@@ -32,14 +32,12 @@ bool delta_chunked(int L) {
 }
 
 // Several waves per sequence or one, measured on MI355X (1024 SIMDs) as the time of a training step
-// (what runs before a kernel changes where its waves land, so kernels timed alone mislead).
-// Backward: the split kernel wins or ties at every sequence count for D = 16 (768 sequences: 28 us
-// against 40 us; 2048: 76 against 77) and up to about a thousand sequences for D = 32 (beyond, it is
-// 5-10 % slower).  Forward: the split kernel up to about a thousand sequences (D = 16, step of forward
-// + backward at 512 / 768 / 1024 sequences of 256 steps: 41.4 / 43.5 / 49.6 us against 44.3 / 46.7 /
-// 50.8 us with the one-wave forward; D = 32, 256 sequences of 1024 steps: 64 us against 117 us), one
-// wave beyond (D = 16, 2048 sequences: 113 us against 123 us; D = 32, 2048 of 256 steps: 108 against
-// 129).
+// (what runs before a kernel changes where its waves land, so kernels timed alone mislead): the split
+// kernels up to 1024 sequences, one wave per sequence beyond.  D = 16, step of forward + backward at
+// 512 / 768 / 1024 sequences of 256 steps: 41 / 44 / 49 us split, 44 / 47 / 50 us one wave; at
+// 1280 / 1536 / 2048 sequences: 74 / 80 / 124 us split, 71 / 74 / 97 us one wave.  D = 32, 256 sequences
+// of 1024 steps: 55 + 106 us split, 117 + 233 us one wave; 1280 sequences of 256 steps: 218 us split,
+// 203 us one wave.
 // The kernels that read through buffer resources address a sequence with 32-bit byte offsets, and
 // may ask for rows up to two blocks past its end (which must not wrap around to rows that exist).
 bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
@@ -59,7 +57,6 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
     if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
     if (L < 32) return false;
-    if (E == 16 && !forward) return true;
     return (int64_t)N * H <= 1024;
 }
 

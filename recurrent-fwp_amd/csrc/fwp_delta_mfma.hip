@@ -261,17 +261,19 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
 //     dS <- dS + Q^T dO - K^T dX
 // The state is kept transposed (all its uses contract over the value index) and is rewound block
 // by block from the checkpoints, S0^T = S'^T - U^T K.  Gradients are produced transposed so that
-// they leave with 16-byte stores.
+// they leave with 16-byte stores; a matrix that is needed transposed goes through LDS.
+// One wave per sequence, several sequences per workgroup like the forward.
 
-template <int NB>
-struct RawBwd {
-    v4f Kt[NB], Qt[NB], Kc[NB], Qc[NB], Oc[NB], Ot[NB], Dc[NB], Dt[NB];   // O: upstream gradient, D: vdiff
-    v4f T;                   // (I + A)^-1 when forward saved it
-    v4f Sck[NB][NB];         // checkpointed state of the block's chunk, transposed (used by the chunk's last block)
+template <int NE, int NM>
+struct BwdRaw {
+    v4f Kt[NE], Qt[NE], Kc[NE], Qc[NE];
+    v4f Oc[NM], Ot[NM], Dc[NM], Dt[NM];   // O: upstream gradient, D: vdiff
+    v4f T;                                // (I + A)^-1 when forward saved it
+    v4f Sck[NM][NE];                      // checkpointed state of the block's chunk, transposed
     float bcol, brow[4];
 };
 
-template <int NB>
+template <int NE, int NM>   // state E = 16 NE by M = 16 NM
 __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_bwd_mfma(fwp_view q, fwp_view k, fwp_view beta,
                                                        const float *__restrict__ vdiff, fwp_view go,
                                                        const float *__restrict__ ckpt,
@@ -280,166 +282,108 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_bwd_mfma(fwp_view q, f
                                                        float *__restrict__ gv,
                                                        float *__restrict__ gbeta, int nseq, int H, int L,
                                                        int chunk, int nchunk) {
-    constexpr int D = 16 * NB;
-    const Geo16 p(threadIdx.x % 64);
+    constexpr int E = 16 * NE, M = 16 * NM, PF = NE + NM <= 2 ? 2 : 1;
+    extern __shared__ __align__(16) unsigned char dyn_lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    LdsMat *scratch = reinterpret_cast<LdsMat *>(dyn_lds) + 4 * wave;        // four matrices per wave
+    const int lane = threadIdx.x % 64;
+    const Geo16 p(lane);
     const int g = p.g, c = p.c;
-    const int64_t seq = (int64_t)blockIdx.x * (blockDim.x / 64) + __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int64_t seq = (int64_t)blockIdx.x * (blockDim.x / 64) + wave;
     if (seq >= nseq) return;
     const int n = (int)(seq / H), h = (int)(seq % H);
-    const float *qb = row(q, n, h, 0), *kb = row(k, n, h, 0), *gob = row(go, n, h, 0),
-                *bb = row(beta, n, h, 0), *db = vdiff + seq * L * D;
+    const int nblk = (L + kBlk - 1) / kBlk;
+    // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
+    const bool have_T = aux && aux[0] == 1.f;
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + M) * 4)),
+        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
+        db(vdiff + seq * L * M, (uint32_t)(L * M * 4)),
+        tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0),
+        cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
+        gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
+        gvb(gv + seq * L * M, (uint32_t)(L * M * 4)), gbb(gbeta + seq * L, (uint32_t)(L * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   o_step = (unsigned)(kBlk * go.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
+                   d_step = (unsigned)(kBlk * M * 4), e_step = (unsigned)(kBlk * E * 4);
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     v4f ident;
 #pragma unroll
     for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-    // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
-    const bool have_T = aux && aux[0] == 1.f;
-    const float *aux_T = have_T ? aux + kAuxHeader + seq * ((L + kBlk - 1) / kBlk) * 256 + 4 * g * 16 + c : nullptr;
-
-    // per-lane element offsets inside a block (32-bit: a block spans 16 rows)
-    unsigned o_kt = (unsigned)(c * k.sL + 4 * g), o_qt = (unsigned)(c * q.sL + 4 * g),
-             o_ot = (unsigned)(c * go.sL + 4 * g), o_dt = (unsigned)(c * D + 4 * g),
-             o_bc = (unsigned)(c * beta.sL);
-    unsigned o_kr[4], o_qr[4], o_or[4], o_dr[4], o_br[4];
+    const unsigned o_bc = (unsigned)(c * beta.sL) * 4, o_t = (unsigned)(4 * g * 16 + c) * 4;
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                   o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4,
+                   o_ge = (unsigned)(c * E + 4 * g) * 4, o_ck = (unsigned)(c * M + 4 * g) * 4;
+    unsigned o_br[4], o_kr[4], o_qr[4], o_or[4], o_dr[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c);
-        o_qr[r] = (unsigned)((4 * g + r) * q.sL + c);
-        o_or[r] = (unsigned)((4 * g + r) * go.sL + c);
-        o_dr[r] = (unsigned)((4 * g + r) * D + c);
-        o_br[r] = (unsigned)((4 * g + r) * beta.sL);
+        o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
+        o_or[r] = (unsigned)((4 * g + r) * go.sL + c) * 4;
+        o_dr[r] = (unsigned)((4 * g + r) * M + c) * 4;
     }
-    auto as_v4f = [](const float *ptr) {
-        const float4 x = *reinterpret_cast<const float4 *>(ptr);
-        return v4f{x.x, x.y, x.z, x.w};
-    };
-    auto load = [&](RawBwd<NB> &w, int t0) {
-        {   // always loaded, so that no load is left to be issued (and waited for) inside the block
-            const float *src = ckpt + (seq * nchunk + (min(t0 + kBlk, L) - 1) / chunk) * D * D;
-#pragma unroll
-            for (int mb = 0; mb < NB; mb++)
-#pragma unroll
-                for (int eb = 0; eb < NB; eb++)
-                    w.Sck[mb][eb] = as_v4f(src + (16 * eb + c) * D + 16 * mb + 4 * g);
-        }
+    const ChunkOf chunk_of(chunk);
+    auto load = [&](BwdRaw<NE, NM> &w, int e) {
+        const int ib = nblk - 1 - e;
         if (have_T) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.T[r] = aux_T[(int64_t)(t0 / kBlk) * 256 + 16 * r];
+            for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
         }
-        if (t0 + kBlk <= L) {    // whole block inside the sequence: uniform block base + lane offsets
-            const float *kblk = kb + (int64_t)t0 * k.sL, *qblk = qb + (int64_t)t0 * q.sL,
-                        *oblk = gob + (int64_t)t0 * go.sL, *dblk = db + (int64_t)t0 * D,
-                        *bblk = bb + (int64_t)t0 * beta.sL;
-            w.bcol = bblk[o_bc];
+        {   // always loaded, so that no load is left to be issued (and waited for) inside the block
+            const unsigned cs = chunk_of(ib) * (E * M * 4);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.brow[r] = bblk[o_br[r]];
+            for (int mb = 0; mb < NM; mb++)
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
-                w.Kt[b] = as_v4f(kblk + (o_kt + 16 * b));
-                w.Qt[b] = as_v4f(qblk + (o_qt + 16 * b));
-                w.Ot[b] = as_v4f(oblk + (o_ot + 16 * b));
-                w.Dt[b] = as_v4f(dblk + (o_dt + 16 * b));
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    w.Kc[b][r] = kblk[o_kr[r] + 16 * b];
-                    w.Qc[b][r] = qblk[o_qr[r] + 16 * b];
-                    w.Oc[b][r] = oblk[o_or[r] + 16 * b];
-                    w.Dc[b][r] = dblk[o_dr[r] + 16 * b];
-                }
-            }
-            return;
+                for (int eb = 0; eb < NE; eb++) w.Sck[mb][eb] = cb.f4(o_ck + (16 * eb * M + 16 * mb) * 4, cs);
         }
-        // ragged last block; rows beyond L: clamped loads, beta = 0 and a zero upstream gradient
-        const bool col_ok = t0 + c < L;
-        const int64_t tc = min(t0 + c, L - 1);
-        w.bcol = col_ok ? bb[tc * beta.sL] : 0.f;
-        int64_t tr[4];
-        bool row_ok[4];
+        const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
+                       bs = ib * b_step;
+        w.bcol = bb.f(o_bc, bs);
 #pragma unroll
-        for (int r = 0; r < 4; r++) {
-            row_ok[r] = t0 + 4 * g + r < L;
-            tr[r] = min(t0 + 4 * g + r, L - 1);
-            w.brow[r] = row_ok[r] ? bb[tr[r] * beta.sL] : 0.f;
-        }
+        for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
 #pragma unroll
-        for (int b = 0; b < NB; b++) {
-            const int ct = 16 * b + 4 * g, cc = 16 * b + c;
-            const float4 kk = *reinterpret_cast<const float4 *>(kb + tc * k.sL + ct);
-            const float4 qq = *reinterpret_cast<const float4 *>(qb + tc * q.sL + ct);
-            const float4 oo = *reinterpret_cast<const float4 *>(gob + tc * go.sL + ct);
-            const float4 dd = *reinterpret_cast<const float4 *>(db + tc * D + ct);
-            w.Kt[b] = v4f{kk.x, kk.y, kk.z, kk.w};
-            w.Qt[b] = v4f{qq.x, qq.y, qq.z, qq.w};
-            w.Ot[b] = col_ok ? v4f{oo.x, oo.y, oo.z, oo.w} : zero;
-            w.Dt[b] = v4f{dd.x, dd.y, dd.z, dd.w};
+        for (int b = 0; b < NE; b++) {
+            w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+            w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
-                w.Kc[b][r] = kb[tr[r] * k.sL + cc];
-                w.Qc[b][r] = qb[tr[r] * q.sL + cc];
-                w.Oc[b][r] = row_ok[r] ? gob[tr[r] * go.sL + cc] : 0.f;
-                w.Dc[b][r] = db[tr[r] * D + cc];
+                w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+                w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < NM; b++) {
+            w.Ot[b] = gob.f4(o_ot + 64 * b, os);
+            w.Dt[b] = db.f4(o_dt + 64 * b, ds);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Oc[b][r] = gob.f(o_or[r] + 64 * b, os);
+                w.Dc[b][r] = db.f(o_dr[r] + 64 * b, ds);
             }
         }
     };
 
-    // St[mb][eb]: register r = S[16eb + c][16mb + 4g + r]  (block (mb, eb) of S^T)
-    // dS[eb][mb]: register r = dS[16eb + 4g + r][16mb + c]
-    v4f St[NB][NB], dS[NB][NB];
+    // dS[eb][mb]: register r = dS[16 eb + 4g + r][16 mb + c]
+    // St[mb][eb]: register r = S[16 eb + c][16 mb + 4g + r]  (block (mb, eb) of S^T)
+    v4f dS[NE][NM], St[NM][NE];
 #pragma unroll
-    for (int a = 0; a < NB; a++)
+    for (int eb = 0; eb < NE; eb++)
 #pragma unroll
-        for (int b = 0; b < NB; b++) dS[a][b] = zero;
+        for (int mb = 0; mb < NM; mb++) dS[eb][mb] = zero;
 
-    // Gradients of a block wait in registers and are stored at the top of the next block (see the
-    // forward kernel).
-    v4f pend_gv[NB], pend_gq[NB], pend_gk[NB];
-    float pend_gb = 0.f;
-    auto flush = [&](auto full_tag, int ib) {
-        constexpr bool FULL = decltype(full_tag)::value;
-        const int t0 = ib * kBlk;
-        if (FULL || t0 + c < L) {      // register r = gradient[t0 + c][16b + 4g + r]
-            const int64_t o = (seq * L + t0 + c) * D + 4 * g;
+    auto block = [&](int e, const BwdRaw<NE, NM> &w) {
+        const int ib = nblk - 1 - e;
+        if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
 #pragma unroll
-            for (int b = 0; b < NB; b++) {
-                *reinterpret_cast<float4 *>(gv + o + 16 * b) =
-                    make_float4(pend_gv[b][0], pend_gv[b][1], pend_gv[b][2], pend_gv[b][3]);
-                *reinterpret_cast<float4 *>(gq + o + 16 * b) =
-                    make_float4(pend_gq[b][0], pend_gq[b][1], pend_gq[b][2], pend_gq[b][3]);
-                *reinterpret_cast<float4 *>(gk + o + 16 * b) =
-                    make_float4(pend_gk[b][0], pend_gk[b][1], pend_gk[b][2], pend_gk[b][3]);
-            }
-            if (g == 0) gbeta[seq * L + t0 + c] = pend_gb;
+            for (int mb = 0; mb < NM; mb++)
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) St[mb][eb] = w.Sck[mb][eb];
         }
-    };
-
-    auto block = [&](auto full_tag, int ib, const RawBwd<NB> &w) {
-        constexpr bool FULL = decltype(full_tag)::value;     // the block lies inside the sequence
-        const int t0 = ib * kBlk;
-        const int t_end = min(t0 + kBlk, L);
-        if (t_end % chunk == 0 || t_end == L) {      // last block of a chunk: the state after it is checkpointed
-#pragma unroll
-            for (int mb = 0; mb < NB; mb++)
-#pragma unroll
-                for (int eb = 0; eb < NB; eb++) St[mb][eb] = w.Sck[mb][eb];
-        }
-        v4f U[NB], Ut[NB], nU[NB];
-#pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
-            Ut[mb] = w.bcol * w.Dt[mb];
-#pragma unroll
-            for (int r = 0; r < 4; r++) U[mb][r] = w.brow[r] * w.Dc[mb][r];
-            nU[mb] = -U[mb];
-        }
-        // state at the start of the block, transposed: S0^T = S'^T - U^T K
-#pragma unroll
-        for (int mb = 0; mb < NB; mb++)
-#pragma unroll
-            for (int eb = 0; eb < NB; eb++) St[mb][eb] = tn(nU[mb], w.Kc[eb], St[mb][eb]);
-
-        // Pm = lower(Q K^T); T = (I + A)^-1 from forward, or inverted again here
         v4f QK = zero;
 #pragma unroll
-        for (int b = 0; b < NB; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
+        for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
         v4f Pm;
 #pragma unroll
         for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
@@ -447,107 +391,90 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_bwd_mfma(fwp_view q, f
         if (!have_T) {
             v4f G = zero, A, At;
 #pragma unroll
-            for (int b = 0; b < NB; b++) G = tn(w.Kt[b], w.Kt[b], G);
+            for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
                 At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
             }
-            T = inv_unit_triangular(At, A, ident);      // (I + A)^-1
+            T = inv_unit_triangular_lds(At, A, ident, scratch, p, lane);      // (I + A)^-1
         }
-
-        // gradient of u and everything that hangs off it
-        v4f dX[NB], dXt[NB], ndX[NB], ndXt[NB];
+        // state at the start of the block, transposed: S0^T = S'^T - U^T K
+        v4f Ut[NM];
+#pragma unroll
+        for (int mb = 0; mb < NM; mb++) {
+            Ut[mb] = w.bcol * w.Dt[mb];
+            v4f nU;
+#pragma unroll
+            for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[mb][r]);
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) St[mb][eb] = tn(nU, w.Kc[eb], St[mb][eb]);
+        }
+        // the adjoint chain of the block, per 16 value columns
+        v4f dXt[NM], ndX[NM], Z = zero, Mx = zero;
         float gb = 0.f;
 #pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
+        for (int mb = 0; mb < NM; mb++) {
             v4f dU = tn(Pm, w.Oc[mb], zero);
 #pragma unroll
-            for (int eb = 0; eb < NB; eb++) dU = tn(w.Kt[eb], dS[eb][mb], dU);
-            const v4f dY = tn(T, dU, zero), dYt = tn(dU, T, zero);
-            dXt[mb] = w.bcol * dYt;
-            ndXt[mb] = -dXt[mb];
+            for (int eb = 0; eb < NE; eb++) dU = tn(w.Kt[eb], dS[eb][mb], dU);
+            const v4f dY = tn(T, dU, zero);
+            scratch[0].put_t(p, dY);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                dX[mb][r] = w.brow[r] * dY[r];
-                gb = fmaf(dYt[r], w.Dt[mb][r], gb);
-            }
-            ndX[mb] = -dX[mb];
-            pend_gv[mb] = dXt[mb];
+            for (int r = 0; r < 4; r++) ndX[mb][r] = -(w.brow[r] * dY[r]);
+            Z = tn(w.Ot[mb], Ut[mb], Z);      // dO U^T
+            __builtin_amdgcn_wave_barrier();
+            const v4f dYt = scratch[0].get(lane);
+            dXt[mb] = w.bcol * dYt;
+#pragma unroll
+            for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[mb][r], gb);
+            // register r = g_v[t0 + c][16 mb + 4g + r]
+            gvb.st4(dXt[mb], o_dt + 64 * mb, ib * d_step);
+            Mx = tn(dXt[mb], Ut[mb], Mx);     // dX U^T
         }
-        {   // g_beta[t0 + c] = sum over the value index: the four 16-lane rows hold partial sums
+        {   // g_beta[t0 + c]: the four 16-lane rows hold partial sums
             float y = gb;
             swap16(gb, y);
             gb += y;
             y = gb;
             swap32(gb, y);
             gb += y;
-            pend_gb = gb;
+            if (g == 0) gbb.st(gb, c * 4, ib * kBlk * 4);
         }
-        v4f Z = zero, Zt = zero, M = zero, Mt = zero;
-#pragma unroll
-        for (int mb = 0; mb < NB; mb++) {
-            Z = tn(w.Ot[mb], Ut[mb], Z);          // dO U^T
-            Zt = tn(Ut[mb], w.Ot[mb], Zt);
-            M = tn(dXt[mb], Ut[mb], M);           // dX U^T
-            Mt = tn(Ut[mb], dXt[mb], Mt);
-        }
-        v4f dPm, dPmt, nMs;
+        v4f dPm, nM;
 #pragma unroll
         for (int r = 0; r < 4; r++) {
             dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-            dPmt[r] = (p.up[r] || p.di[r]) ? Zt[r] : 0.f;
-            nMs[r] = -((p.lo[r] ? M[r] : 0.f) + (p.up[r] ? Mt[r] : 0.f));
+            nM[r] = p.lo[r] ? -Mx[r] : 0.f;
         }
+        scratch[1].put_t(p, dPm);
+        scratch[2].put_t(p, nM);
+        __builtin_amdgcn_wave_barrier();
+        const v4f dPmt = scratch[1].get(lane);
+        const v4f nMs = nM + scratch[2].get(lane);
+        // g_q, g_k per 16 key columns (with dS as it was after the block), then dS for the block before
 #pragma unroll
-        for (int eb = 0; eb < NB; eb++) {
-            v4f gQt = tn(w.Kc[eb], dPmt, zero);
-            v4f gKt = tn(w.Qc[eb], dPm, zero);
+        for (int eb = 0; eb < NE; eb++) {
+            v4f gQt = tn(w.Kc[eb], dPmt, zero), gKt = tn(w.Qc[eb], dPm, zero);
             gKt = tn(w.Kc[eb], nMs, gKt);
 #pragma unroll
-            for (int mb = 0; mb < NB; mb++) {
-                const v4f dSt = tn(dS[eb][mb], ident, zero);       // block (mb, eb) of dS^T
+            for (int mb = 0; mb < NM; mb++) {
+                LdsMat &tr = scratch[(eb * NM + mb) % 2 ? 3 : 0];
+                tr.put_t(p, dS[eb][mb]);
                 gQt = tn(St[mb][eb], w.Ot[mb], gQt);
+                gKt = tn(St[mb][eb], -dXt[mb], gKt);
+                __builtin_amdgcn_wave_barrier();
+                const v4f dSt = tr.get(lane);            // block (mb, eb) of dS^T
                 gKt = tn(dSt, Ut[mb], gKt);
-                gKt = tn(St[mb][eb], ndXt[mb], gKt);
-            }
-            pend_gq[eb] = gQt;
-            pend_gk[eb] = gKt;
-        }
-#pragma unroll
-        for (int eb = 0; eb < NB; eb++)
-#pragma unroll
-            for (int mb = 0; mb < NB; mb++) {
                 dS[eb][mb] = tn(w.Qc[eb], w.Oc[mb], dS[eb][mb]);
                 dS[eb][mb] = tn(w.Kc[eb], ndX[mb], dS[eb][mb]);
             }
-    };
-
-    // The ragged last block first (clamped variant), then one straight-line loop over whole blocks.
-    const int nblk = (L + kBlk - 1) / kBlk;
-    RawBwd<NB> cur, nxt;
-    load(cur, (nblk - 1) * kBlk);
-    int ib = nblk - 1;
-    const bool ragged = nblk * kBlk != L;
-    if (ragged) {
-        load(nxt, max(ib - 1, 0) * kBlk);
-        __builtin_amdgcn_sched_barrier(0);
-        block(std::false_type(), ib, cur);
-        cur = nxt;
-        ib--;
-    }
-    for (; ib >= 0; ib--) {
-        load(nxt, max(ib - 1, 0) * kBlk);
-        if (ib + 1 < nblk) {        // the block done before this one
-            if (ragged && ib + 2 == nblk) flush(std::false_type(), ib + 1);
-            else flush(std::true_type(), ib + 1);
+            // register r = gradient[t0 + c][16 eb + 4g + r]
+            gqb.st4(gQt, o_ge + 64 * eb, ib * e_step);
+            gkb.st4(gKt, o_ge + 64 * eb, ib * e_step);
         }
-        __builtin_amdgcn_sched_barrier(0);      // loads and stores stay a whole block ahead of the next wait
-        block(std::true_type(), ib, cur);
-        cur = nxt;
-    }
-    if (nblk == 1 && ragged) flush(std::false_type(), 0);
-    else flush(std::true_type(), 0);
+    };
+    ring_loop<PF, BwdRaw<NE, NM>, false>(nblk, load, block);
 }
 
 // ------------------------------------------------------------------ sum rule
@@ -868,12 +795,13 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
     const float *aux = delta_aux_of(ckpt, N, H, L, D, D, chunk);
     const int spw = seq_per_wg(N * H);
     const dim3 grid((N * H + spw - 1) / spw), block(64 * spw);
+    const size_t lds = spw * 4 * sizeof(LdsMat);
     if (D == 16)
-        hipLaunchKernelGGL(k_delta_bwd_mfma<1>, grid, block, 0, s, q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv,
-                           gbeta, N * H, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_bwd_mfma<1, 1>), grid, block, lds, s, q, k, beta, vdiff, go, ckpt, aux, gq, gk,
+                           gv, gbeta, N * H, H, L, chunk, nchunk);
     else
-        hipLaunchKernelGGL(k_delta_bwd_mfma<2>, grid, block, 0, s, q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv,
-                           gbeta, N * H, H, L, chunk, nchunk);
+        hipLaunchKernelGGL((k_delta_bwd_mfma<2, 2>), grid, block, lds, s, q, k, beta, vdiff, go, ckpt, aux, gq, gk,
+                           gv, gbeta, N * H, H, L, chunk, nchunk);
     return (int)hipGetLastError();
 }
 
