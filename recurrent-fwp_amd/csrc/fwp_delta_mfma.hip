@@ -1,25 +1,25 @@
-// Chunked delta-rule kernels on the matrix cores (fp32 MFMA), E = M = D in {16, 32}.
+// Chunked delta-rule kernels on the matrix cores (fp32 MFMA), E = M = D in {16, 32}, and the
+// chunked sum-rule kernels; one wave per sequence.
 //
 // Inside a block of C = 16 steps the delta rule is a small triangular system: with S the state at
 // the start of the block, K, Q, V the block's rows and b its write strengths,
 //     A = strict_lower(diag(b) K K^T)              X = V - K S
 //     U = (I + A)^-1 diag(b) X                     (the values actually written, u_t = b_t d_t)
-//     d = X - strict_lower(K K^T) U                (v - v_old per step)
+//     d = X - strict_lower(K K^T) U = U / b        (v - v_old per step)
 //     O = Q S + lower(Q K^T) U                     S' = S + K^T U
-// (I + A)^-1 = (I - A)(I + A^2)(I + A^4)(I + A^8) because A is nilpotent of order 16, so the whole
-// block is 16x16x16 products; only X -> U -> S' lies on the sequential path.
+// T = (I + A)^-1 is found by substitution on the vector ALU (SolveRow); the rest is 16x16x16
+// products, of which only X -> U -> S' lies on the sequential path.
 //
-// One wave64 per sequence.  Every 16x16 matrix lives in the accumulator layout of
-// v_mfma_f32_16x16x4_f32 (4 VGPRs: lane l, register r holds element [4*(l/16) + r][l % 16]).  In that
-// layout register r of a matrix is directly the B operand of the r-th MFMA of a product, and the
-// A operand of the transposed matrix, so the primitive is  tn(X, Y, acc) = acc + X^T Y  with no
-// data movement between products; transposed inputs (K^T, Q^T) are single 16-byte loads per lane,
-// and the output is produced as O^T so that it leaves with 16-byte stores.  No LDS is used.
+// Every 16x16 matrix lives in the accumulator layout of v_mfma_f32_16x16x4_f32 (4 VGPRs: lane l,
+// register r holds element [4*(l/16) + r][l % 16]).  In that layout register r of a matrix is
+// directly the B operand of the r-th MFMA of a product, and the A operand of the transposed
+// matrix, so the primitive is  tn(X, Y, acc) = acc + X^T Y  with no data movement between products;
+// transposed inputs (K^T, Q^T, V^T) are single 16-byte loads per lane, outputs are produced
+// transposed so that they leave with 16-byte stores, and what is needed both ways round is
+// transposed through LDS.
 #include "fwp_common.hpp"
 #include "fwp_wave.hpp"
 #include "fwp_mfma.hpp"
-
-#include <type_traits>
 
 namespace fwp {
 namespace {

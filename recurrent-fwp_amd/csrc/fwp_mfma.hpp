@@ -23,19 +23,6 @@ __device__ __forceinline__ v4f tn(v4f X, v4f Y, v4f acc) {
 constexpr int kBlk = 16;   // steps per block = MFMA tile edge
 constexpr int kAuxHeader = 16;   // floats before the per-block matrices in the auxiliary buffer
 
-// (I + At)^-1 for a strictly triangular 16x16 matrix given both as A and as its transpose At
-// (accumulator layout): (I - At)(I + At^2)(I + At^4)(I + At^8), 8 products.
-__device__ __forceinline__ v4f inv_unit_triangular(v4f A, v4f At, v4f identity) {
-    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f T = identity - At;
-    const v4f A2 = tn(At, A, zero), At2 = tn(A, At, zero);
-    T = tn(A2, T, T);
-    const v4f A4 = tn(At2, A2, zero), At4 = tn(A2, At2, zero);
-    T = tn(A4, T, T);
-    const v4f A8 = tn(At4, A4, zero);
-    return tn(A8, T, T);
-}
-
 // Position of this lane's four registers in the accumulator layout.
 struct Geo16 {
     int g, c;
