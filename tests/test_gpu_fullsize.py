@@ -120,6 +120,30 @@ def test_delta_rectangular_states_at_full_occupancy(fwp, E, M):
         assert np.all(np.abs(got - want) <= 1e-4 + 1e-3 * np.abs(want)), float(np.abs(got - want).max())
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 20000, 16), (1, 1, 70001, 32)])
+def test_delta_long_sequences_blocked_against_scan(fwp, shape):
+    """Thousands of blocks and checkpoints per sequence (32-bit block offsets, the chunk index
+    arithmetic, groups of four blocks with a partial last group): blocked kernels against the
+    step-by-step kernels, outputs, final state and gradients."""
+    N, H, T, D = shape
+    q, k, v, beta, W0, go = (dev(a) for a in delta_inputs(5, N, H, T, D, D, dtype=np.float32))
+    L_ = fwp._lib
+    res = {}
+    try:
+        for kind in ("scan", "chunked", "split"):
+            L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED,
+                                             "split": L_.DELTA_SPLIT}[kind])
+            W = W0.clone()
+            out, g = grads_of(lambda t: fwp.fast_weight_delta(*t, W), [q, k, v, beta], go)
+            res[kind] = (out, W, *g)
+    finally:
+        L_.config(L_.CFG_DELTA_KERNELS, L_.DELTA_AUTO)
+    for kind in ("chunked", "split"):
+        for i, (x, y) in enumerate(zip(res[kind], res["scan"])):
+            assert torch.isfinite(x).all()
+            assert torch.allclose(x, y, atol=1e-4, rtol=1e-3), (kind, i, float((x - y).abs().max()))
+
+
 def test_rnn_full_size_properties(fwp):
     z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(1, 64, 8, 256, 32, dtype=np.float32))
 
