@@ -59,7 +59,8 @@ def test_delta_full_size_properties(fwp):
     assert torch.allclose(g3[2], 2 * g1[2], atol=1e-5, rtol=1e-5)
 
 
-@pytest.mark.parametrize("shape", [(96, 8, 256, 16), (32, 8, 1024, 32), (160, 8, 250, 16), (64, 8, 128, 32), (40, 8, 100, 16)])
+@pytest.mark.parametrize("shape", [(96, 8, 256, 16), (32, 8, 1024, 32), (160, 8, 250, 16), (64, 8, 128, 32), (40, 8, 100, 16),
+                                   (41, 25, 40, 16), (129, 9, 50, 32)])
 @pytest.mark.parametrize("op", ["delta", "sum"])
 def test_blocked_kernels_against_scan_kernels_at_full_occupancy(fwp, op, shape):
     """The blocked kernels (matrix cores, buffer-resource loads and stores) against the step-by-step
