@@ -662,13 +662,13 @@ namespace {
 constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }
 constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
 
-// The output wave is built for the two square shapes and used up to one and a half waves per SIMD
+// The output wave is built for one or two state waves and used up to one and a half waves per SIMD
 // (D = 16, forward at 256 / 512 / 768 sequences of 256 steps: 12.5 / 15.2 / 18.4 us with it,
 // 14.8 / 17.4 / 18.1 us without; D = 32, 256 sequences of 1024 steps: 54 against 62 us).
 template <int NE, int NM>
 void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
                 float *ckpt, float *aux, int nseq, int H, int L, int chunk, int nchunk, hipStream_t s) {
-    if constexpr (NE == NM && NE <= 2) {
+    if constexpr (NM <= 2) {
         if ((int64_t)nseq * (NM + 2) <= 1536) {
             hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), true>), dim3(nseq), dim3(64 * (NM + 2)), 0,
                                s, q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
