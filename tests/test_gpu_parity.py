@@ -168,12 +168,16 @@ def test_delta_strided_views_and_segments(fwp, delta_kernels):
     check("grad_beta", tb.grad[:, :, a], refs[3])
 
 
-def test_delta_no_grad_path(fwp):
-    q, k, v, beta, W0, _ = delta_inputs(8, 2, 2, 40, 16, 16)
+@pytest.mark.parametrize("E,M,L", [(16, 16, 40), (32, 32, 100), (96, 16, 50), (16, 64, 33)])
+def test_delta_no_grad_path(fwp, delta_kernels, E, M, L):
+    # nothing is saved for backward: no vdiff, no checkpoints, no per-block inverses
+    q, k, v, beta, W0, _ = delta_inputs(8, 2, 2, L, E, M, w0=True)
     with torch.no_grad():
         W = dev(W0)
         out = fwp.fast_weight_delta(dev(q), dev(k), dev(v), dev(beta), W)
-    check("out", out, oracle.delta_fwd(q, k, v, beta, W0)[0])
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
 
 
 RNN_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 64, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
