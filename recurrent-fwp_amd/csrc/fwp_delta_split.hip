@@ -646,6 +646,262 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
     ring_loop<PF, StateRaw<NM>>(nblk, load, block);
 }
 
+// ------------------------------------------------- backward, E = M = 16, four waves per sequence
+//
+// The same algebra cut into four roles of 12-16 MFMAs per block, one wave each, so that the four
+// waves of a workgroup take one SIMD each and every SIMD of a CU holds the same load whatever the
+// number of sequences.  In round r (one barrier per round):
+//   P  block r      Pm = lower(Q K^T), Pm^T dO, Q^T dO, dPm = lower(dO U^T)       (nothing of the chain)
+//   C  block r - 1  dU = K dS + Pm^T dO, dY = T^T dU, dS <- dS + Q^T dO - K^T dX   (the chain)
+//   R  block r - 2  S0^T = S'^T - U^T K, g_q = dO S0^T + dPm K, -dX S0^T           (the state)
+//   G  block r - 2  g_v, g_beta, M, U dS^T + dPm^T Q - (M + M^T) K;  g_k one round later, with R's term
+// Hand-over through LDS: P -> C two slots alternately, P -> R, G three (read two rounds later),
+// C -> R, G two, R -> G two.
+struct QuadP {
+    v4f Kt, Qt, Qc, Oc, Ot, Dt;
+    float bcol;
+};
+struct QuadC {
+    v4f Kt, Kc, T;
+    float bcol, brow[4];
+};
+struct QuadR {
+    v4f Kc, Dc, Ot, Sck;
+    float bcol, brow[4];
+};
+struct QuadG {
+    v4f Kc, Qc, Dt;
+    float bcol;
+};
+
+template <int PF>
+__global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, fwp_view beta,
+                                                        const float *__restrict__ vdiff, fwp_view go,
+                                                        const float *__restrict__ ckpt,
+                                                        const float *__restrict__ aux,
+                                                        float *__restrict__ gq, float *__restrict__ gk,
+                                                        float *__restrict__ gv, float *__restrict__ gbeta,
+                                                        int H, int L, int chunk, int nchunk) {
+    constexpr int E = 16, M = 16;
+    __shared__ LdsMat pc[2][2];        // P -> C: Pm^T dO, Q^T dO
+    __shared__ LdsMat pg[3][2];        // P -> G, R: dPm, dPm^T
+    __shared__ LdsMat cg[2][2];        // C -> G, R: dS^T (before the block's update), dY^T
+    __shared__ LdsMat rg[2];           // R -> G: -dX S0^T, transposed like g_k
+    __shared__ LdsMat own[3];          // transposes inside P and G, the inverse inside C
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
+    const int lane = threadIdx.x % 64;
+    const Geo16 p(lane);
+    const int g = p.g, c = p.c;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const int nblk = (L + kBlk - 1) / kBlk;
+    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
+        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
+        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + M) * 4)),
+        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
+        db(vdiff + seq * L * M, (uint32_t)(L * M * 4));
+    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
+                   o_step = (unsigned)(kBlk * go.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
+                   d_step = (unsigned)(kBlk * M * 4), e_step = (unsigned)(kBlk * E * 4);
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
+    const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
+                   o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4;
+    unsigned o_br[4], o_kr[4], o_qr[4], o_or[4], o_dr[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
+        o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
+        o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
+        o_or[r] = (unsigned)((4 * g + r) * go.sL + c) * 4;
+        o_dr[r] = (unsigned)((4 * g + r) * M + c) * 4;
+    }
+    auto third = [](int e) { return e - 3 * (int)__umulhi((unsigned)e, 0x55555556u); };   // e % 3
+
+    if (wave == 0) {
+        // ------------------------------------------------ P
+        auto load = [&](QuadP &w, int e) {
+            const int ib = nblk - 1 - e;
+            const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step;
+            w.bcol = bb.f(o_bc, ib * b_step);
+            w.Kt = kb.f4(o_kt, ks);
+            w.Qt = qb.f4(o_qt, qs);
+            w.Ot = gob.f4(o_ot, os);
+            w.Dt = db.f4(o_dt, ib * d_step);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Qc[r] = qb.f(o_qr[r], qs);
+                w.Oc[r] = gob.f(o_or[r], os);
+            }
+        };
+        auto block = [&](int e, const QuadP &w) {
+            const v4f QK = tn(w.Qt, w.Kt, zero);
+            v4f Pm;
+#pragma unroll
+            for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
+            const v4f Ut = w.bcol * w.Dt;
+            const v4f Z = tn(w.Ot, Ut, zero);          // dO U^T
+            pc[e & 1][0].put(lane, tn(Pm, w.Oc, zero));
+            pc[e & 1][1].put(lane, tn(w.Qc, w.Oc, zero));
+            v4f dPm;
+#pragma unroll
+            for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
+            LdsMat *to = pg[third(e)];
+            to[0].put(lane, dPm);
+            to[1].put_t(p, dPm);
+        };
+        ring_loop<PF, QuadP>(nblk, load, block);
+        lds_barrier();
+        lds_barrier();
+        lds_barrier();
+        return;
+    }
+    if (wave == 1) {
+        // ------------------------------------------------ C
+        // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
+        const bool have_T = aux && aux[0] == 1.f;
+        const RowBuf tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0);
+        const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4;
+        v4f ident;
+#pragma unroll
+        for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
+        auto load = [&](QuadC &w, int e) {
+            const int ib = nblk - 1 - e;
+            if (have_T) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
+            }
+            const unsigned ks = ib * k_step, bs = ib * b_step;
+            w.bcol = bb.f(o_bc, bs);
+            w.Kt = kb.f4(o_kt, ks);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.brow[r] = bb.f(o_br[r], bs);
+                w.Kc[r] = kb.f(o_kr[r], ks);
+            }
+        };
+        v4f dS = zero;        // register r = dS[4g + r][c]
+        auto block = [&](int e, const QuadC &w) {
+            v4f T = w.T;
+            if (!have_T) {
+                const v4f G = tn(w.Kt, w.Kt, zero);
+                v4f A, At;
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
+                    At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
+                }
+                T = inv_unit_triangular_lds(At, A, ident, own, p, lane);      // (I + A)^-1
+            }
+            const v4f dU0 = pc[e & 1][0].get(lane), dSi = pc[e & 1][1].get(lane);
+            cg[e & 1][0].put_t(p, dS);
+            const v4f dU = tn(w.Kt, dS, dU0);
+            const v4f dY = tn(T, dU, zero);
+            cg[e & 1][1].put_t(p, dY);
+            v4f ndX;
+#pragma unroll
+            for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
+            dS = tn(w.Kc, ndX, dS + dSi);
+        };
+        lds_barrier();
+        ring_loop<PF, QuadC>(nblk, load, block);
+        lds_barrier();
+        lds_barrier();
+        return;
+    }
+    if (wave == 2) {
+        // ------------------------------------------------ R
+        const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
+            gqb(gq + seq * L * E, (uint32_t)(L * E * 4));
+        const ChunkOf chunk_of(chunk);
+        auto load = [&](QuadR &w, int e) {
+            const int ib = nblk - 1 - e;
+            w.Sck = cb.f4(o_dt, chunk_of(ib) * (E * M * 4));       // register r = S[c][4g + r]
+            const unsigned ks = ib * k_step, bs = ib * b_step, ds = ib * d_step;
+            w.bcol = bb.f(o_bc, bs);
+            w.Ot = gob.f4(o_ot, ib * o_step);
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.brow[r] = bb.f(o_br[r], bs);
+                w.Kc[r] = kb.f(o_kr[r], ks);
+                w.Dc[r] = db.f(o_dr[r], ds);
+            }
+        };
+        v4f St = zero;        // register r = S[c][4g + r]
+        auto block = [&](int e, const QuadR &w) {
+            const int ib = nblk - 1 - e;
+            if (chunk_of.closes(ib) || ib + 1 == nblk) St = w.Sck;      // the state after the block is checkpointed
+            v4f nU;
+#pragma unroll
+            for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[r]);
+            St = tn(nU, w.Kc, St);                                      // S0^T = S'^T - U^T K
+            v4f gQt = tn(St, w.Ot, zero);
+            const v4f dPmt = pg[third(e)][1].get(lane);
+            const v4f dXt = w.bcol * cg[e & 1][1].get(lane);
+            gQt = tn(w.Kc, dPmt, gQt);
+            rg[e & 1].put(lane, tn(St, -dXt, zero));
+            gqb.st4(gQt, o_dt, ib * e_step);        // register r = g_q[t0 + c][4g + r]
+        };
+        lds_barrier();
+        lds_barrier();
+        ring_loop<PF, QuadR>(nblk, load, block);
+        lds_barrier();
+        return;
+    }
+    // ---------------------------------------------------- G
+    const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)), gvb(gv + seq * L * M, (uint32_t)(L * M * 4)),
+        gbb(gbeta + seq * L, (uint32_t)(L * 4));
+    auto load = [&](QuadG &w, int e) {
+        const int ib = nblk - 1 - e;
+        const unsigned ks = ib * k_step, qs = ib * q_step;
+        w.bcol = bb.f(o_bc, ib * b_step);
+        w.Dt = db.f4(o_dt, ib * d_step);
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            w.Kc[r] = kb.f(o_kr[r], ks);
+            w.Qc[r] = qb.f(o_qr[r], qs);
+        }
+    };
+    v4f gKt = zero;           // of the block before, still without R's term
+    auto finish = [&](int e) {        // g_k of block e (as counted from the end)
+        gkb.st4(gKt + rg[e & 1].get(lane), o_dt, (nblk - 1 - e) * e_step);
+    };
+    auto block = [&](int e, const QuadG &w) {
+        const int ib = nblk - 1 - e;
+        if (e > 0) finish(e - 1);
+        const v4f dSt = cg[e & 1][0].get(lane), dYt = cg[e & 1][1].get(lane);
+        const v4f dPm = pg[third(e)][0].get(lane);
+        const v4f dXt = w.bcol * dYt, Ut = w.bcol * w.Dt;
+        gvb.st4(dXt, o_dt, ib * d_step);            // register r = g_v[t0 + c][4g + r]
+        float gb = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
+        {   // g_beta[t0 + c]: the four 16-lane rows hold partial sums
+            float y = gb;
+            swap16(gb, y);
+            gb += y;
+            y = gb;
+            swap32(gb, y);
+            gb += y;
+            if (g == 0) gbb.st(gb, c * 4, ib * kBlk * 4);
+        }
+        const v4f Mx = tn(dXt, Ut, zero);           // dX U^T
+        v4f nM;
+#pragma unroll
+        for (int r = 0; r < 4; r++) nM[r] = p.lo[r] ? -Mx[r] : 0.f;
+        own[2].put_t(p, nM);
+        gKt = tn(dSt, Ut, zero);
+        gKt = tn(w.Qc, dPm, gKt);
+        __builtin_amdgcn_wave_barrier();
+        gKt = tn(w.Kc, nM + own[2].get(lane), gKt);
+    };
+    lds_barrier();
+    lds_barrier();
+    ring_loop<PF, QuadG>(nblk, load, block);
+    finish(nblk - 1);
+    lds_barrier();
+}
+
 }  // namespace
 
 // Supported state shapes: E = 16 NE, M = 16 NM with NE in {1, 2, 4, 6}, NM in {1, 2, 4} and at most
@@ -707,6 +963,11 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
                     int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     const float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
+    if (E == 16 && M == 16) {
+        hipLaunchKernelGGL(k_delta_bwd_quad<3>, dim3(N * H), dim3(256), 0, s, q, k, beta, vdiff, go, ckpt, aux, gq,
+                           gk, gv, gbeta, H, L, chunk, nchunk);
+        return (int)hipGetLastError();
+    }
 #define X(ne, nm)                                                                                        \
     if (E == 16 * ne && M == 16 * nm)                                                                    \
         launch_bwd<ne, nm>(q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, N * H, H, L, chunk, nchunk, s);
