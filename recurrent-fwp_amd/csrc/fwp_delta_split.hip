@@ -57,8 +57,10 @@ struct OutRaw {
 
 // OUT: one more wave takes the products that only feed the output (S^T Q^T, lower(Q K^T), O), one
 // block behind the state waves, which hand it their columns of the state and of U.
+// With one state wave and the output wave a fourth wave only keeps the barriers: the four waves of a
+// 256-thread workgroup take one SIMD each, three-wave workgroups are placed unevenly.
 template <int NE, int NM, int PF, bool OUT>   // E = 16 NE, M = 16 NM, PF = blocks in flight
-__global__ __launch_bounds__(64 * (NM + 1 + OUT)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
+__global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
                                                                   fwp_view beta, float *__restrict__ W,
                                                                   float *__restrict__ out,
                                                                   float *__restrict__ vdiff,
@@ -192,6 +194,10 @@ __global__ __launch_bounds__(64 * (NM + 1 + OUT)) void k_delta_fwd_split(fwp_vie
     }
 
     const unsigned m_step = (unsigned)(kBlk * M * 4);
+    if (OUT && wave == NM + 2) {       // the wave that fills the workgroup up to four
+        for (int r = 0; r < nblk + 2; r++) lds_barrier();
+        return;
+    }
     if (OUT && wave == NM + 1) {
         // ------------------------------------------------ output wave, one block behind
         using Raw = OutRaw<NE, !kPrepQK>;
@@ -918,15 +924,17 @@ namespace {
 constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }
 constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
 
-// The output wave is built for one or two state waves and used up to one and a half waves per SIMD
-// (D = 16, forward at 256 / 512 / 768 sequences of 256 steps: 12.5 / 15.2 / 18.4 us with it,
-// 14.8 / 17.4 / 18.1 us without; D = 32, 256 sequences of 1024 steps: 54 against 62 us).
+// The output wave is built for one or two state waves; with one (a workgroup of four waves, one per
+// SIMD) it is always used, with two up to one and a half waves per SIMD (D = 16, forward at 256 / 512 /
+// 768 / 1024 sequences of 256 steps: 12.5 / 15.0 / 18.2 / 20.7 us with it, 14.8 / 17.4 / 18.2 / 21.7 us
+// without; D = 32, 256 sequences of 1024 steps: 54 against 62 us).
 template <int NE, int NM>
 void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
                 float *ckpt, float *aux, int nseq, int H, int L, int chunk, int nchunk, hipStream_t s) {
     if constexpr (NM <= 2) {
-        if ((int64_t)nseq * (NM + 2) <= 1536) {
-            hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), true>), dim3(nseq), dim3(64 * (NM + 2)), 0,
+        if (NM == 1 || (int64_t)nseq * (NM + 2) <= 1536) {
+            hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), true>), dim3(nseq),
+                               dim3(64 * (NM == 1 ? 4 : NM + 2)), 0,
                                s, q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
             return;
         }
