@@ -662,7 +662,8 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
 //   R  block r - 2  S0^T = S'^T - U^T K, g_q = dO S0^T + dPm K, -dX S0^T           (the state)
 //   G  block r - 2  g_v, g_beta, M, U dS^T + dPm^T Q - (M + M^T) K;  g_k one round later, with R's term
 // Hand-over through LDS: P -> C two slots alternately, P -> R, G three (read two rounds later),
-// C -> R, G two, R -> G two.
+// C -> R, G two, R -> G two.  Rows that P or C have read anyway and R or G need too (K, Q, dO, d,
+// beta) travel the same way instead of being read from memory again.
 struct QuadP {
     v4f Kt, Qt, Qc, Oc, Ot, Dt;
     float bcol;
@@ -672,12 +673,8 @@ struct QuadC {
     float bcol, brow[4];
 };
 struct QuadR {
-    v4f Kc, Dc, Ot, Sck;
-    float bcol, brow[4];
-};
-struct QuadG {
-    v4f Kc, Qc, Dt;
-    float bcol;
+    v4f Dc, Sck;
+    float brow[4];
 };
 
 template <int PF>
@@ -690,8 +687,9 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
                                                         int H, int L, int chunk, int nchunk) {
     constexpr int E = 16, M = 16;
     __shared__ LdsMat pc[2][2];        // P -> C: Pm^T dO, Q^T dO
-    __shared__ LdsMat pg[3][2];        // P -> G, R: dPm, dPm^T
-    __shared__ LdsMat cg[2][2];        // C -> G, R: dS^T (before the block's update), dY^T
+    __shared__ LdsMat pg[3][5];        // P -> G, R: dPm, dPm^T, Q (rows), d^T, dO^T
+    __shared__ float pb[3][16];        // P -> G, R: beta[t0 + c]
+    __shared__ LdsMat cg[2][3];        // C -> G, R: dS^T (before the block's update), dY^T, K (rows)
     __shared__ LdsMat rg[2];           // R -> G: -dX S0^T, transposed like g_k
     __shared__ LdsMat own[3];          // transposes inside P and G, the inverse inside C
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -752,9 +750,14 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
             v4f dPm;
 #pragma unroll
             for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-            LdsMat *to = pg[third(e)];
+            const int s3 = third(e);
+            LdsMat *to = pg[s3];
             to[0].put(lane, dPm);
             to[1].put_t(p, dPm);
+            to[2].put(lane, w.Qc);
+            to[3].put(lane, w.Dt);
+            to[4].put(lane, w.Ot);
+            if (g == 0) pb[s3][c] = w.bcol;
         };
         ring_loop<PF, QuadP>(nblk, load, block);
         lds_barrier();
@@ -804,6 +807,7 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
             const v4f dU = tn(w.Kt, dS, dU0);
             const v4f dY = tn(T, dU, zero);
             cg[e & 1][1].put_t(p, dY);
+            cg[e & 1][2].put(lane, w.Kc);
             v4f ndX;
 #pragma unroll
             for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
@@ -818,18 +822,15 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
     if (wave == 2) {
         // ------------------------------------------------ R
         const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
-            gqb(gq + seq * L * E, (uint32_t)(L * E * 4));
+            gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gvb(gv + seq * L * M, (uint32_t)(L * M * 4));
         const ChunkOf chunk_of(chunk);
         auto load = [&](QuadR &w, int e) {
             const int ib = nblk - 1 - e;
             w.Sck = cb.f4(o_dt, chunk_of(ib) * (E * M * 4));       // register r = S[c][4g + r]
-            const unsigned ks = ib * k_step, bs = ib * b_step, ds = ib * d_step;
-            w.bcol = bb.f(o_bc, bs);
-            w.Ot = gob.f4(o_ot, ib * o_step);
+            const unsigned bs = ib * b_step, ds = ib * d_step;
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 w.brow[r] = bb.f(o_br[r], bs);
-                w.Kc[r] = kb.f(o_kr[r], ks);
                 w.Dc[r] = db.f(o_dr[r], ds);
             }
         };
@@ -840,13 +841,16 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
             v4f nU;
 #pragma unroll
             for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[r]);
-            St = tn(nU, w.Kc, St);                                      // S0^T = S'^T - U^T K
-            v4f gQt = tn(St, w.Ot, zero);
-            const v4f dPmt = pg[third(e)][1].get(lane);
-            const v4f dXt = w.bcol * cg[e & 1][1].get(lane);
-            gQt = tn(w.Kc, dPmt, gQt);
+            const int s3 = third(e);
+            const v4f Kc = cg[e & 1][2].get(lane);
+            St = tn(nU, Kc, St);                                        // S0^T = S'^T - U^T K
+            v4f gQt = tn(St, pg[s3][4].get(lane), zero);
+            const v4f dPmt = pg[s3][1].get(lane);
+            const v4f dXt = pb[s3][c] * cg[e & 1][1].get(lane);
+            gQt = tn(Kc, dPmt, gQt);
             rg[e & 1].put(lane, tn(St, -dXt, zero));
             gqb.st4(gQt, o_dt, ib * e_step);        // register r = g_q[t0 + c][4g + r]
+            gvb.st4(dXt, o_dt, ib * d_step);        // register r = g_v[t0 + c][4g + r]
         };
         lds_barrier();
         lds_barrier();
@@ -854,34 +858,25 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
         lds_barrier();
         return;
     }
-    // ---------------------------------------------------- G
-    const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)), gvb(gv + seq * L * M, (uint32_t)(L * M * 4)),
-        gbb(gbeta + seq * L, (uint32_t)(L * 4));
-    auto load = [&](QuadG &w, int e) {
-        const int ib = nblk - 1 - e;
-        const unsigned ks = ib * k_step, qs = ib * q_step;
-        w.bcol = bb.f(o_bc, ib * b_step);
-        w.Dt = db.f4(o_dt, ib * d_step);
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            w.Kc[r] = kb.f(o_kr[r], ks);
-            w.Qc[r] = qb.f(o_qr[r], qs);
-        }
-    };
+    // ---------------------------------------------------- G (reads nothing from memory)
+    const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)), gbb(gbeta + seq * L, (uint32_t)(L * 4));
+    struct QuadG {};
+    auto load = [&](QuadG &, int) {};
     v4f gKt = zero;           // of the block before, still without R's term
     auto finish = [&](int e) {        // g_k of block e (as counted from the end)
         gkb.st4(gKt + rg[e & 1].get(lane), o_dt, (nblk - 1 - e) * e_step);
     };
-    auto block = [&](int e, const QuadG &w) {
+    auto block = [&](int e, const QuadG &) {
         const int ib = nblk - 1 - e;
         if (e > 0) finish(e - 1);
-        const v4f dSt = cg[e & 1][0].get(lane), dYt = cg[e & 1][1].get(lane);
-        const v4f dPm = pg[third(e)][0].get(lane);
-        const v4f dXt = w.bcol * dYt, Ut = w.bcol * w.Dt;
-        gvb.st4(dXt, o_dt, ib * d_step);            // register r = g_v[t0 + c][4g + r]
+        const int s3 = third(e);
+        const v4f dSt = cg[e & 1][0].get(lane), dYt = cg[e & 1][1].get(lane), Kc = cg[e & 1][2].get(lane);
+        const v4f dPm = pg[s3][0].get(lane), Qc = pg[s3][2].get(lane), Dt = pg[s3][3].get(lane);
+        const float bcol = pb[s3][c];
+        const v4f dXt = bcol * dYt, Ut = bcol * Dt;
         float gb = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
+        for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], Dt[r], gb);
         {   // g_beta[t0 + c]: the four 16-lane rows hold partial sums
             float y = gb;
             swap16(gb, y);
@@ -897,9 +892,9 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
         for (int r = 0; r < 4; r++) nM[r] = p.lo[r] ? -Mx[r] : 0.f;
         own[2].put_t(p, nM);
         gKt = tn(dSt, Ut, zero);
-        gKt = tn(w.Qc, dPm, gKt);
+        gKt = tn(Qc, dPm, gKt);
         __builtin_amdgcn_wave_barrier();
-        gKt = tn(w.Kc, nM + own[2].get(lane), gKt);
+        gKt = tn(Kc, nM + own[2].get(lane), gKt);
     };
     lds_barrier();
     lds_barrier();
