@@ -652,46 +652,57 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
     ring_loop<PF, StateRaw<NM>>(nblk, load, block);
 }
 
-// ------------------------------------------------- backward, E = M = 16, four waves per sequence
+// ------------------------------------------------- backward in four roles
 //
-// The same algebra cut into four roles of 12-16 MFMAs per block, one wave each, so that the four
-// waves of a workgroup take one SIMD each and every SIMD of a CU holds the same load whatever the
-// number of sequences.  In round r (one barrier per round):
-//   P  block r      Pm = lower(Q K^T), Pm^T dO, Q^T dO, dPm = lower(dO U^T)       (nothing of the chain)
-//   C  block r - 1  dU = K dS + Pm^T dO, dY = T^T dU, dS <- dS + Q^T dO - K^T dX   (the chain)
-//   R  block r - 2  S0^T = S'^T - U^T K, g_q = dO S0^T + dPm K, -dX S0^T           (the state)
-//   G  block r - 2  g_v, g_beta, M, U dS^T + dPm^T Q - (M + M^T) K;  g_k one round later, with R's term
-// Hand-over through LDS: P -> C two slots alternately, P -> R, G three (read two rounds later),
-// C -> R, G two, R -> G two.  Rows that P or C have read anyway and R or G need too (K, Q, dO, d,
-// beta) travel the same way instead of being read from memory again.
+// The same algebra cut into roles of a few products per block each, so that no wave carries much
+// more than the others however wide the keys are, and (E = M = 16: four waves) the waves of a
+// workgroup take one SIMD each.  In round r (one barrier per round):
+//   P      block r      Pm = lower(Q K^T), Pm^T dO, Q^T dO, dPm = lower(dO U^T)     (nothing of the chain)
+//   C[mb]  block r - 1  dU = K dS + Pm^T dO, dY = T^T dU, dS <- dS + Q^T dO - K^T dX (the chain, 16 value columns)
+//   R[j]   block r - 2  S0^T = S'^T - U^T K, g_q = dO S0^T + dPm K, -dX S0^T         (the state, its key tiles)
+//   G[j]   block r - 2  g_beta, M, U dS^T + dPm^T Q - (M + M^T) K;  g_k one round later, with R's term
+// R[j] and G[j] own the key tiles [j NE / WR, (j + 1) NE / WR).  Hand-over through LDS: P -> C two
+// slots alternately, P -> R, G three (read two rounds later), C -> R, G two, R -> G two.
+template <int NE, int NM>
 struct QuadP {
-    v4f Kt, Qt, Qc, Oc, Ot, Dt;
+    v4f Kt[NE], Qt[NE], Qc[NE], Oc[NM], Ot[NM], Dt[NM];
     float bcol;
 };
+template <int NE>
 struct QuadC {
-    v4f Kt, Kc, T;
+    v4f Kt[NE], Kc[NE], T;
     float bcol, brow[4];
 };
+template <int NEW, int NM>
 struct QuadR {
-    v4f Dc, Sck;
+    v4f Kc[NEW], Dc[NM], Sck[NM][NEW];
     float brow[4];
 };
+template <int NEW>
+struct QuadG {
+    v4f Kc[NEW], Qc[NEW];
+};
 
-template <int PF>
-__global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, fwp_view beta,
-                                                        const float *__restrict__ vdiff, fwp_view go,
-                                                        const float *__restrict__ ckpt,
-                                                        const float *__restrict__ aux,
-                                                        float *__restrict__ gq, float *__restrict__ gk,
-                                                        float *__restrict__ gv, float *__restrict__ gbeta,
-                                                        int H, int L, int chunk, int nchunk) {
-    constexpr int E = 16, M = 16;
-    __shared__ LdsMat pc[2][2];        // P -> C: Pm^T dO, Q^T dO
-    __shared__ LdsMat pg[3][5];        // P -> G, R: dPm, dPm^T, Q (rows), d^T, dO^T
-    __shared__ float pb[3][16];        // P -> G, R: beta[t0 + c]
-    __shared__ LdsMat cg[2][3];        // C -> G, R: dS^T (before the block's update), dY^T, K (rows)
-    __shared__ LdsMat rg[2];           // R -> G: -dX S0^T, transposed like g_k
-    __shared__ LdsMat own[3];          // transposes inside P and G, the inverse inside C
+template <int NE, int NM, int WR>
+constexpr int quad_lds_mats() {
+    return 2 * (NM + NE * NM) + 3 * (2 + 2 * NM) + 2 * (NE * NM + NM) + 2 * NE + 2 * NM + WR;
+}
+
+template <int NE, int NM, int WR, int PF>
+__global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
+    fwp_view q, fwp_view k, fwp_view beta, const float *__restrict__ vdiff, fwp_view go,
+    const float *__restrict__ ckpt, const float *__restrict__ aux, float *__restrict__ gq,
+    float *__restrict__ gk, float *__restrict__ gv, float *__restrict__ gbeta, int H, int L, int chunk,
+    int nchunk) {
+    constexpr int E = 16 * NE, M = 16 * NM, NEW = NE / WR;
+    static_assert(NE % WR == 0, "key tiles divide evenly over the waves of a role");
+    __shared__ LdsMat pc[2][NM + NE * NM];     // P -> C: Pm^T dO per mb, then Q^T dO per (eb, mb)
+    __shared__ LdsMat pg[3][2 + 2 * NM];       // P -> G, R: dPm, dPm^T, d^T per mb, dO^T per mb
+    __shared__ float pb[3][16];                // P -> G, R: beta[t0 + c]
+    __shared__ LdsMat cg[2][NE * NM + NM];     // C -> G, R: dS^T per (eb, mb) before the block's update, dY^T per mb
+    __shared__ LdsMat rg[2][NE];               // R -> G: -dX S0^T per eb, transposed like g_k
+    __shared__ LdsMat inv[NM][2];              // the inverse inside C where forward left none
+    __shared__ LdsMat own[WR];                 // the transpose inside G
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -710,7 +721,8 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
     const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
-                   o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4;
+                   o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4,
+                   o_ge = (unsigned)(c * E + 4 * g) * 4;
     unsigned o_br[4], o_kr[4], o_qr[4], o_or[4], o_dr[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
@@ -724,49 +736,61 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
 
     if (wave == 0) {
         // ------------------------------------------------ P
-        auto load = [&](QuadP &w, int e) {
+        using Raw = QuadP<NE, NM>;
+        auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
-            const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step;
+            const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step;
             w.bcol = bb.f(o_bc, ib * b_step);
-            w.Kt = kb.f4(o_kt, ks);
-            w.Qt = qb.f4(o_qt, qs);
-            w.Ot = gob.f4(o_ot, os);
-            w.Dt = db.f4(o_dt, ib * d_step);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                w.Qc[r] = qb.f(o_qr[r], qs);
-                w.Oc[r] = gob.f(o_or[r], os);
+            for (int b = 0; b < NE; b++) {
+                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
+            }
+#pragma unroll
+            for (int b = 0; b < NM; b++) {
+                w.Ot[b] = gob.f4(o_ot + 64 * b, os);
+                w.Dt[b] = db.f4(o_dt + 64 * b, ds);
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.Oc[b][r] = gob.f(o_or[r] + 64 * b, os);
             }
         };
-        auto block = [&](int e, const QuadP &w) {
-            const v4f QK = tn(w.Qt, w.Kt, zero);
+        auto block = [&](int e, const Raw &w) {
+            v4f QK = zero, Z = zero;
+#pragma unroll
+            for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
             v4f Pm;
 #pragma unroll
             for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
-            const v4f Ut = w.bcol * w.Dt;
-            const v4f Z = tn(w.Ot, Ut, zero);          // dO U^T
-            pc[e & 1][0].put(lane, tn(Pm, w.Oc, zero));
-            pc[e & 1][1].put(lane, tn(w.Qc, w.Oc, zero));
+            const int s3 = third(e);
+            LdsMat *to = pg[s3];
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) {
+                Z = tn(w.Ot[mb], w.bcol * w.Dt[mb], Z);         // dO U^T
+                pc[e & 1][mb].put(lane, tn(Pm, w.Oc[mb], zero));
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) pc[e & 1][NM + eb * NM + mb].put(lane, tn(w.Qc[eb], w.Oc[mb], zero));
+                to[2 + mb].put(lane, w.Dt[mb]);
+                to[2 + NM + mb].put(lane, w.Ot[mb]);
+            }
             v4f dPm;
 #pragma unroll
             for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-            const int s3 = third(e);
-            LdsMat *to = pg[s3];
             to[0].put(lane, dPm);
             to[1].put_t(p, dPm);
-            to[2].put(lane, w.Qc);
-            to[3].put(lane, w.Dt);
-            to[4].put(lane, w.Ot);
             if (g == 0) pb[s3][c] = w.bcol;
         };
-        ring_loop<PF, QuadP>(nblk, load, block);
+        ring_loop<PF, Raw>(nblk, load, block);
         lds_barrier();
         lds_barrier();
         lds_barrier();
         return;
     }
-    if (wave == 1) {
-        // ------------------------------------------------ C
+    if (wave <= NM) {
+        // ------------------------------------------------ C of value columns [16 mb, 16 mb + 16)
+        const int mb = wave - 1;
+        using Raw = QuadC<NE>;
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
         const bool have_T = aux && aux[0] == 1.f;
         const RowBuf tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0);
@@ -774,7 +798,7 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
         v4f ident;
 #pragma unroll
         for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-        auto load = [&](QuadC &w, int e) {
+        auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
             if (have_T) {
 #pragma unroll
@@ -782,101 +806,160 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
             }
             const unsigned ks = ib * k_step, bs = ib * b_step;
             w.bcol = bb.f(o_bc, bs);
-            w.Kt = kb.f4(o_kt, ks);
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                w.brow[r] = bb.f(o_br[r], bs);
-                w.Kc[r] = kb.f(o_kr[r], ks);
+            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
+#pragma unroll
+            for (int b = 0; b < NE; b++) {
+                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
             }
         };
-        v4f dS = zero;        // register r = dS[4g + r][c]
-        auto block = [&](int e, const QuadC &w) {
+        v4f dS[NE];           // register r = dS[16 eb + 4g + r][16 mb + c]
+#pragma unroll
+        for (int eb = 0; eb < NE; eb++) dS[eb] = zero;
+        auto block = [&](int e, const Raw &w) {
             v4f T = w.T;
             if (!have_T) {
-                const v4f G = tn(w.Kt, w.Kt, zero);
-                v4f A, At;
+                v4f G = zero, A, At;
+#pragma unroll
+                for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
                     At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
                 }
-                T = inv_unit_triangular_lds(At, A, ident, own, p, lane);      // (I + A)^-1
+                T = inv_unit_triangular_lds(At, A, ident, inv[mb], p, lane);      // (I + A)^-1
             }
-            const v4f dU0 = pc[e & 1][0].get(lane), dSi = pc[e & 1][1].get(lane);
-            cg[e & 1][0].put_t(p, dS);
-            const v4f dU = tn(w.Kt, dS, dU0);
+            const LdsMat *from = pc[e & 1];
+            LdsMat *to = cg[e & 1];
+            v4f dU = from[mb].get(lane);
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) {
+                to[eb * NM + mb].put_t(p, dS[eb]);
+                dU = tn(w.Kt[eb], dS[eb], dU);
+            }
             const v4f dY = tn(T, dU, zero);
-            cg[e & 1][1].put_t(p, dY);
-            cg[e & 1][2].put(lane, w.Kc);
+            to[NE * NM + mb].put_t(p, dY);
             v4f ndX;
 #pragma unroll
             for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
-            dS = tn(w.Kc, ndX, dS + dSi);
+#pragma unroll
+            for (int eb = 0; eb < NE; eb++) dS[eb] = tn(w.Kc[eb], ndX, dS[eb] + from[NM + eb * NM + mb].get(lane));
         };
         lds_barrier();
-        ring_loop<PF, QuadC>(nblk, load, block);
+        ring_loop<PF, Raw>(nblk, load, block);
         lds_barrier();
         lds_barrier();
         return;
     }
-    if (wave == 2) {
-        // ------------------------------------------------ R
+    if (wave <= NM + WR) {
+        // ------------------------------------------------ R of key tiles [eb0, eb0 + NEW)
+        const int j = wave - 1 - NM, eb0 = j * NEW;
+        using Raw = QuadR<NEW, NM>;
         const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
-            gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gvb(gv + seq * L * M, (uint32_t)(L * M * 4));
+            gqb(gq + seq * L * E, (uint32_t)(L * E * 4)),
+            gvb(j == 0 ? gv + seq * L * M : nullptr, j == 0 ? (uint32_t)(L * M * 4) : 0);
         const ChunkOf chunk_of(chunk);
-        auto load = [&](QuadR &w, int e) {
+        auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
-            w.Sck = cb.f4(o_dt, chunk_of(ib) * (E * M * 4));       // register r = S[c][4g + r]
-            const unsigned bs = ib * b_step, ds = ib * d_step;
+            const unsigned cs = chunk_of(ib) * (E * M * 4), ks = ib * k_step, bs = ib * b_step, ds = ib * d_step;
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                w.brow[r] = bb.f(o_br[r], bs);
-                w.Dc[r] = db.f(o_dr[r], ds);
+            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
+#pragma unroll
+            for (int b = 0; b < NEW; b++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) {
+#pragma unroll
+                for (int r = 0; r < 4; r++) w.Dc[mb][r] = db.f(o_dr[r] + 64 * mb, ds);
+#pragma unroll
+                for (int b = 0; b < NEW; b++)      // register r = S[16 eb + c][16 mb + 4g + r]
+                    w.Sck[mb][b] = cb.f4(o_dt + (16 * (eb0 + b) * M + 16 * mb) * 4, cs);
             }
         };
-        v4f St = zero;        // register r = S[c][4g + r]
-        auto block = [&](int e, const QuadR &w) {
-            const int ib = nblk - 1 - e;
-            if (chunk_of.closes(ib) || ib + 1 == nblk) St = w.Sck;      // the state after the block is checkpointed
-            v4f nU;
+        v4f St[NM][NEW];
 #pragma unroll
-            for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[r]);
+        for (int mb = 0; mb < NM; mb++)
+#pragma unroll
+            for (int b = 0; b < NEW; b++) St[mb][b] = zero;
+        auto block = [&](int e, const Raw &w) {
+            const int ib = nblk - 1 - e;
             const int s3 = third(e);
-            const v4f Kc = cg[e & 1][2].get(lane);
-            St = tn(nU, Kc, St);                                        // S0^T = S'^T - U^T K
-            v4f gQt = tn(St, pg[s3][4].get(lane), zero);
+            const float bcol = pb[s3][c];
             const v4f dPmt = pg[s3][1].get(lane);
-            const v4f dXt = pb[s3][c] * cg[e & 1][1].get(lane);
-            gQt = tn(Kc, dPmt, gQt);
-            rg[e & 1].put(lane, tn(St, -dXt, zero));
-            gqb.st4(gQt, o_dt, ib * e_step);        // register r = g_q[t0 + c][4g + r]
-            gvb.st4(dXt, o_dt, ib * d_step);        // register r = g_v[t0 + c][4g + r]
+            v4f gQt[NEW], part[NEW];
+#pragma unroll
+            for (int b = 0; b < NEW; b++) gQt[b] = tn(w.Kc[b], dPmt, zero), part[b] = zero;
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) {
+                v4f nU;
+#pragma unroll
+                for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[mb][r]);
+                const v4f Ot = pg[s3][2 + NM + mb].get(lane);
+                const v4f dXt = bcol * cg[e & 1][NE * NM + mb].get(lane);
+                gvb.st4(dXt, o_dt + 64 * mb, ib * d_step);      // register r = g_v[t0 + c][16 mb + 4g + r]
+#pragma unroll
+                for (int b = 0; b < NEW; b++) {
+                    if (chunk_of.closes(ib) || ib + 1 == nblk) St[mb][b] = w.Sck[mb][b];   // the state after the block is checkpointed
+                    St[mb][b] = tn(nU, w.Kc[b], St[mb][b]);     // S0^T = S'^T - U^T K
+                    gQt[b] = tn(St[mb][b], Ot, gQt[b]);
+                    part[b] = tn(St[mb][b], -dXt, part[b]);
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < NEW; b++) {
+                rg[e & 1][eb0 + b].put(lane, part[b]);
+                gqb.st4(gQt[b], o_ge + 64 * (eb0 + b), ib * e_step);     // register r = g_q[t0 + c][16 eb + 4g + r]
+            }
         };
         lds_barrier();
         lds_barrier();
-        ring_loop<PF, QuadR>(nblk, load, block);
+        ring_loop<PF, Raw>(nblk, load, block);
         lds_barrier();
         return;
     }
-    // ---------------------------------------------------- G (reads nothing from memory)
-    const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)), gbb(gbeta + seq * L, (uint32_t)(L * 4));
-    struct QuadG {};
-    auto load = [&](QuadG &, int) {};
-    v4f gKt = zero;           // of the block before, still without R's term
-    auto finish = [&](int e) {        // g_k of block e (as counted from the end)
-        gkb.st4(gKt + rg[e & 1].get(lane), o_dt, (nblk - 1 - e) * e_step);
+    // ---------------------------------------------------- G of key tiles [eb0, eb0 + NEW)
+    const int j = wave - 1 - NM - WR, eb0 = j * NEW;
+    using Raw = QuadG<NEW>;
+    const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
+        gbb(j == 0 ? gbeta + seq * L : nullptr, j == 0 ? (uint32_t)(L * 4) : 0);
+    auto load = [&](Raw &w, int e) {
+        const int ib = nblk - 1 - e;
+        const unsigned ks = ib * k_step, qs = ib * q_step;
+#pragma unroll
+        for (int b = 0; b < NEW; b++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
+                w.Qc[b][r] = qb.f(o_qr[r] + 64 * (eb0 + b), qs);
+            }
     };
-    auto block = [&](int e, const QuadG &) {
+    v4f gKt[NEW];             // of the block before, still without R's term
+#pragma unroll
+    for (int b = 0; b < NEW; b++) gKt[b] = zero;
+    auto finish = [&](int e) {        // g_k of block e (as counted from the end)
+#pragma unroll
+        for (int b = 0; b < NEW; b++)
+            gkb.st4(gKt[b] + rg[e & 1][eb0 + b].get(lane), o_ge + 64 * (eb0 + b), (nblk - 1 - e) * e_step);
+    };
+    auto block = [&](int e, const Raw &w) {
         const int ib = nblk - 1 - e;
         if (e > 0) finish(e - 1);
         const int s3 = third(e);
-        const v4f dSt = cg[e & 1][0].get(lane), dYt = cg[e & 1][1].get(lane), Kc = cg[e & 1][2].get(lane);
-        const v4f dPm = pg[s3][0].get(lane), Qc = pg[s3][2].get(lane), Dt = pg[s3][3].get(lane);
         const float bcol = pb[s3][c];
-        const v4f dXt = bcol * dYt, Ut = bcol * Dt;
+        const v4f dPm = pg[s3][0].get(lane);
+        v4f Mx = zero, Ut[NM];
         float gb = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], Dt[r], gb);
+        for (int mb = 0; mb < NM; mb++) {
+            const v4f dYt = cg[e & 1][NE * NM + mb].get(lane), Dt = pg[s3][2 + mb].get(lane);
+            Ut[mb] = bcol * Dt;
+#pragma unroll
+            for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], Dt[r], gb);
+            Mx = tn(bcol * dYt, Ut[mb], Mx);            // dX U^T
+        }
         {   // g_beta[t0 + c]: the four 16-lane rows hold partial sums
             float y = gb;
             swap16(gb, y);
@@ -886,19 +969,24 @@ __global__ __launch_bounds__(256) void k_delta_bwd_quad(fwp_view q, fwp_view k, 
             gb += y;
             if (g == 0) gbb.st(gb, c * 4, ib * kBlk * 4);
         }
-        const v4f Mx = tn(dXt, Ut, zero);           // dX U^T
         v4f nM;
 #pragma unroll
         for (int r = 0; r < 4; r++) nM[r] = p.lo[r] ? -Mx[r] : 0.f;
-        own[2].put_t(p, nM);
-        gKt = tn(dSt, Ut, zero);
-        gKt = tn(Qc, dPm, gKt);
+        own[j].put_t(p, nM);
+#pragma unroll
+        for (int b = 0; b < NEW; b++) {
+            gKt[b] = tn(w.Qc[b], dPm, zero);
+#pragma unroll
+            for (int mb = 0; mb < NM; mb++) gKt[b] = tn(cg[e & 1][(eb0 + b) * NM + mb].get(lane), Ut[mb], gKt[b]);
+        }
         __builtin_amdgcn_wave_barrier();
-        gKt = tn(Kc, nM + own[2].get(lane), gKt);
+        const v4f nMs = nM + own[j].get(lane);
+#pragma unroll
+        for (int b = 0; b < NEW; b++) gKt[b] = tn(w.Kc[b], nMs, gKt[b]);
     };
     lds_barrier();
     lds_barrier();
-    ring_loop<PF, QuadG>(nblk, load, block);
+    ring_loop<PF, Raw>(nblk, load, block);
     finish(nblk - 1);
     lds_barrier();
 }
@@ -966,11 +1054,16 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
                     int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     const float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
-    if (E == 16 && M == 16) {
-        hipLaunchKernelGGL(k_delta_bwd_quad<3>, dim3(N * H), dim3(256), 0, s, q, k, beta, vdiff, go, ckpt, aux, gq,
-                           gk, gv, gbeta, H, L, chunk, nchunk);
-        return (int)hipGetLastError();
+    // the shapes whose hand-over fits the 64 KB of LDS a workgroup may declare
+#define Q(ne, nm, wr, pf)                                                                                   \
+    if (E == 16 * ne && M == 16 * nm) {                                                                     \
+        static_assert(quad_lds_mats<ne, nm, wr>() * sizeof(LdsMat) + 192 <= 65536, "LDS of the hand-over"); \
+        hipLaunchKernelGGL((k_delta_bwd_quad<ne, nm, wr, pf>), dim3(N * H), dim3(64 * (1 + nm + 2 * wr)), 0, s, q, \
+                           k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);          \
+        return (int)hipGetLastError();                                                                      \
     }
+    Q(1, 1, 1, 3) Q(2, 1, 1, 3) Q(1, 2, 1, 3) Q(2, 2, 2, 3) Q(4, 1, 2, 2) Q(6, 1, 3, 2)
+#undef Q
 #define X(ne, nm)                                                                                        \
     if (E == 16 * ne && M == 16 * nm)                                                                    \
         launch_bwd<ne, nm>(q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, N * H, H, L, chunk, nchunk, s);
