@@ -688,8 +688,9 @@ constexpr int quad_lds_mats() {
     return 2 * (NM + NE * NM) + 3 * (2 + 2 * NM) + 2 * (NE * NM + NM) + 2 * NE + 2 * NM + WR;
 }
 
-template <int NE, int NM, int WR, int PF>
-__global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
+// PW = 2: P on two waves, one with the products of Pm, one with the others.
+template <int NE, int NM, int WR, int PW, int PF>
+__global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
     fwp_view q, fwp_view k, fwp_view beta, const float *__restrict__ vdiff, fwp_view go,
     const float *__restrict__ ckpt, const float *__restrict__ aux, float *__restrict__ gq,
     float *__restrict__ gk, float *__restrict__ gv, float *__restrict__ gbeta, int H, int L, int chunk,
@@ -734,52 +735,66 @@ __global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
     }
     auto third = [](int e) { return e - 3 * (int)__umulhi((unsigned)e, 0x55555556u); };   // e % 3
 
-    if (wave == 0) {
+    if (wave < PW) {
         // ------------------------------------------------ P
+        const bool with_pm = wave == 0, with_rest = wave == PW - 1;
         using Raw = QuadP<NE, NM>;
         auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
             const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step;
-            w.bcol = bb.f(o_bc, ib * b_step);
+            if (with_rest) w.bcol = bb.f(o_bc, ib * b_step);
 #pragma unroll
             for (int b = 0; b < NE; b++) {
-                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
-                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+                if (with_pm) {
+                    w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                    w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
+                }
+                if (with_rest) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
+                    for (int r = 0; r < 4; r++) w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
+                }
             }
 #pragma unroll
             for (int b = 0; b < NM; b++) {
-                w.Ot[b] = gob.f4(o_ot + 64 * b, os);
-                w.Dt[b] = db.f4(o_dt + 64 * b, ds);
+                if (with_rest) {
+                    w.Ot[b] = gob.f4(o_ot + 64 * b, os);
+                    w.Dt[b] = db.f4(o_dt + 64 * b, ds);
+                }
 #pragma unroll
                 for (int r = 0; r < 4; r++) w.Oc[b][r] = gob.f(o_or[r] + 64 * b, os);
             }
         };
         auto block = [&](int e, const Raw &w) {
-            v4f QK = zero, Z = zero;
+            if (with_pm) {
+                v4f QK = zero;
 #pragma unroll
-            for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
-            v4f Pm;
+                for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
+                v4f Pm;
 #pragma unroll
-            for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
-            const int s3 = third(e);
-            LdsMat *to = pg[s3];
+                for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
 #pragma unroll
-            for (int mb = 0; mb < NM; mb++) {
-                Z = tn(w.Ot[mb], w.bcol * w.Dt[mb], Z);         // dO U^T
-                pc[e & 1][mb].put(lane, tn(Pm, w.Oc[mb], zero));
-#pragma unroll
-                for (int eb = 0; eb < NE; eb++) pc[e & 1][NM + eb * NM + mb].put(lane, tn(w.Qc[eb], w.Oc[mb], zero));
-                to[2 + mb].put(lane, w.Dt[mb]);
-                to[2 + NM + mb].put(lane, w.Ot[mb]);
+                for (int mb = 0; mb < NM; mb++) pc[e & 1][mb].put(lane, tn(Pm, w.Oc[mb], zero));
             }
-            v4f dPm;
+            if (with_rest) {
+                v4f Z = zero;
+                const int s3 = third(e);
+                LdsMat *to = pg[s3];
 #pragma unroll
-            for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-            to[0].put(lane, dPm);
-            to[1].put_t(p, dPm);
-            if (g == 0) pb[s3][c] = w.bcol;
+                for (int mb = 0; mb < NM; mb++) {
+                    Z = tn(w.Ot[mb], w.bcol * w.Dt[mb], Z);         // dO U^T
+#pragma unroll
+                    for (int eb = 0; eb < NE; eb++)
+                        pc[e & 1][NM + eb * NM + mb].put(lane, tn(w.Qc[eb], w.Oc[mb], zero));
+                    to[2 + mb].put(lane, w.Dt[mb]);
+                    to[2 + NM + mb].put(lane, w.Ot[mb]);
+                }
+                v4f dPm;
+#pragma unroll
+                for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
+                to[0].put(lane, dPm);
+                to[1].put_t(p, dPm);
+                if (g == 0) pb[s3][c] = w.bcol;
+            }
         };
         ring_loop<PF, Raw>(nblk, load, block);
         lds_barrier();
@@ -787,9 +802,9 @@ __global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
         lds_barrier();
         return;
     }
-    if (wave <= NM) {
+    if (wave < PW + NM) {
         // ------------------------------------------------ C of value columns [16 mb, 16 mb + 16)
-        const int mb = wave - 1;
+        const int mb = wave - PW;
         using Raw = QuadC<NE>;
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
         const bool have_T = aux && aux[0] == 1.f;
@@ -853,9 +868,9 @@ __global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
         lds_barrier();
         return;
     }
-    if (wave <= NM + WR) {
+    if (wave < PW + NM + WR) {
         // ------------------------------------------------ R of key tiles [eb0, eb0 + NEW)
-        const int j = wave - 1 - NM, eb0 = j * NEW;
+        const int j = wave - PW - NM, eb0 = j * NEW;
         using Raw = QuadR<NEW, NM>;
         const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4)),
             gqb(gq + seq * L * E, (uint32_t)(L * E * 4)),
@@ -921,7 +936,7 @@ __global__ __launch_bounds__(64 * (1 + NM + 2 * WR)) void k_delta_bwd_quad(
         return;
     }
     // ---------------------------------------------------- G of key tiles [eb0, eb0 + NEW)
-    const int j = wave - 1 - NM - WR, eb0 = j * NEW;
+    const int j = wave - PW - NM - WR, eb0 = j * NEW;
     using Raw = QuadG<NEW>;
     const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
         gbb(j == 0 ? gbeta + seq * L : nullptr, j == 0 ? (uint32_t)(L * 4) : 0);
@@ -1055,14 +1070,14 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
     const int nchunk = (L + chunk - 1) / chunk;
     const float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
     // the shapes whose hand-over fits the 64 KB of LDS a workgroup may declare
-#define Q(ne, nm, wr, pf)                                                                                   \
+#define Q(ne, nm, wr, pw, pf)                                                                               \
     if (E == 16 * ne && M == 16 * nm) {                                                                     \
         static_assert(quad_lds_mats<ne, nm, wr>() * sizeof(LdsMat) + 192 <= 65536, "LDS of the hand-over"); \
-        hipLaunchKernelGGL((k_delta_bwd_quad<ne, nm, wr, pf>), dim3(N * H), dim3(64 * (1 + nm + 2 * wr)), 0, s, q, \
-                           k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);          \
+        hipLaunchKernelGGL((k_delta_bwd_quad<ne, nm, wr, pw, pf>), dim3(N * H), dim3(64 * (pw + nm + 2 * wr)), 0, \
+                           s, q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);    \
         return (int)hipGetLastError();                                                                      \
     }
-    Q(1, 1, 1, 3) Q(2, 1, 1, 3) Q(1, 2, 1, 3) Q(2, 2, 2, 3) Q(4, 1, 2, 2) Q(6, 1, 3, 2)
+    Q(1, 1, 1, 1, 3) Q(2, 1, 1, 1, 3) Q(1, 2, 1, 1, 3) Q(2, 2, 2, 2, 3) Q(4, 1, 2, 1, 2) Q(6, 1, 3, 1, 2)
 #undef Q
 #define X(ne, nm)                                                                                        \
     if (E == 16 * ne && M == 16 * nm)                                                                    \
