@@ -26,7 +26,7 @@ PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
 # HBM bytes per launch of the forward / backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch; FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by what the same counters read
 # for a 2 GiB device-to-device copy, `--copy-calibration`).
-MEASURED_TRAFFIC = {'delta': {'fwd': 84400000.0, 'bwd': 105900000.0}, 'delta_lm': {'fwd': 204700000.0, 'bwd': 270900000.0},
+MEASURED_TRAFFIC = {'delta': {'fwd': 84400000.0, 'bwd': 105900000.0}, 'delta_lm': {'fwd': 204700000.0, 'bwd': 271100000.0},
                     'sum': {'fwd': 55100000.0, 'bwd': 91500000.0}, 'rnn': {'fwd': 97500000.0, 'bwd': 127400000.0}, 'rec': {'fwd': 132100000.0, 'bwd': 150800000.0}}
 
 # name -> (B, H, T, D, algorithmic flops per token-head = c*D^2, fwd bytes, bwd bytes per token-head)
