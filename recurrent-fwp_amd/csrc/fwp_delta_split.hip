@@ -1037,8 +1037,9 @@ void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, flo
             return;
         }
     }
-    hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), false>), dim3(nseq), dim3(64 * (NM + 1)), 0, s, q,
-                       k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
+    if constexpr (NM > 1)
+        hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), false>), dim3(nseq), dim3(64 * (NM + 1)), 0, s,
+                           q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
 }
 template <int NE, int NM>
 void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go, const float *ckpt,
@@ -1079,10 +1080,11 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
     }
     Q(1, 1, 1, 1, 3) Q(2, 1, 1, 1, 3) Q(1, 2, 1, 1, 3) Q(2, 2, 2, 2, 3) Q(4, 1, 2, 1, 2) Q(6, 1, 3, 1, 2)
 #undef Q
+    // the others: adjoint and state waves
 #define X(ne, nm)                                                                                        \
     if (E == 16 * ne && M == 16 * nm)                                                                    \
         launch_bwd<ne, nm>(q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, N * H, H, L, chunk, nchunk, s);
-    FWP_SPLIT_SHAPES(X)
+    X(1, 4) X(2, 4) X(4, 2) X(4, 4) X(6, 2)
 #undef X
     return (int)hipGetLastError();
 }
