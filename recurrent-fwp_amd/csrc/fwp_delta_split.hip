@@ -3,20 +3,21 @@
 // The algebra is that of the one-wave blocked kernels (16-step blocks, fp32 MFMA, every 16x16 matrix
 // in the accumulator layout).  A sequence is one dependent chain and a wave issues one instruction
 // at a time, so a lone wave leaves the matrix pipe idle while it issues vector instructions or
-// waits for memory; there are fewer sequences than SIMDs, so the spare SIMDs take the part of a
-// block that does not lie on the chain:
+// waits for memory; while there are not many more sequences than SIMDs, other waves take the parts
+// of a block that do not lie on the chain:
 //
 // (the state is E x M, NE = E/16 by NM = M/16 tiles; E and M need not be equal here)
-//   forward, NM + 1 waves:    wave mb < NM owns the state columns [16 mb, 16 mb + 16) and does
-//       the products that need the state (X, U, O, d, S'); the last wave prepares, one block ahead,
-//       what depends on K, Q, beta only: (I + A)^-T, strict_lower(K K^T)^T, lower(Q K^T)^T.
-//   backward, NM + NE waves:  wave mb < NM ("adjoint") owns the columns of dS and walks the chain
-//       dS -> dU -> dY -> dX -> dS, stores g_v, and forms its share of lower(dO U^T) and
-//       strict_lower(dX U^T); wave NM + eb ("state"), one block behind, owns rows
-//       [16 eb, 16 eb + 16) of S, rewinds them and forms g_q, g_k for those columns, and g_beta.
+//   forward:   wave mb < NM owns the state columns [16 mb, 16 mb + 16) and does the products that
+//       need the state (X, U, S', and d); one wave prepares, four blocks ahead, what depends on K,
+//       Q, beta only ((I + A)^-T by substitution, lower(Q K^T)^T); with one or two state waves a
+//       further wave, one block behind, forms the output from the state and U handed to it.
+//   backward:  four roles, each a round behind the one before (k_delta_bwd_quad), for the shapes
+//       whose hand-over fits the LDS; for the others NM "adjoint" waves that own the columns of dS
+//       and walk the chain dS -> dU -> dY -> dX -> dS, and NE "state" waves, one block behind, that
+//       own rows [16 eb, 16 eb + 16) of S, rewind them and form g_q, g_k for those columns.
 //
-// Hand-over is through LDS, two slots used alternately, one workgroup barrier per block: every
-// wave executes the same number of barriers whatever its role.  A last block of fewer than 16 steps
+// Hand-over is through LDS in slots used in turn, one workgroup barrier per block: every wave
+// executes the same number of barriers whatever its role.  A last block of fewer than 16 steps
 // needs no code of its own: every tensor is read and written through a buffer resource of exactly
 // the sequence's size, so its missing rows read as zeros (beta = 0: nothing is written to the
 // state; zero upstream gradient) and stores to them are dropped; the loops stay straight-line.
