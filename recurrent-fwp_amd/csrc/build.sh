@@ -5,9 +5,12 @@ here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 root="$(cd "$here/../.." && pwd)"
 out="$here/../libfwp_hip.so"
 HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
-"$HIPCC" --offload-arch=gfx950 -O3 -std=c++17 -fPIC -shared \
-    -Xclang -target-feature -Xclang -packed-fp32-ops -mllvm -amdgpu-mfma-vgpr-form \
-    -I"$root/include" -I"$here" \
+common=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xclang -packed-fp32-ops
+        -I"$root/include" -I"$here")
+# the widest sum-rule kernels crash the compiler pass that -amdgpu-mfma-vgpr-form adds: compiled apart
+wide="$(mktemp -d)/fwp_sum_wide.o"
+"$HIPCC" "${common[@]}" -c "$here"/fwp_sum_wide.hip -o "$wide" "$@"
+"$HIPCC" "${common[@]}" -shared -mllvm -amdgpu-mfma-vgpr-form "$wide" \
     "$here"/fwp_api.hip "$here"/fwp_generic.hip "$here"/fwp_delta_reg.hip "$here"/fwp_delta_mfma.hip "$here"/fwp_delta_split.hip "$here"/fwp_rnn_reg.hip "$here"/fwp_lstm_reg.hip "$here"/fwp_rec_reg.hip "$here"/fwp_layer.hip \
     -o "$out" "$@"
 echo "built $out"

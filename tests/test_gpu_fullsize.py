@@ -89,6 +89,35 @@ def test_blocked_kernels_against_scan_kernels_at_full_occupancy(fwp, op, shape):
             assert torch.allclose(x, y, atol=1e-4, rtol=1e-3), (kind, i, float((x - y).abs().max()))
 
 
+def off_by_one_float(t):
+    """The same values at an address that is not a multiple of 16 bytes: the blocked and the
+    step-by-step kernels refuse such a view and the generic kernels take the call."""
+    buf = torch.empty(t.numel() + 1, device=t.device, dtype=t.dtype)
+    buf[1:].copy_(t.reshape(-1))
+    return buf[1:].view(t.shape)
+
+
+@pytest.mark.parametrize("B,H,T,E,M", [(96, 8, 100, 32, 128), (96, 8, 100, 128, 32), (64, 4, 130, 16, 128),
+                                       (33, 9, 47, 128, 16)])
+def test_sum_widest_states_blocked_against_generic_kernels(fwp, B, H, T, E, M):
+    """The fast-net layers' memories (d_head x 4 d_head and back) at hundreds of sequences: the
+    blocked kernels against the generic ones, which a misaligned q selects.  Tolerance as for the
+    oracle parity: |a - b| <= 1e-4 + 1e-3 |b|."""
+    q, k, v, _, W0, go = (dev(a) for a in delta_inputs(5, B, H, T, E, M, dtype=np.float32, w0=True))
+    res = []
+    for misaligned in (False, True):
+        W = W0.clone()
+        ts = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        if misaligned:
+            ts[0] = off_by_one_float(q).requires_grad_(True)
+            assert ts[0].data_ptr() % 16 == 4
+        out = fwp.fast_weight_sum(*ts, W)
+        res.append((out.detach(), W, *torch.autograd.grad(out, ts, go)))
+    for i, (x, y) in enumerate(zip(*res)):
+        assert torch.isfinite(x).all()
+        assert torch.allclose(x, y, atol=1e-4, rtol=1e-3), (i, float((x - y).abs().max()))
+
+
 @pytest.mark.parametrize("E,M", [(64, 32), (96, 16), (16, 64), (64, 64)])
 def test_delta_rectangular_states_at_full_occupancy(fwp, E, M):
     """1024 sequences (several waves on every SIMD) of the rectangular state shapes: a split on a

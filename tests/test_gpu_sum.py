@@ -42,6 +42,10 @@ SHAPES = [
     (1, 2, 1, 32, 32, True),
     (2, 2, 40, 32, 128, True),    # fast-net layers: d_head x fast_ff_d_head and back
     (2, 2, 40, 128, 32, False),
+    (1, 2, 70, 16, 128, True),
+    (2, 1, 33, 128, 16, True),
+    (1, 2, 200, 32, 128, True),   # longer than one chunk of the state checkpoints
+    (1, 1, 150, 128, 32, True),
     (1, 1, 20, 5, 3, True),
     # rectangular and larger states on the matrix cores (feature maps that widen the keys; d_head 64)
     (2, 2, 40, 96, 16, True),
