@@ -12,7 +12,7 @@
 namespace fwp {
 namespace {
 
-__device__ __forceinline__ float sigmoidf_fast(float x) { return __fdividef(1.f, 1.f + __expf(-x)); }
+__device__ __forceinline__ float sigmoidf_fast(float x) { return fast_div(1.f, 1.f + __expf(-x)); }
 
 template <int D>
 constexpr int lstm_tile() { return D == 32 ? 8 : 16; }
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_fwd_reg(LstmGates g, float
     auto compute = [&](const LstmFwdOps<D> &o, int tt) {
         const float mx = across_groups<S>(hcur, OpMax());
         const float e = __expf(hcur - mx);
-        const float s_m = __fdividef(e, across_groups<S>(e, OpSum()));
+        const float s_m = fast_div(e, across_groups<S>(e, OpSum()));
         float s[NP];
         to_periodic<D>(s_m, s, lane);
         float d[3], pre[3];
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_bwd_reg(
             float4 &r = ps.r[x];
             const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
             r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
-            const float inv = 1.f / row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum());
+            const float inv = fast_div(1.f, row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum()));
             r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
         }
         ps.commit(ss[buf], lane);

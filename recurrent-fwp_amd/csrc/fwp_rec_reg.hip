@@ -13,10 +13,10 @@ namespace fwp {
 namespace {
 
 __device__ __forceinline__ float fast_tanh(float x) {
-    return 1.f - __fdividef(2.f, 1.f + __expf(2.f * x));
+    return 1.f - fast_div(2.f, 1.f + __expf(2.f * x));
 }
 __device__ __forceinline__ float fast_sigmoid(float x) {
-    return __fdividef(1.f, 1.f + __expf(-x));
+    return fast_div(1.f, 1.f + __expf(-x));
 }
 
 // ------------------------------------------------------------------ forward
@@ -127,8 +127,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
         const float b = fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum()));
         const float eq = __expf(qa - across_groups<S>(qa, OpMax()));
         const float ek = __expf(ka - across_groups<S>(ka, OpMax()));
-        const float q_m = __fdividef(eq, across_groups<S>(eq, OpSum()));
-        const float k_m = __fdividef(ek, across_groups<S>(ek, OpSum()));
+        const float q_m = fast_div(eq, across_groups<S>(eq, OpSum()));
+        const float k_m = fast_div(ek, across_groups<S>(ek, OpSum()));
         to_periodic<D>(k_m, kp, lane);
         to_periodic<D>(q_m, qp, lane);
         const float d = va - group_sum<S>(dot_rot<D>(Wc, kp));

@@ -55,11 +55,32 @@ __device__ __forceinline__ float fmac_ror(float acc, float x, float y) {
     }
 }
 
-template <int S, int... J>
-__device__ __forceinline__ float dot_rot1(const float *w, float x, float acc,
-                                          std::integer_sequence<int, J...>) {
-    ((acc = fmac_ror<S * J>(acc, x, w[J])), ...);
-    return acc;
+// ror(x, ROT) * y; the same restriction on x as for fmac_ror.
+template <int ROT>
+__device__ __forceinline__ float mul_ror(float x, float y) {
+    if constexpr (ROT == 0) {
+        return x * y;
+    } else {
+        float r;
+        asm("v_mul_f32_dpp %0, %1, %2 row_ror:%3 row_mask:0xf bank_mask:0xf bound_ctrl:1"
+            : "=v"(r)
+            : "v"(x), "v"(y), "n"(ROT));
+        return r;
+    }
+}
+
+// The products of a dot go to two accumulators in turn and are added up at the end: the wave
+// issues in order, and an instruction that needs the result of the one just before it waits about
+// as long again as an independent one takes to issue.  START: acc[0] comes with a value; the other
+// accumulators start from their first product.
+template <int D, bool START, int... JJ>
+__device__ __forceinline__ void dot_rot1(const float *w, const float *x, float (&acc)[2],
+                                         std::integer_sequence<int, JJ...>) {
+    using G = Geo<D>;
+    ((acc[JJ % 2] = JJ < 2 && !(START && JJ == 0)
+                        ? mul_ror<G::S * (JJ % G::NR)>(x[JJ / G::NR], w[JJ])
+                        : fmac_ror<G::S * (JJ % G::NR)>(acc[JJ % 2], x[JJ / G::NR], w[JJ])),
+     ...);
 }
 template <int S, bool NEG, int... J>
 __device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
@@ -69,13 +90,18 @@ __device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
 
 // sum_jj w[jj] * x[index(jj)]  for a periodic vector x[NP]
 template <int D>
+__device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP]) {
+    float acc[2];
+    dot_rot1<D, false>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
+    return acc[0] + acc[1];
+}
+// the same, added to acc0
+template <int D>
 __device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
-                                         float acc = 0.f) {
-    using G = Geo<D>;
-#pragma unroll
-    for (int p = 0; p < G::NP; p++)
-        acc = dot_rot1<G::S>(&w[p * G::NR], x[p], acc, std::make_integer_sequence<int, G::NR>{});
-    return acc;
+                                         float acc0) {
+    float acc[2] = {acc0, 0.f};
+    dot_rot1<D, true>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
+    return acc[0] + acc[1];
 }
 // w[jj] += x[index(jj)] * y   (NEG: -= )
 template <int D, bool NEG = false>

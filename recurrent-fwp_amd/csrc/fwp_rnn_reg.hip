@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
         // s = softmax(h_{t-1}); independent of the delta write below, which overlaps its latency
         const float mx = across_groups<S>(hcur, OpMax());
         const float e = __expf(hcur - mx);
-        const float s_m = __fdividef(e, across_groups<S>(e, OpSum()));
+        const float s_m = fast_div(e, across_groups<S>(e, OpSum()));
         float s[NP];
         to_periodic<D>(s_m, s, lane);
         const float d = o.v - group_sum<S>(dot_rot<D>(Wc, o.k));
@@ -236,7 +236,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_bwd_reg(
             float4 &r = ps.r[x];
             const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
             r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
-            const float inv = 1.f / row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum());
+            const float inv = fast_div(1.f, row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum()));
             r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
         }
         ps.commit(ss[buf], lane);

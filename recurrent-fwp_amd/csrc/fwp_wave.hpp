@@ -53,9 +53,19 @@ __device__ __forceinline__ float pinned(float x) {
 struct OpSum {
     __device__ __forceinline__ float operator()(float a, float b) const { return a + b; }
 };
+// The instruction itself: fmaxf() makes the compiler quiet each operand first (one more v_max_f32
+// apiece), which nothing here needs.
 struct OpMax {
-    __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); }
+    __device__ __forceinline__ float operator()(float a, float b) const {
+        float r;
+        asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+        return r;
+    }
 };
+
+// a / b for b well inside the normal range, to 1 ulp of 1 / b (a / b and __fdividef(a, b) are both
+// compiled into the full eleven-instruction division).
+__device__ __forceinline__ float fast_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
 
 // All-reduce over the D groups of a wave for a value that is already uniform
 // inside each group of S lanes (S*D = 64).  Every lane gets the result.
