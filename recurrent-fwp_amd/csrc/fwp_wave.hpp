@@ -21,6 +21,8 @@ constexpr int kQuadXor1 = 0xB1;  // quad_perm:[1,0,3,2]
 constexpr int kQuadXor2 = 0x4E;  // quad_perm:[2,3,0,1]
 constexpr int kRowRor4 = 0x124;
 constexpr int kRowRor8 = 0x128;
+constexpr int kRowBcast15 = 0x142;  // lane 15 of each row to every lane of the next row
+constexpr int kRowBcast31 = 0x143;  // lane 31 to every lane of rows 2 and 3
 
 // Sum over the S adjacent lanes of a group; every lane of the group gets the sum.
 template <int S>
@@ -68,7 +70,12 @@ struct OpMax {
 __device__ __forceinline__ float fast_div(float a, float b) { return a * __builtin_amdgcn_rcpf(b); }
 
 // All-reduce over the D groups of a wave for a value that is already uniform
-// inside each group of S lanes (S*D = 64).  Every lane gets the result.
+// inside each group of S lanes (S*D = 64).  Every lane gets the result (it is wave-uniform and
+// ends up in a scalar register).  After the stages inside the 16-lane rows every lane holds its
+// row's result r0..r3; row_bcast:15 brings the last lane of the row before (rows 1 and 3 then
+// hold r0 op r1 and r2 op r3), row_bcast:31 the last lane of the first half (the last row then
+// holds all four), and the last lane is read out: five instructions, where two row swaps take
+// twelve issue slots with their wait states.
 template <int S, typename Op>
 __device__ __forceinline__ float across_groups(float x, Op op) {
     static_assert(S == 1 || S == 2 || S == 4, "group of 1, 2 or 4 lanes");
@@ -76,12 +83,9 @@ __device__ __forceinline__ float across_groups(float x, Op op) {
     if constexpr (S <= 2) x = op(x, dpp<kQuadXor2>(x));
     x = op(x, dpp<kRowRor4>(x));
     x = op(x, dpp<kRowRor8>(x));
-    float y = x;
-    swap16(x, y);
-    x = op(x, y);
-    y = x;
-    swap32(x, y);
-    return op(x, y);
+    x = op(x, dpp<kRowBcast15>(x));
+    x = op(x, dpp<kRowBcast31>(x));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
 
 }  // namespace fwp
