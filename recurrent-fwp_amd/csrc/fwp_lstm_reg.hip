@@ -125,15 +125,17 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_fwd_reg(LstmGates g, float
     auto compute = [&](const LstmFwdOps<D> &o, int tt) {
         const float mx = across_groups<S>(hcur, OpMax());
         const float e = __expf(hcur - mx);
-        const float s_m = fast_div(e, across_groups<S>(e, OpSum()));
+        // the reads below use e and are scaled by 1 / sum(e) afterwards: the wave-wide sum then runs
+        // beside them instead of ahead of them on the sequential path
         float s[NP];
-        to_periodic<D>(s_m, s, lane);
+        to_periodic<D>(e, s, lane);
+        const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));
         float d[3], pre[3];
 #pragma unroll
         for (int a = 0; a < 3; a++) {
             d[a] = o.v[a] - group_sum<S>(dot_rot<D>(Wc[a], o.k[a]));
             rank1_rot<D>(Wc[a], o.k[a], o.b[a] * d[a]);
-            pre[a] = group_sum<S>(dot_rot<D>(Wc[a], s)) + o.z[a];
+            pre[a] = fmaf(group_sum<S>(dot_rot<D>(Wc[a], s)), rsum, o.z[a]);
         }
         const float gi = sigmoidf_fast(pre[0]), go = sigmoidf_fast(pre[2]);
         ccur = fmaf(gi, pre[1] - ccur, ccur);          // i u + (1 - i) c

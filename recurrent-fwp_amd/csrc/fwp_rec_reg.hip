@@ -127,15 +127,18 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
         const float b = fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum()));
         const float eq = __expf(qa - across_groups<S>(qa, OpMax()));
         const float ek = __expf(ka - across_groups<S>(ka, OpMax()));
-        const float q_m = fast_div(eq, across_groups<S>(eq, OpSum()));
-        const float k_m = fast_div(ek, across_groups<S>(ek, OpSum()));
-        to_periodic<D>(k_m, kp, lane);
-        to_periodic<D>(q_m, qp, lane);
-        const float d = va - group_sum<S>(dot_rot<D>(Wc, kp));
-        rank1_rot<D>(Wc, kp, b * d);
-        hcur = group_sum<S>(dot_rot<D>(Wc, qp));
+        // The softmaxes are eq / sum(eq) and ek / sum(ek); the state is read and written with eq and
+        // ek and the results are scaled afterwards: the wave-wide sums then run beside the reads
+        // instead of ahead of them on the sequential path.
+        to_periodic<D>(ek, kp, lane);
+        to_periodic<D>(eq, qp, lane);
+        const float rk = fast_div(1.f, across_groups<S>(ek, OpSum()));
+        const float rq = fast_div(1.f, across_groups<S>(eq, OpSum()));
+        const float d = fmaf(-group_sum<S>(dot_rot<D>(Wc, kp)), rk, va);
+        rank1_rot<D>(Wc, kp, b * d * rk);
+        hcur = group_sum<S>(dot_rot<D>(Wc, qp)) * rq;
         hcur = pinned(hcur);
-        const float o_d = pinned(d), o_q = pinned(q_m), o_k = pinned(k_m);
+        const float o_d = pinned(d), o_q = pinned(eq * rq), o_k = pinned(ek * rk);
         if constexpr (S == 4) {
             stage1[tt * D] = sl == 0 ? hcur : (sl == 1 ? o_d : (sl == 2 ? o_q : o_k));
         } else {

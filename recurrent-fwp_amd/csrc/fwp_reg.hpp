@@ -69,18 +69,27 @@ __device__ __forceinline__ float mul_ror(float x, float y) {
     }
 }
 
-// The products of a dot go to two accumulators in turn and are added up at the end: the wave
-// issues in order, and an instruction that needs the result of the one just before it waits about
-// as long again as an independent one takes to issue.  START: acc[0] comes with a value; the other
-// accumulators start from their first product.
-template <int D, bool START, int... JJ>
-__device__ __forceinline__ void dot_rot1(const float *w, const float *x, float (&acc)[2],
+// The products of a dot go to NA accumulators in turn and are added up at the end: the wave issues
+// in order, and an instruction that needs the result of the one just before it waits about as long
+// again as an independent one takes to issue; between two of these asm statements of which the
+// second reads what the first wrote, the compiler also wants two other instructions or puts wait
+// states there (it cannot tell which operand the DPP modifier applies to).  START: acc[0] comes with
+// a value; the other accumulators start from their first product.
+template <int D, int NA, bool START, int... JJ>
+__device__ __forceinline__ void dot_rot1(const float *w, const float *x, float (&acc)[NA],
                                          std::integer_sequence<int, JJ...>) {
     using G = Geo<D>;
-    ((acc[JJ % 2] = JJ < 2 && !(START && JJ == 0)
-                        ? mul_ror<G::S * (JJ % G::NR)>(x[JJ / G::NR], w[JJ])
-                        : fmac_ror<G::S * (JJ % G::NR)>(acc[JJ % 2], x[JJ / G::NR], w[JJ])),
+    ((acc[JJ % NA] = JJ < NA && !(START && JJ == 0)
+                         ? mul_ror<G::S * (JJ % G::NR)>(x[JJ / G::NR], w[JJ])
+                         : fmac_ror<G::S * (JJ % G::NR)>(acc[JJ % NA], x[JJ / G::NR], w[JJ])),
      ...);
+}
+template <int R>
+constexpr int kDotAccs = R >= 8 ? 3 : 2;
+template <int NA>
+__device__ __forceinline__ float sum_accs(const float (&acc)[NA]) {
+    if constexpr (NA == 3) return (acc[0] + acc[1]) + acc[2];
+    else return acc[0] + acc[1];
 }
 template <int S, bool NEG, int... J>
 __device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
@@ -91,17 +100,19 @@ __device__ __forceinline__ void rank1_rot1(float *w, float x, float y,
 // sum_jj w[jj] * x[index(jj)]  for a periodic vector x[NP]
 template <int D>
 __device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP]) {
-    float acc[2];
-    dot_rot1<D, false>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
-    return acc[0] + acc[1];
+    constexpr int NA = kDotAccs<Geo<D>::R>;
+    float acc[NA];
+    dot_rot1<D, NA, false>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
+    return sum_accs(acc);
 }
 // the same, added to acc0
 template <int D>
 __device__ __forceinline__ float dot_rot(const float (&w)[Geo<D>::R], const float (&x)[Geo<D>::NP],
                                          float acc0) {
-    float acc[2] = {acc0, 0.f};
-    dot_rot1<D, true>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
-    return acc[0] + acc[1];
+    constexpr int NA = kDotAccs<Geo<D>::R>;
+    float acc[NA] = {acc0};
+    dot_rot1<D, NA, true>(w, x, acc, std::make_integer_sequence<int, Geo<D>::R>{});
+    return sum_accs(acc);
 }
 // w[jj] += x[index(jj)] * y   (NEG: -= )
 template <int D, bool NEG = false>

@@ -93,17 +93,20 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
         o.b = sb[buf][tt];
     };
     auto compute = [&](const RnnFwdOps<D> &o, float *o_ptr) {
-        // s = softmax(h_{t-1}); independent of the delta write below, which overlaps its latency
+        // s = softmax(h_{t-1}) = e / sum(e); independent of the delta write below, which overlaps
+        // its latency.  The read is done with e and scaled afterwards: the wave-wide sum then runs
+        // beside the read instead of ahead of it on the sequential path.
         const float mx = across_groups<S>(hcur, OpMax());
         const float e = __expf(hcur - mx);
-        const float s_m = fast_div(e, across_groups<S>(e, OpSum()));
         float s[NP];
-        to_periodic<D>(s_m, s, lane);
+        to_periodic<D>(e, s, lane);
+        const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));
         const float d = o.v - group_sum<S>(dot_rot<D>(Wc, o.k));
         rank1_rot<D>(Wc, o.k, o.b * d);
-        hcur = group_sum<S>(dot_rot<D>(Wc, s)) + o.z;
+        hcur = fmaf(group_sum<S>(dot_rot<D>(Wc, s)), rsum, o.z);
         hcur = pinned(hcur);
-        *o_ptr = store_d ? pinned(d) : hcur;
+        const float o_d = pinned(d);     // outside the select, which is then one v_cndmask and no branch
+        *o_ptr = store_d ? o_d : hcur;
     };
 
     const int ntile = (L + kTile - 1) / kTile;
