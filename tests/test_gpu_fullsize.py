@@ -194,6 +194,29 @@ def test_rnn_full_size_properties(fwp):
     assert torch.equal(g1[0][:, :, -1], go[:, :, -1])      # grad_z of the last step is the upstream gradient
 
 
+@pytest.mark.parametrize("D,T", [(32, 100), (16, 70)])
+def test_rnn_backward_one_and_two_waves_per_sequence(fwp, D, T):
+    """The backward pass of the Delta RNN puts two waves on a sequence up to 512 sequences and one
+    from there to 1024: 1024 sequences in one call against the same sequences in two calls of
+    512 and in calls of 511 (an odd count leaves a workgroup with one sequence) and 513.
+    Tolerance: |a - b| <= 1e-4 + 1e-3 |b|."""
+    z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(7, 128, 8, T, D, dtype=np.float32, w0=True))
+
+    def grads(sl):
+        fn = lambda t: fwp.fast_rnn_v2(t[0], t[1], t[2], W0.reshape(-1, 1, D, D)[sl].clone(), t[3],
+                                       h0.reshape(-1, 1, 1, D)[sl].clone())
+        flat = [x.reshape(-1, 1, T, x.shape[-1])[sl] for x in (z, k, v, beta)]
+        return grads_of(fn, flat, go.reshape(-1, 1, T, D)[sl])[1]
+
+    whole = grads(slice(0, 1024))
+    for cut in (512, 511):
+        parts = [grads(slice(0, cut)), grads(slice(cut, 1024))]
+        for i, w in enumerate(whole):
+            got = torch.cat([parts[0][i], parts[1][i]], 0)
+            assert torch.isfinite(got).all()
+            assert torch.allclose(got, w, atol=1e-4, rtol=1e-3), (cut, i, float((got - w).abs().max()))
+
+
 def test_rec_full_size_properties(fwp):
     *x, go = (dev(a) for a in rec_inputs(2, 64, 8, 256, 32, dtype=np.float32))
     qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0 = x
