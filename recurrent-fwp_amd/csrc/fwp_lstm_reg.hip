@@ -464,7 +464,357 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_bwd_reg(
     flush(0, min(TL, L));
 }
 
+// ------------------------------------------- backward, four waves per sequence
+//
+// One wave cannot issue the backward step's instructions any faster, so the step is divided: wave C
+// keeps what is sequential (the cell, the gradient of h through the three states and the softmax,
+// with it grad_z) and a copy of the three states; one wave per gate, one tile behind, takes that
+// gate's g = grad_z from LDS, keeps G = dL/dW in both layouts and its own copy of W, and computes
+// grad_v, grad_beta and grad_k.  C also loads the tiles the others need (k, vdiff, beta and the
+// softmax of the delayed output) into a ring of three slots: it fills the slot of tile it - 1 while
+// it works on tile it and the gate waves on tile it + 1.  One workgroup barrier per tile.
+template <int D>
+struct LstmQuadLds {
+    static constexpr int TL = lstm_tile<D>();
+    float k[3][3][TL * D], d[3][3][TL * D], s[3][TL * D];   // [slot][gate]
+    float b[3][3][16];
+    float go[2][TL * D], co[4][2][TL * D];
+    float g[2][3][TL * D];                                   // C -> gate waves, by tile parity
+    float pd[3][TL * D], gk[3][TL * D], gv[3][TL * D];       // per gate wave
+};
+
+template <int D>
+struct LstmBwdOpsC {
+    float u[3][Geo<D>::NP], k_i[3];
+    float s_i, go_i, po, pa, pb, pi;
+};
+template <int D>
+struct LstmBwdOpsG {
+    float gp[Geo<D>::NP], s[Geo<D>::NP], k[Geo<D>::NP], u[Geo<D>::NP];
+    float ga_i, s_i, k_i, d_i, b;
+};
+
+template <int D>
+__device__ __forceinline__ void lstm_bwd_quad_c(LstmQuadLds<D> &M, const LstmGates &g,
+                                                const float *__restrict__ vdiff,
+                                                const float *__restrict__ gates,
+                                                const float *__restrict__ out,
+                                                const float *__restrict__ cell,
+                                                const float *__restrict__ h_init,
+                                                const float *__restrict__ c_init, fwp_view go,
+                                                const float *__restrict__ ckpt, float *__restrict__ gz,
+                                                int N, int H, int L, int chunk, int nchunk, int64_t seq,
+                                                int lane) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    using Tile = TileRegs<D, TL>;
+    const int i = lane / S, sl = lane % S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+    const int64_t base = seq * L * D;
+
+    float Wr[3][R];   // per gate: Wr[jj] = W[i][reg_index(jj)]
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wr[a][jj] = 0.f;
+    float dh_i = 0.f, dc_i = 0.f;   // gradients carried to the previous output and cell, entry i
+
+    Tile pk[3], pd[3], pgo, ps, pco[4];
+    float pb[3] = {0.f, 0.f, 0.f};
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane[3], *bb[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        klane[a] = row(g.k[a], n, h, 0) + lrow * g.k[a].sL + 4 * lc4;
+        bb[a] = row(g.beta[a], n, h, 0);
+    }
+    const float *golane = row(go, n, h, 0) + lrow * go.sL + 4 * lc4;
+    const int64_t lane_off = (int64_t)lrow * D + 4 * lc4;     // into the contiguous saved tensors
+    auto fetch = [&](int t0) {
+        const bool full = t0 + TL <= L;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float *dl = vdiff + a * gate_stride + base + lane_off;
+            if (full) {
+                pk[a].template fetch<true>(klane[a], g.k[a].sL, t0, L, lane);
+                pd[a].template fetch<true>(dl, D, t0, L, lane);
+            } else {
+                pk[a].template fetch<false>(klane[a], g.k[a].sL, t0, L, lane);
+                pd[a].template fetch<false>(dl, D, t0, L, lane);
+            }
+            pb[a] = bb[a][(int64_t)min(t0 + per % TL, L - 1) * g.beta[a].sL];
+        }
+        if (full) pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+        else pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+        // gates, cell, delayed cell and delayed output of the tile's rows -> coefficients
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            const int t = t0 + lrow + Tile::kRowsPerLoad * x;
+            const int64_t r = (int64_t)min(t, L - 1) * D + 4 * lc4;
+            const float4 gi = *reinterpret_cast<const float4 *>(gates + base + r);
+            const float4 gu = *reinterpret_cast<const float4 *>(gates + gate_stride + base + r);
+            const float4 go_ = *reinterpret_cast<const float4 *>(gates + 2 * gate_stride + base + r);
+            const float4 ct = *reinterpret_cast<const float4 *>(cell + base + r);
+            // row t of a delayed tensor is row t-1, or the initial state for t = 0
+            const int64_t rp = (int64_t)(min(t, L) - 1) * D + 4 * lc4;
+            const float4 cp = *reinterpret_cast<const float4 *>(t == 0 ? c_init + seq * D + 4 * lc4
+                                                                       : cell + base + rp);
+            ps.r[x] = *reinterpret_cast<const float4 *>(t == 0 ? h_init + seq * D + 4 * lc4
+                                                                : out + base + rp);
+            pco[0].r[x] = go_;
+            pco[1].r[x] = make_float4(ct.x * go_.x * (1.f - go_.x), ct.y * go_.y * (1.f - go_.y),
+                                      ct.z * go_.z * (1.f - go_.z), ct.w * go_.w * (1.f - go_.w));
+            pco[2].r[x] = make_float4((gu.x - cp.x) * gi.x * (1.f - gi.x), (gu.y - cp.y) * gi.y * (1.f - gi.y),
+                                      (gu.z - cp.z) * gi.z * (1.f - gi.z), (gu.w - cp.w) * gi.w * (1.f - gi.w));
+            pco[3].r[x] = gi;
+        }
+    };
+    auto commit = [&](int it) {
+        const int slot = it % 3, buf = it & 1;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            pk[a].commit(M.k[slot][a], lane);
+            pd[a].commit(M.d[slot][a], lane);
+            M.b[slot][a][per % TL] = pb[a];
+        }
+        pgo.commit(M.go[buf], lane);
+#pragma unroll
+        for (int x = 0; x < 4; x++) pco[x].commit(M.co[x][buf], lane);
+        // softmax of each row of the delayed output, off the sequential path
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            float4 &r = ps.r[x];
+            const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
+            r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
+            const float inv = fast_div(1.f, row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum()));
+            r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
+        }
+        ps.commit(M.s[slot], lane);
+    };
+    auto load_state = [&](int c) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float *src = ckpt + a * ckpt_stride + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[a][jj] = src[reg_index<D>(lane, jj)];
+        }
+    };
+    auto load_ops = [&](LstmBwdOpsC<D> &o, int it, int tt) {
+        const int slot = it % 3, buf = it & 1, off = tt * D;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float b = M.b[slot][a][tt];
+#pragma unroll
+            for (int p = 0; p < NP; p++) o.u[a][p] = b * M.d[slot][a][off + 16 * p + per];     // u = beta d
+            o.k_i[a] = M.k[slot][a][off + i];
+        }
+        o.s_i = M.s[slot][off + i];
+        o.go_i = M.go[buf][off + i];
+        o.po = M.co[0][buf][off + i];
+        o.pa = M.co[1][buf][off + i];
+        o.pb = M.co[2][buf][off + i];
+        o.pi = M.co[3][buf][off + i];
+    };
+    auto compute = [&](const LstmBwdOpsC<D> &o, int it, int tt) {
+        // cell: h = o c, c = i u + (1 - i) c_prev
+        const float gh = dh_i + o.go_i;
+        const float gc = fmaf(gh, o.po, dc_i);
+        const float ga[3] = {gc * o.pb, gc * o.pi, gh * o.pa};     // gradients of the pre-activations = grad_z
+        dc_i = gc * (1.f - o.pi);
+        float ds_part = 0.f;
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            float gp[NP];
+            to_periodic<D>(ga[a], gp, lane);
+            ds_part = dot_rot<D>(Wr[a], gp, ds_part);              // (W_t ga)[i], summed over the gates
+            rank1_rot<D, true>(Wr[a], o.u[a], o.k_i[a]);           // W_{t-1}
+        }
+        // gradient of s = softmax(h_{t-1}) back to h_{t-1}
+        const float ds_i = group_sum<S>(ds_part);
+        const float dot = across_groups<S>(ds_i * o.s_i, OpSum());
+        dh_i = o.s_i * (ds_i - dot);
+        const float o0 = pinned(ga[0]), o1 = pinned(ga[1]), o2 = pinned(ga[2]);
+        float *h0 = M.g[it & 1][0] + tt * D + i, *h1 = M.g[it & 1][1] + tt * D + i,
+              *h2 = M.g[it & 1][2] + tt * D + i;
+        if constexpr (S == 4) {
+            *(sl == 0 ? h0 : (sl == 1 ? h1 : h2)) = sl == 0 ? o0 : (sl == 1 ? o1 : o2);
+        } else {
+            *(sl == 0 ? h0 : h1) = sl == 0 ? o0 : o1;
+            *h2 = o2;
+        }
+    };
+    auto flush = [&](int it) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) flush_tile<D, TL>(M.g[it & 1][a], gz + a * gate_stride + base, it * TL, L, lane);
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    fetch((ntile - 1) * TL);
+    commit(ntile - 1);
+    if (ntile > 1) fetch((ntile - 2) * TL);
+    __syncthreads();
+
+    for (int it = ntile - 1; it >= 0; it--) {
+        const int t0 = it * TL;
+        const int nst = min(TL, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) load_state((t_end - 1) / chunk);  // first tile (in reverse) of a chunk
+        if (it >= 1) commit(it - 1);
+        if (it + 1 < ntile) flush(it + 1);
+        if (it >= 2) fetch(t0 - 2 * TL);
+        if (nst == TL) {
+            LstmBwdOpsC<D> ring[2];
+            load_ops(ring[(TL - 1) & 1], it, TL - 1);
+#pragma unroll
+            for (int tt = TL - 1; tt >= 0; tt--) {
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], it, tt - 1);
+                compute(ring[tt & 1], it, tt);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                LstmBwdOpsC<D> o;
+                load_ops(o, it, tt);
+                compute(o, it, tt);
+            }
+        }
+        __syncthreads();
+    }
+    flush(0);
+}
+
+template <int D>
+__device__ __forceinline__ void lstm_bwd_quad_g(LstmQuadLds<D> &M, int a, const float *__restrict__ ckpt,
+                                                float *__restrict__ gk, float *__restrict__ gv,
+                                                float *__restrict__ gbeta, int N, int H, int L, int chunk,
+                                                int nchunk, int64_t seq, int lane) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    const int i = lane / S, sl = lane % S, per = lane % 16;
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t beta_stride = (int64_t)N * H * L;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+    const int64_t base = seq * L * D;
+    // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
+    float Wr[R], Gr[R], Gc[R];
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Gr[jj] = Gc[jj] = Wr[jj] = 0.f;
+    auto load_state = [&](int c) {
+        const float *src = ckpt + a * ckpt_stride + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wr[jj] = src[reg_index<D>(lane, jj)];
+    };
+    float *spd = M.pd[a], *sgk = M.gk[a], *sgv = M.gv[a];
+    auto load_ops = [&](LstmBwdOpsG<D> &o, int ty, int tt) {
+        const int slot = ty % 3, buf = ty & 1, off = tt * D;
+        o.b = M.b[slot][a][tt];
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.gp[p] = M.g[buf][a][off + 16 * p + per];
+            o.s[p] = M.s[slot][off + 16 * p + per];
+            o.k[p] = M.k[slot][a][off + 16 * p + per];
+            o.u[p] = o.b * M.d[slot][a][off + 16 * p + per];     // u = beta d
+        }
+        o.ga_i = M.g[buf][a][off + i];
+        o.s_i = M.s[slot][off + i];
+        o.k_i = M.k[slot][a][off + i];
+        o.d_i = M.d[slot][a][off + i];
+    };
+    auto compute = [&](const LstmBwdOpsG<D> &o, int tt) {
+        float ap[NP];
+        // G' = G + s (x) ga (both layouts);  r = G'^T k
+        rank1_rot<D>(Gc, o.s, o.ga_i);
+        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        const float gv_i = o.b * r_i;
+        const float a_i = -gv_i;                               // gradient w.r.t. v_old
+        to_periodic<D>(a_i, ap, lane);
+        spd[tt * D + i] = r_i * o.d_i;
+        rank1_rot<D>(Gr, o.gp, o.s_i);
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                    // W_{t-1}
+        rank1_rot<D>(Gc, o.k, a_i);
+        float gk_i = dot_rot<D>(Gr, o.u);                      // G' u + W_{t-1} a
+        gk_i = group_sum<S>(dot_rot<D>(Wr, ap, gk_i));
+        rank1_rot<D>(Gr, ap, o.k_i);
+        const float o_k = pinned(gk_i), o_v = pinned(gv_i);
+        *(sl == 0 ? sgk + tt * D + i : sgv + tt * D + i) = sl == 0 ? o_k : o_v;
+    };
+    auto flush = [&](int ty) {
+        const int t0 = ty * TL, nst = min(TL, L - t0);
+        flush_tile<D, TL>(sgk, gk + a * gate_stride + base, t0, L, lane);
+        flush_tile<D, TL>(sgv, gv + a * gate_stride + base, t0, L, lane);
+        // gbeta of the tile's steps: sums of spd[tt][:] over the D entries, four lanes per step
+        const int tt = lane / 4, part = lane % 4;
+        if (tt < TL) {
+            float acc = 0.f;
+#pragma unroll
+            for (int j = 0; j < D / 4; j += 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(&spd[tt * D + part * (D / 4) + j]);
+                acc += (x.x + x.y) + (x.z + x.w);
+            }
+            acc = group_sum<4>(acc);
+            if (tt < nst) gbeta[a * beta_stride + seq * L + t0 + tt] = acc;
+        }
+    };
+    auto run_tile = [&](int ty) {
+        const int t0 = ty * TL;
+        const int nst = min(TL, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) load_state((t_end - 1) / chunk);
+        if (ty + 1 < (L + TL - 1) / TL) flush(ty + 1);
+        if (nst == TL) {
+            LstmBwdOpsG<D> ring[2];
+            load_ops(ring[(TL - 1) & 1], ty, TL - 1);
+#pragma unroll
+            for (int tt = TL - 1; tt >= 0; tt--) {
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], ty, tt - 1);
+                compute(ring[tt & 1], tt);
+            }
+        } else {
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                LstmBwdOpsG<D> o;
+                load_ops(o, ty, tt);
+                compute(o, tt);
+            }
+        }
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    __syncthreads();
+    for (int it = ntile - 1; it >= 0; it--) {     // the tile C works on; this wave is one behind
+        if (it + 1 < ntile) run_tile(it + 1);
+        __syncthreads();
+    }
+    run_tile(0);
+    flush(0);
+}
+
+template <int D>
+__global__ __launch_bounds__(kWave * 4) void k_lstm_bwd_quad(
+    LstmGates g, const float *__restrict__ vdiff, const float *__restrict__ gates,
+    const float *__restrict__ out, const float *__restrict__ cell, const float *__restrict__ h_init,
+    const float *__restrict__ c_init, fwp_view go, const float *__restrict__ ckpt,
+    float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv, float *__restrict__ gbeta,
+    int N, int H, int L, int chunk, int nchunk) {
+    __shared__ __align__(16) LstmQuadLds<D> M;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int64_t seq = blockIdx.x;
+    if (wave == 0)
+        lstm_bwd_quad_c<D>(M, g, vdiff, gates, out, cell, h_init, c_init, go, ckpt, gz, N, H, L, chunk, nchunk,
+                           seq, lane);
+    else
+        lstm_bwd_quad_g<D>(M, wave - 1, ckpt, gk, gv, gbeta, N, H, L, chunk, nchunk, seq, lane);
+}
+
 }  // namespace
+
+// Below this many sequences the backward pass puts four waves on each (D = 32 over 256 steps, four
+// waves against one: 512 sequences 227 against 408 us, 768: 365 against 415 us, 1024: 437 against
+// 426 us; beyond that the two are level).
+constexpr int kQuadMaxSeq = 1023;
 
 bool reg_lstm_supported(int D) { return D == 16 || D == 32; }
 
@@ -485,6 +835,15 @@ int reg_lstm_bwd(const LstmGates &g, const float *vdiff, const float *gates, con
                  const float *ckpt, float *gz, float *gk, float *gv, float *gbeta, int N, int H, int L,
                  int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (nseq <= kQuadMaxSeq) {
+        if (D == 16)
+            hipLaunchKernelGGL((k_lstm_bwd_quad<16>), dim3(nseq), dim3(kWave * 4), 0, s, g, vdiff, gates, out,
+                               cell, h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, chunk, nchunk);
+        else
+            hipLaunchKernelGGL((k_lstm_bwd_quad<32>), dim3(nseq), dim3(kWave * 4), 0, s, g, vdiff, gates, out,
+                               cell, h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, chunk, nchunk);
+        return (int)hipGetLastError();
+    }
     if (D == 16)
         hipLaunchKernelGGL((k_lstm_bwd_reg<16, 2, 1, 1>), dim3(nseq), dim3(kWave), 0, s, g, vdiff, gates,
                            out, cell, h_init, c_init, go, ckpt, gz, gk, gv, gbeta, N, H, L, chunk, nchunk,

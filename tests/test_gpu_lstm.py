@@ -91,3 +91,28 @@ def test_lstm_gradient_from_the_cell_output_is_ignored(fwp):
     (out * dev(go)).sum().backward()
     want = oracle.lstm_bwd(Zs, Ks, Vs, Bs, Ws, h0, c0, go)
     check("grad_z_u", diff[1][0].grad, want[0][1])
+
+
+@pytest.mark.parametrize("D,T", [(32, 45), (16, 70)])
+def test_lstm_backward_one_and_four_waves_per_sequence(fwp, D, T):
+    """Below 1024 sequences the backward pass puts four waves on a sequence, from there on one:
+    1100 sequences in one call against the same sequences in calls of 600 and 500.
+    Tolerance: |a - b| <= 1e-4 + 1e-3 |b|."""
+    Zs, Ks, Vs, Bs, Ws, h0, c0, go = lstm_inputs(21, 1100, 1, T, D, dtype=np.float32, w0=True)
+    tens = [dev(x) for x in (*Zs, *Ks, *Vs, *Bs)]
+    Wd, hd, cd, god = [dev(w) for w in Ws], dev(h0), dev(c0), dev(go)
+
+    def grads(sl):
+        ts = [t[sl].clone().requires_grad_(True) for t in tens]
+        args = []
+        for a in range(3):
+            args += [ts[a], ts[3 + a], ts[6 + a], ts[9 + a], Wd[a][sl].clone()]
+        out, _ = fwp.fast_lstm_v4(*args, hd[sl].clone(), cd[sl].clone())
+        return torch.autograd.grad(out, ts, god[sl])
+
+    whole = grads(slice(0, 1100))
+    parts = [grads(slice(0, 600)), grads(slice(600, 1100))]
+    for i, w in enumerate(whole):
+        got = torch.cat([parts[0][i], parts[1][i]], 0)
+        assert torch.isfinite(got).all()
+        assert torch.allclose(got, w, atol=1e-4, rtol=1e-3), (i, float((got - w).abs().max()))
