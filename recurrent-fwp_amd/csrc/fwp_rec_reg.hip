@@ -1,12 +1,12 @@
 // Register-state kernels of the Recurrent Delta Net op (rec_update_fwm_tanh) for D in {16, 32}.
 //
 // On top of the delta-rule state, the slow recurrent matrices R_q, R_k, R_v of the head are held
-// in VGPRs in the same layout as the state (by columns in forward, by rows in backward, where the
-// three gradient accumulators of R_* live in VGPRs too and are written out once per sequence).
-// Per step the fed-back vector tanh(out_{t-1}) and the activated q and k are "grouped" vectors
-// (every lane of group m holds entry m) that become periodic operands through ds_bpermute; the
-// softmax maxima/sums, the beta logit and the softmax-Jacobian dot products are wave-wide
-// reductions (DPP row rotates + two row swaps).
+// in VGPRs in the same layout as the state (by columns in forward, by rows in backward; the
+// gradients of R_* are accumulated by a second wave on the matrix cores and written out once per
+// sequence).  Per step the fed-back vector tanh(out_{t-1}) and the activated q and k are "grouped"
+// vectors (every lane of group m holds entry m) that become periodic operands through ds_bpermute;
+// the softmax maxima/sums, the beta logit and the softmax-Jacobian dot products are wave-wide
+// reductions (DPP row rotates, two row broadcasts and a lane read).
 #include "fwp_reg.hpp"
 
 namespace fwp {
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
     if (sl == 0) hstate[seq * D + col] = hcur;
 }
 
-// ----------------------------------------------------------------- backward
+// ----------------------------------------------------------------- backward, two waves per sequence
 
 template <int D>
 struct RecBwdOps {
@@ -198,58 +198,53 @@ struct RecBwdOps {
     float q_i, k_i, go_i, d_i, y_i, b;
 };
 
-template <int D, int RING, int PF, int WPB>
-__global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
-    const float *__restrict__ q_act, const float *__restrict__ k_act,
-    const float *__restrict__ beta_act, const float *__restrict__ vdiff,
-    const float *__restrict__ out, const float *__restrict__ h_init, fwp_view go,
-    const float *__restrict__ Rq, const float *__restrict__ Rk, const float *__restrict__ Rv,
-    const float *__restrict__ rb, const float *__restrict__ ckpt, float *__restrict__ gqx,
-    float *__restrict__ gkx, float *__restrict__ gvx, float *__restrict__ gbx,
-    float *__restrict__ workspace, int H, int L, int chunk, int nchunk, int nseq) {
+// Nearly all of the backward step is sequential (the gradient reaches h_{t-1} through q, k, v and
+// beta alike); what is not is the gradient of the slow recurrent weights, sums over time of
+// tanh(h_{t-1}) (x) grad_qx, grad_kx, grad_vx and tanh(h_{t-1}) grad_bx.  A second wave, one tile
+// of 16 steps behind, takes those tiles from LDS and accumulates the sums on the matrix cores
+// (X^T Y over the 16 steps of a tile).  One workgroup barrier per tile; a workgroup holds two
+// sequences.
+template <int D>
+struct RecPairLds {
+    float q[2][kTile * D], k[2][kTile * D], go[2][kTile * D], d[2][kTile * D], u[2][kTile * D];
+    float y[3][kTile * D];                    // tanh of the delayed output: ring of three tiles
+    float grad[2][3][kTile * D + 16];         // staged gqx, gkx, gvx, by tile parity
+    float b[2][kTile], gb[2][kTile];
+};
+
+template <int D>
+__device__ __forceinline__ void rec_bwd_pair_x(RecPairLds<D> &M, const float *__restrict__ q_act,
+                                               const float *__restrict__ k_act,
+                                               const float *__restrict__ beta_act,
+                                               const float *__restrict__ vdiff,
+                                               const float *__restrict__ out,
+                                               const float *__restrict__ h_init, fwp_view go,
+                                               const float *__restrict__ Rq, const float *__restrict__ Rk,
+                                               const float *__restrict__ Rv, const float *__restrict__ rb,
+                                               const float *__restrict__ ckpt, float *__restrict__ gqx,
+                                               float *__restrict__ gkx, float *__restrict__ gvx,
+                                               float *__restrict__ gbx, int H, int L, int chunk, int nchunk,
+                                               int64_t seq, int lane) {
     using G = Geo<D>;
     constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
-    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
-    __shared__ __align__(16) float sq_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sgo_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sd_[WPB][2][kTile * D];
-    __shared__ __align__(16) float su_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sy_[WPB][2][kTile * D];   // tanh of the delayed output
-    __shared__ __align__(16) float sb_[WPB][2][kTile];
-    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gqx, gkx, gvx tiles
-    __shared__ __align__(16) float sgb_[WPB][kTile];                 // staged gbx
-
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
-    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
-    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
-    if (seq >= nseq) return;
+    const int i = lane / S, sl = lane % S, per = lane % 16;
     const int h = (int)(seq % H), n = (int)(seq / H);
-    auto &sq = sq_[wave];
-    auto &sk = sk_[wave];
-    auto &sgo = sgo_[wave];
-    auto &sd = sd_[wave];
-    auto &su = su_[wave];
-    auto &sy = sy_[wave];
-    auto &sb = sb_[wave];
-    auto &sgrad = sgrad_[wave];
-    auto &sgb = sgb_[wave];
     const float *gob = row(go, n, h, 0);
     const float *qb = q_act + seq * L * D, *kb = k_act + seq * L * D, *db = vdiff + seq * L * D,
                 *ob = out + seq * L * D, *hib = h_init + seq * D, *bb = beta_act + seq * L;
 
-    // row i of: the state, its gradient (also column i of it), the recurrent matrices and their gradients
-    float Wr[R], Gr[R], Gc[R], Wnext[R], Rqr[R], Rkr[R], Rvr[R], gRq[R], gRk[R], gRv[R];
+    // row i of: the state, its gradient (also column i of it) and the recurrent matrices
+    float Wr[R], Gr[R], Gc[R], Wnext[R], Rqr[R], Rkr[R], Rvr[R];
 #pragma unroll
     for (int jj = 0; jj < R; jj++) {
         const int m = reg_index<D>(lane, jj);
-        Gr[jj] = Gc[jj] = Wr[jj] = gRq[jj] = gRk[jj] = gRv[jj] = 0.f;
+        Gr[jj] = Gc[jj] = Wr[jj] = 0.f;
         Rqr[jj] = Rq[((int64_t)h * D + i) * D + m];
         Rkr[jj] = Rk[((int64_t)h * D + i) * D + m];
         Rvr[jj] = Rv[((int64_t)h * D + i) * D + m];
     }
     const float rb_i = rb[(int64_t)h * D + i];
-    float grb_i = 0.f, dh_i = 0.f;
+    float dh_i = 0.f;
 
     TileRegs<D> pq, pk, pgo, pd, pu, py;
     float pb = 0.f;
@@ -281,47 +276,44 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
         pu.scale_rows(bs);
         pb = bb[min(t0 + per, L - 1)];
     };
-    auto commit = [&](int buf) {
-        pq.commit(sq[buf], lane);
-        pk.commit(sk[buf], lane);
-        pgo.commit(sgo[buf], lane);
-        pd.commit(sd[buf], lane);
-        pu.commit(su[buf], lane);
-        sb[buf][per] = pb;
+    auto commit = [&](int it) {
+        const int buf = it & 1;
+        pq.commit(M.q[buf], lane);
+        pk.commit(M.k[buf], lane);
+        pgo.commit(M.go[buf], lane);
+        pd.commit(M.d[buf], lane);
+        pu.commit(M.u[buf], lane);
+        M.b[buf][per] = pb;
 #pragma unroll
         for (int x = 0; x < NV4; x++) {
             float4 &r = py.r[x];
             r.x = fast_tanh(r.x); r.y = fast_tanh(r.y); r.z = fast_tanh(r.z); r.w = fast_tanh(r.w);
         }
-        py.commit(sy[buf], lane);
+        py.commit(M.y[it % 3], lane);
     };
     auto fetch_state = [&](int c) {
         const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
 #pragma unroll
         for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
     };
-
-    // S = 4: s=0 -> gqx, s=1 -> gkx, s=2,3 -> gvx.   S = 2: s=0 -> gqx, s=1 -> gkx, second write gvx.
-    float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
-    float *dst2 = sgrad[2] + i;
     float *gq_rows = gqx + seq * L * D, *gk_rows = gkx + seq * L * D, *gv_rows = gvx + seq * L * D;
 
-    auto load_ops = [&](RecBwdOps<D> &o, int buf, int tt) {
-        const int off = tt * D;
+    auto load_ops = [&](RecBwdOps<D> &o, int it, int tt) {
+        const int buf = it & 1, off = tt * D;
 #pragma unroll
         for (int p = 0; p < NP; p++) {
-            o.q[p] = sq[buf][off + 16 * p + per];
-            o.k[p] = sk[buf][off + 16 * p + per];
-            o.u[p] = su[buf][off + 16 * p + per];
+            o.q[p] = M.q[buf][off + 16 * p + per];
+            o.k[p] = M.k[buf][off + 16 * p + per];
+            o.u[p] = M.u[buf][off + 16 * p + per];
         }
-        o.q_i = sq[buf][off + i];
-        o.k_i = sk[buf][off + i];
-        o.go_i = sgo[buf][off + i];
-        o.d_i = sd[buf][off + i];
-        o.y_i = sy[buf][off + i];
-        o.b = sb[buf][tt];
+        o.q_i = M.q[buf][off + i];
+        o.k_i = M.k[buf][off + i];
+        o.go_i = M.go[buf][off + i];
+        o.d_i = M.d[buf][off + i];
+        o.y_i = M.y[it % 3][off + i];
+        o.b = M.b[buf][tt];
     };
-    auto compute = [&](const RecBwdOps<D> &o, int tt) {
+    auto compute = [&](const RecBwdOps<D> &o, int it, int tt) {
         const float g_i = dh_i + o.go_i;                      // gradient of out_t
         float g[NP], a[NP], gqp[NP], gkp[NP], gvp[NP];
         to_periodic<D>(g_i, g, lane);
@@ -352,79 +344,155 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_bwd_reg(
         acc = group_sum<S>(dot_rot<D>(Rvr, gvp, acc));
         acc = fmaf(rb_i, gbx_t, acc);
         dh_i = (1.f - o.y_i * o.y_i) * acc;
-        rank1_rot<D>(gRq, gqp, o.y_i);
-        rank1_rot<D>(gRk, gkp, o.y_i);
-        rank1_rot<D>(gRv, gvp, o.y_i);
-        grb_i = fmaf(o.y_i, gbx_t, grb_i);
         const float o_q = pinned(gqx_i), o_k = pinned(gkx_i), o_v = pinned(gvx_i);
+        float *g0 = M.grad[it & 1][0] + tt * D + i, *g1 = M.grad[it & 1][1] + tt * D + i,
+              *g2 = M.grad[it & 1][2] + tt * D + i;
         if constexpr (S == 4) {
-            dst1[tt * D] = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
+            *(sl == 0 ? g0 : (sl == 1 ? g1 : g2)) = sl == 0 ? o_q : (sl == 1 ? o_k : o_v);
         } else {
-            dst1[tt * D] = sl == 0 ? o_q : o_k;
-            dst2[tt * D] = o_v;
+            *(sl == 0 ? g0 : g1) = sl == 0 ? o_q : o_k;
+            *g2 = o_v;
         }
-        sgb[tt] = gbx_t;
+        M.gb[it & 1][tt] = gbx_t;
     };
-    auto flush = [&](int t0) {
-        flush_tile<D>(sgrad[0], gq_rows, t0, L, lane);
-        flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
-        flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
-        const float x = sgb[per];
+    auto flush = [&](int it) {
+        const int t0 = it * kTile;
+        flush_tile<D>(M.grad[it & 1][0], gq_rows, t0, L, lane);
+        flush_tile<D>(M.grad[it & 1][1], gk_rows, t0, L, lane);
+        flush_tile<D>(M.grad[it & 1][2], gv_rows, t0, L, lane);
+        const float x = M.gb[it & 1][per];
         if (lane < kTile && t0 + lane < L) gbx[seq * L + t0 + lane] = x;
     };
 
     const int ntile = (L + kTile - 1) / kTile;
     fetch((ntile - 1) * kTile);
-    commit((ntile - 1) & 1);
+    commit(ntile - 1);
     fetch_state(nchunk - 1);
     if (ntile > 1) fetch((ntile - 2) * kTile);
-    RecBwdOps<D> ring[RING];
-    bool primed = false;
+    __syncthreads();
 
     for (int it = ntile - 1; it >= 0; it--) {
-        const int buf = it & 1, t0 = it * kTile;
+        const int t0 = it * kTile;
         const int nst = min(kTile, L - t0);
         const int t_end = t0 + nst;
         if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
 #pragma unroll
             for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
         }
-        if (it >= 1) commit(buf ^ 1);
-        if (it + 1 < ntile) flush(t0 + kTile);
+        if (it >= 1) commit(it - 1);
+        if (it + 1 < ntile) flush(it + 1);
         if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
         if (it >= 2) fetch(t0 - 2 * kTile);
         if (nst == kTile) {
-            if (!primed) {
-#pragma unroll
-                for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
-                primed = true;
-            }
+            RecBwdOps<D> ring[2];
+            load_ops(ring[(kTile - 1) & 1], it, kTile - 1);
 #pragma unroll
             for (int tt = kTile - 1; tt >= 0; tt--) {
-                const int nt = tt - PF;
-                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
-                else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
-                compute(ring[tt % RING], tt);
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], it, tt - 1);
+                compute(ring[tt & 1], it, tt);
             }
         } else {  // ragged last tile (first in reverse): not pipelined
             for (int tt = nst - 1; tt >= 0; tt--) {
                 RecBwdOps<D> o;
-                load_ops(o, buf, tt);
-                compute(o, tt);
+                load_ops(o, it, tt);
+                compute(o, it, tt);
             }
         }
+        __syncthreads();
     }
     flush(0);
+}
+
+typedef float rec_v4f __attribute__((ext_vector_type(4)));
+
+template <int D>
+__device__ __forceinline__ void rec_bwd_pair_y(RecPairLds<D> &M, float *__restrict__ workspace, int L,
+                                               int64_t seq, int lane) {
+    constexpr int NT = D / 16;
+    // acc[x][mt][nt]: lane l, register r holds entry (16 mt + 4 (l / 16) + r, 16 nt + l % 16) of
+    // sum_t y_t (x) grad_x; accb the same for y_t grad_bx in column 0
+    rec_v4f acc[3][NT][NT], accb[NT];
+#pragma unroll
+    for (int mt = 0; mt < NT; mt++) {
+        accb[mt] = rec_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int x = 0; x < 3; x++)
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) acc[x][mt][nt] = rec_v4f{0.f, 0.f, 0.f, 0.f};
+    }
+    const int r4 = lane / 16, c = lane % 16;
+    auto run_tile = [&](int ty) {
+        const int nst = min(kTile, L - ty * kTile);
+        const float *y = M.y[ty % 3];
+#pragma unroll
+        for (int j = 0; j < kTile / 4; j++) {       // four steps to an MFMA: step 4 j + l / 16
+            const int tt = 4 * j + r4;
+            const bool ok = tt < nst;
+            float a[NT], b[3][NT];
+#pragma unroll
+            for (int mt = 0; mt < NT; mt++) a[mt] = ok ? y[tt * D + 16 * mt + c] : 0.f;
+#pragma unroll
+            for (int x = 0; x < 3; x++)
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) b[x][nt] = ok ? M.grad[ty & 1][x][tt * D + 16 * nt + c] : 0.f;
+            const float bcol = ok && c == 0 ? M.gb[ty & 1][tt] : 0.f;
+#pragma unroll
+            for (int mt = 0; mt < NT; mt++) {
+#pragma unroll
+                for (int x = 0; x < 3; x++)
+#pragma unroll
+                    for (int nt = 0; nt < NT; nt++)
+                        acc[x][mt][nt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], b[x][nt], acc[x][mt][nt], 0, 0, 0);
+                accb[mt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[mt], bcol, accb[mt], 0, 0, 0);
+            }
+        }
+    };
+    const int ntile = (L + kTile - 1) / kTile;
+    __syncthreads();
+    for (int it = ntile - 1; it >= 0; it--) {     // the tile X works on; this wave is one behind
+        if (it + 1 < ntile) run_tile(it + 1);
+        __syncthreads();
+    }
+    run_tile(0);
     // this sequence's share of the parameter gradients: [gRq | gRk | gRv | grb], rows e, columns m
     float *ws = workspace + seq * (3 * D * D + D);
 #pragma unroll
-    for (int jj = 0; jj < R; jj++) {
-        const int m = reg_index<D>(lane, jj);
-        ws[i * D + m] = gRq[jj];
-        ws[D * D + i * D + m] = gRk[jj];
-        ws[2 * D * D + i * D + m] = gRv[jj];
+    for (int mt = 0; mt < NT; mt++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const int e = 16 * mt + 4 * r4 + r;
+#pragma unroll
+            for (int x = 0; x < 3; x++)
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) ws[x * D * D + e * D + 16 * nt + c] = acc[x][mt][nt][r];
+            if (c == 0) ws[3 * D * D + e] = accb[mt][r];
+        }
+}
+
+template <int D>
+__global__ __launch_bounds__(kWave * 4) void k_rec_bwd_pair(
+    const float *__restrict__ q_act, const float *__restrict__ k_act,
+    const float *__restrict__ beta_act, const float *__restrict__ vdiff,
+    const float *__restrict__ out, const float *__restrict__ h_init, fwp_view go,
+    const float *__restrict__ Rq, const float *__restrict__ Rk, const float *__restrict__ Rv,
+    const float *__restrict__ rb, const float *__restrict__ ckpt, float *__restrict__ gqx,
+    float *__restrict__ gkx, float *__restrict__ gvx, float *__restrict__ gbx,
+    float *__restrict__ workspace, int H, int L, int chunk, int nchunk, int nseq) {
+    extern __shared__ __align__(16) unsigned char pair_lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
+    RecPairLds<D> &M = reinterpret_cast<RecPairLds<D> *>(pair_lds)[wave & 1];
+    if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
+        const int ntile = (L + kTile - 1) / kTile;
+        for (int it = ntile; it >= 0; it--) __syncthreads();
+        return;
     }
-    if (sl == 0) ws[3 * D * D + i] = grb_i;
+    if (wave < 2)
+        rec_bwd_pair_x<D>(M, q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx, gkx, gvx,
+                          gbx, H, L, chunk, nchunk, seq, lane);
+    else
+        rec_bwd_pair_y<D>(M, workspace, L, seq, lane);
 }
 
 }  // namespace
@@ -453,15 +521,17 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
                 float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
                 int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
-    if (D == 16)
-        hipLaunchKernelGGL((k_rec_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                           q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
-                           gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
-    else
-        hipLaunchKernelGGL((k_rec_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
-                           q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx,
-                           gkx, gvx, gbx, workspace, H, L, chunk, nchunk, nseq);
-    return (int)hipGetLastError();
+    auto launch = [&](auto kernel, size_t lds) {
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+            return (int)e;
+        hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, q_act, k_act, beta_act, vdiff,
+                           out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx, gkx, gvx, gbx, workspace, H, L, chunk,
+                           nchunk, nseq);
+        return (int)hipGetLastError();
+    };
+    return D == 16 ? launch(k_rec_bwd_pair<16>, 2 * sizeof(RecPairLds<16>))
+                   : launch(k_rec_bwd_pair<32>, 2 * sizeof(RecPairLds<32>));
 }
 
 }  // namespace fwp

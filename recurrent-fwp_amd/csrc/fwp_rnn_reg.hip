@@ -2,7 +2,7 @@
 // fwp_delta_reg.hip plus the recurrent read h_t = W_t^T softmax(h_{t-1}) + z_t.
 //
 // The recurrent vector lives "grouped" (every lane of group m holds h[m]); its softmax needs a max
-// and a sum over the whole wave (DPP row rotates + two row swaps each) and then becomes a periodic
+// and a sum over the whole wave (DPP row rotates, two row broadcasts and a lane read each) and then becomes a periodic
 // operand with one ds_bpermute per 16 entries.  In backward the softmax of the delayed output does
 // not sit on the sequential path: it is recomputed for a whole tile when the tile is committed.
 #include "fwp_reg.hpp"

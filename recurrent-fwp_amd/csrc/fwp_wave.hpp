@@ -3,7 +3,7 @@
 // A sequence is owned by ONE wave.  The D x D state lives in VGPRs: lane
 // l = i*S + s (i in [0,D), s in [0,S), D*S = 64) holds R = D/S elements of row or
 // column i.  Sums over the S lanes of a group are DPP quad permutes; sums over the
-// D groups are DPP row rotates plus two row swaps.
+// D groups are DPP row rotates, two row broadcasts and a lane read.
 #pragma once
 #include <hip/hip_runtime.h>
 
