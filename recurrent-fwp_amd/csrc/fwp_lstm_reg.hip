@@ -203,6 +203,305 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_fwd_reg(LstmGates g, float
     }
 }
 
+// ------------------------------------------- forward, two waves per sequence
+//
+// The three delta-rule writes do not depend on h, only the reads do.  Wave H, one tile ahead, runs
+// the writes on a copy of the states of its own and hands u = beta * (v - W^T k) over through LDS
+// (it also stores vdiff); wave M applies the same rank-one updates to its copy, reads the states
+// with softmax(h_{t-1}) and runs the cell: a third fewer multiply-adds on the sequential wave.  H
+// loads k (a ring of three tiles, which M reads too), v and beta, M loads z.  One workgroup barrier
+// per tile; a workgroup holds two sequences, that is four waves, one for each SIMD of a CU.
+template <int D>
+struct LstmFwdPairLds {
+    static constexpr int TL = lstm_tile<D>();
+    float k[3][3][TL * D];            // [slot][gate]
+    float v[3][TL * D], b[3][16];     // H only
+    float z[2][3][TL * D];            // M only
+    float u[2][3][TL * D];            // H -> M, by tile parity
+    float vd[3][TL * D + 16];         // staged vdiff (H)
+    float out[5][TL * D + 16];        // staged gates i, u, o, out, cell (M)
+};
+
+template <int D>
+struct LstmFwdOpsH {
+    float k[3][Geo<D>::NP], v[3], b[3];
+};
+template <int D>
+struct LstmFwdOpsM {
+    float k[3][Geo<D>::NP], u[3], z[3];
+};
+
+template <int D>
+__device__ __forceinline__ void lstm_fwd_pair_h(LstmFwdPairLds<D> &M, const LstmGates &g,
+                                                float *__restrict__ vdiff, int N, int H, int L,
+                                                int64_t seq, int lane) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    using Tile = TileRegs<D, TL>;
+    const int col = lane / S, sl = lane % S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+
+    float Wc[3][R];  // W_a[reg_index(jj)][col]
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++)
+            Wc[a][jj] = g.W[a][(seq * D + reg_index<D>(lane, jj)) * D + col];
+
+    Tile pk[3], pv[3];
+    float pb[3] = {0.f, 0.f, 0.f};
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane[3], *vlane[3], *bb[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) {
+        klane[a] = row(g.k[a], n, h, 0) + lrow * g.k[a].sL + 4 * lc4;
+        vlane[a] = row(g.v[a], n, h, 0) + lrow * g.v[a].sL + 4 * lc4;
+        bb[a] = row(g.beta[a], n, h, 0);
+    }
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            if (t0 + TL <= L) {
+                pk[a].template fetch<true>(klane[a], g.k[a].sL, t0, L, lane);
+                pv[a].template fetch<true>(vlane[a], g.v[a].sL, t0, L, lane);
+            } else {
+                pk[a].template fetch<false>(klane[a], g.k[a].sL, t0, L, lane);
+                pv[a].template fetch<false>(vlane[a], g.v[a].sL, t0, L, lane);
+            }
+            pb[a] = bb[a][(int64_t)min(t0 + per % TL, L - 1) * g.beta[a].sL];
+        }
+    };
+    auto commit = [&](int it) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            pk[a].commit(M.k[it % 3][a], lane);
+            pv[a].commit(M.v[a], lane);
+            M.b[a][per % TL] = pb[a];
+        }
+    };
+    auto flush = [&](int it) {
+        if (!vdiff) return;
+#pragma unroll
+        for (int a = 0; a < 3; a++)
+            flush_tile<D, TL>(M.vd[a], vdiff + a * gate_stride + seq * L * D, it * TL, L, lane);
+    };
+    auto load_ops = [&](LstmFwdOpsH<D> &o, int it, int tt) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) o.k[a][p] = M.k[it % 3][a][tt * D + 16 * p + per];
+            o.v[a] = M.v[a][tt * D + col];
+            o.b[a] = M.b[a][tt];
+        }
+    };
+    auto compute = [&](const LstmFwdOpsH<D> &o, int it, int tt) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            const float d = o.v[a] - group_sum<S>(dot_rot<D>(Wc[a], o.k[a]));
+            const float u = o.b[a] * d;
+            rank1_rot<D>(Wc[a], o.k[a], u);
+            const float o_d = pinned(d), o_u = pinned(u);
+            // lane 0 of a group stages vdiff, lane 1 hands u over: one LDS write for both
+            *(sl == 0 ? M.vd[a] + tt * D + col : M.u[it & 1][a] + tt * D + col) = sl == 0 ? o_d : o_u;
+        }
+    };
+    auto run_tile = [&](int it) {
+        const int nst = min(TL, L - it * TL);
+        if (nst == TL) {
+            LstmFwdOpsH<D> ring[2];
+            load_ops(ring[0], it, 0);
+#pragma unroll
+            for (int tt = 0; tt < TL; tt++) {
+                if (tt + 1 < TL) load_ops(ring[(tt + 1) & 1], it, tt + 1);
+                compute(ring[tt & 1], it, tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                LstmFwdOpsH<D> o;
+                load_ops(o, it, tt);
+                compute(o, it, tt);
+            }
+        }
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    fetch(0);
+    for (int it = -1; it < ntile; it++) {     // the tile M works on; this wave is one ahead
+        if (it + 1 < ntile) {
+            if (it >= 0) flush(it);
+            commit(it + 1);
+            if (it + 2 < ntile) fetch((it + 2) * TL);
+            run_tile(it + 1);
+        }
+        __syncthreads();
+    }
+    flush(ntile - 1);
+}
+
+template <int D>
+__device__ __forceinline__ void lstm_fwd_pair_m(LstmFwdPairLds<D> &M, const LstmGates &g,
+                                                float *__restrict__ hstate, float *__restrict__ cstate,
+                                                float *__restrict__ out, float *__restrict__ cell,
+                                                float *__restrict__ gates, float *__restrict__ ckpt, int N,
+                                                int H, int L, int chunk, int nchunk, int64_t seq,
+                                                int lane) {
+    constexpr int TL = lstm_tile<D>();
+    using G = Geo<D, TL>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    using Tile = TileRegs<D, TL>;
+    const int col = lane / S, sl = lane % S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const int64_t gate_stride = (int64_t)N * H * L * D;
+    const int64_t ckpt_stride = (int64_t)N * H * nchunk * D * D;
+
+    float Wc[3][R];  // W_a[reg_index(jj)][col]
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++)
+            Wc[a][jj] = g.W[a][(seq * D + reg_index<D>(lane, jj)) * D + col];
+    float hcur = hstate[seq * D + col], ccur = cstate[seq * D + col];
+
+    Tile pz[3];
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *zlane[3];
+#pragma unroll
+    for (int a = 0; a < 3; a++) zlane[a] = row(g.z[a], n, h, 0) + lrow * g.z[a].sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            if (t0 + TL <= L) pz[a].template fetch<true>(zlane[a], g.z[a].sL, t0, L, lane);
+            else pz[a].template fetch<false>(zlane[a], g.z[a].sL, t0, L, lane);
+        }
+    };
+    auto commit = [&](int it) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) pz[a].commit(M.z[it & 1][a], lane);
+    };
+    auto flush = [&](int it) {
+        const int64_t base = seq * L * D;
+        if (gates) {
+#pragma unroll
+            for (int a = 0; a < 3; a++)
+                flush_tile<D, TL>(M.out[a], gates + a * gate_stride + base, it * TL, L, lane);
+        }
+        flush_tile<D, TL>(M.out[3], out + base, it * TL, L, lane);
+        flush_tile<D, TL>(M.out[4], cell + base, it * TL, L, lane);
+    };
+    auto load_ops = [&](LstmFwdOpsM<D> &o, int it, int tt) {
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+#pragma unroll
+            for (int p = 0; p < NP; p++) o.k[a][p] = M.k[it % 3][a][tt * D + 16 * p + per];
+            o.u[a] = M.u[it & 1][a][tt * D + col];
+            o.z[a] = M.z[it & 1][a][tt * D + col];
+        }
+    };
+    auto compute = [&](const LstmFwdOpsM<D> &o, int tt) {
+        const float mx = across_groups<S>(hcur, OpMax());
+        const float e = __expf(hcur - mx);
+        // the reads below use e and are scaled by 1 / sum(e) afterwards: the wave-wide sum then runs
+        // beside them instead of ahead of them on the sequential path
+        float s[NP];
+        to_periodic<D>(e, s, lane);
+        const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));
+        float pre[3];
+#pragma unroll
+        for (int a = 0; a < 3; a++) {
+            rank1_rot<D>(Wc[a], o.k[a], o.u[a]);
+            pre[a] = fmaf(group_sum<S>(dot_rot<D>(Wc[a], s)), rsum, o.z[a]);
+        }
+        const float gi = sigmoidf_fast(pre[0]), go = sigmoidf_fast(pre[2]);
+        ccur = fmaf(gi, pre[1] - ccur, ccur);          // i u + (1 - i) c
+        hcur = pinned(go * ccur);
+        const float o_i = pinned(gi), o_u = pinned(pre[1]), o_o = pinned(go), o_c = pinned(ccur);
+        float *st = M.out[0] + tt * D + col;
+        constexpr int kStride = TL * D + 16;
+        if constexpr (S == 4) {
+            st[sl * kStride] = sl == 0 ? o_i : (sl == 1 ? o_u : (sl == 2 ? o_o : hcur));
+            st[4 * kStride] = o_c;
+        } else {
+            st[sl * kStride] = sl == 0 ? o_i : o_u;
+            st[(2 + sl) * kStride] = sl == 0 ? o_o : hcur;
+            st[4 * kStride] = o_c;
+        }
+    };
+
+    const int ntile = (L + TL - 1) / TL;
+    fetch(0);
+    commit(0);
+    if (ntile > 1) fetch(TL);
+    __syncthreads();
+    for (int it = 0; it < ntile; it++) {
+        const int t0 = it * TL;
+        const int nst = min(TL, L - t0);
+        if (it + 1 < ntile) commit(it + 1);
+        if (it > 0) flush(it - 1);
+        if (it + 2 < ntile) fetch(t0 + 2 * TL);
+        if (nst == TL) {
+            LstmFwdOpsM<D> ring[2];
+            load_ops(ring[0], it, 0);
+#pragma unroll
+            for (int tt = 0; tt < TL; tt++) {
+                if (tt + 1 < TL) load_ops(ring[(tt + 1) & 1], it, tt + 1);
+                compute(ring[tt & 1], tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                LstmFwdOpsM<D> o;
+                load_ops(o, it, tt);
+                compute(o, tt);
+            }
+        }
+        const int t_end = t0 + nst;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+#pragma unroll
+            for (int a = 0; a < 3; a++) {
+                float *c = ckpt + a * ckpt_stride + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+                for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[a][jj];
+            }
+        }
+        __syncthreads();
+    }
+    flush(ntile - 1);
+#pragma unroll
+    for (int a = 0; a < 3; a++)
+#pragma unroll
+        for (int jj = 0; jj < R; jj++)
+            g.W[a][(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[a][jj];
+    if (sl == 0) {
+        hstate[seq * D + col] = hcur;
+        cstate[seq * D + col] = ccur;
+    }
+}
+
+template <int D>
+__global__ __launch_bounds__(kWave * 4) void k_lstm_fwd_pair(LstmGates g, float *__restrict__ hstate,
+                                                             float *__restrict__ cstate,
+                                                             float *__restrict__ out,
+                                                             float *__restrict__ cell,
+                                                             float *__restrict__ gates,
+                                                             float *__restrict__ vdiff,
+                                                             float *__restrict__ ckpt, int N, int H, int L,
+                                                             int chunk, int nchunk, int nseq) {
+    extern __shared__ __align__(16) unsigned char pair_lds[];
+    constexpr int TL = lstm_tile<D>();
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
+    LstmFwdPairLds<D> &M = reinterpret_cast<LstmFwdPairLds<D> *>(pair_lds)[wave & 1];
+    if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
+        const int ntile = (L + TL - 1) / TL;
+        for (int it = ntile; it >= 0; it--) __syncthreads();
+        return;
+    }
+    if (wave < 2) lstm_fwd_pair_m<D>(M, g, hstate, cstate, out, cell, gates, ckpt, N, H, L, chunk, nchunk, seq, lane);
+    else lstm_fwd_pair_h<D>(M, g, vdiff, N, H, L, seq, lane);
+}
+
 // ----------------------------------------------------------------- backward
 
 template <int D>
@@ -811,6 +1110,9 @@ __global__ __launch_bounds__(kWave * 4) void k_lstm_bwd_quad(
 
 }  // namespace
 
+// Up to this many sequences (two waves on a SIMD beyond it) the forward pass puts two waves on each
+// (D = 32 over 256 steps, two waves against one: 512 sequences 143 against 175 us, 768: 279 against 198 us).
+constexpr int kFwdPairMaxSeq = 512;
 // Below this many sequences the backward pass puts four waves on each (D = 32 over 256 steps, four
 // waves against one: 512 sequences 227 against 408 us, 768: 365 against 415 us, 1024: 437 against
 // 426 us; beyond that the two are level).
@@ -821,6 +1123,18 @@ bool reg_lstm_supported(int D) { return D == 16 || D == 32; }
 int reg_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, float *gates,
                  float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (nseq <= kFwdPairMaxSeq) {
+        auto launch = [&](auto kernel, size_t lds) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return (int)e;
+            hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, g, h, c, out, cell, gates,
+                               vdiff, ckpt, N, H, L, chunk, nchunk, nseq);
+            return (int)hipGetLastError();
+        };
+        return D == 16 ? launch(k_lstm_fwd_pair<16>, 2 * sizeof(LstmFwdPairLds<16>))
+                       : launch(k_lstm_fwd_pair<32>, 2 * sizeof(LstmFwdPairLds<32>));
+    }
     if (D == 16)
         hipLaunchKernelGGL((k_lstm_fwd_reg<16, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, g,
                            h, c, out, cell, gates, vdiff, ckpt, N, H, L, chunk, nchunk, nseq);
