@@ -151,6 +151,218 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
     if (sl == 0) hstate[seq * D + col] = hcur;
 }
 
+// ------------------------------------------- forward, two waves per sequence
+//
+// The delta-rule write does not depend on h, only the read does.  Wave H, one tile ahead, runs the
+// writes on a copy of the state of its own and hands u = beta * (v - W^T k) over through LDS (it also
+// stores vdiff); wave M applies the same rank-one updates to its copy and reads the state with
+// softmax(h_{t-1}): a third fewer multiply-adds on the sequential wave.  H loads k (a ring of three
+// tiles, which M reads too), v and beta, M loads z.  One workgroup barrier per tile; a workgroup
+// holds two sequences, that is four waves, one for each SIMD of a CU.
+template <int D>
+struct RnnFwdPairLds {
+    float k[3][kTile * D];
+    float v[kTile * D], b[kTile];     // H only
+    float z[2][kTile * D];            // M only
+    float u[2][kTile * D];            // H -> M, by tile parity
+    float vd[kTile * D + 16];         // staged vdiff (H)
+    float out[kTile * D + 16];        // staged out (M)
+};
+
+template <int D>
+struct RnnFwdOpsH {
+    float k[Geo<D>::NP], v, b;
+};
+template <int D>
+struct RnnFwdOpsM {
+    float k[Geo<D>::NP], u, z;
+};
+
+template <int D>
+__device__ __forceinline__ void rnn_fwd_pair_h(RnnFwdPairLds<D> &M, fwp_view k, fwp_view v, fwp_view beta,
+                                               const float *__restrict__ W, float *__restrict__ vdiff,
+                                               int H, int L, int64_t seq, int lane) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    const int col = lane / S, sl = lane % S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *kb = row(k, n, h, 0), *vb = row(v, n, h, 0), *bb = row(beta, n, h, 0);
+
+    float Wc[R];  // W[reg_index(jj)][col]
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Wc[jj] = W[(seq * D + reg_index<D>(lane, jj)) * D + col];
+
+    TileRegs<D> pk, pv;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane = kb + lrow * k.sL + 4 * lc4, *vlane = vb + lrow * v.sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pv.template fetch<true>(vlane, v.sL, t0, L, lane);
+        } else {
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pv.template fetch<false>(vlane, v.sL, t0, L, lane);
+        }
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+    };
+    auto commit = [&](int it) {
+        pk.commit(M.k[it % 3], lane);
+        pv.commit(M.v, lane);
+        M.b[per] = pb;
+    };
+    auto load_ops = [&](RnnFwdOpsH<D> &o, int it, int tt) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) o.k[p] = M.k[it % 3][tt * D + 16 * p + per];
+        o.v = M.v[tt * D + col];
+        o.b = M.b[tt];
+    };
+    auto compute = [&](const RnnFwdOpsH<D> &o, int it, int tt) {
+        const float d = o.v - group_sum<S>(dot_rot<D>(Wc, o.k));
+        const float u = o.b * d;
+        rank1_rot<D>(Wc, o.k, u);
+        const float o_d = pinned(d), o_u = pinned(u);
+        // lane 0 of a group stages vdiff, lane 1 hands u over: one LDS write for both
+        *(sl == 0 ? M.vd + tt * D + col : M.u[it & 1] + tt * D + col) = sl == 0 ? o_d : o_u;
+    };
+    auto run_tile = [&](int it) {
+        const int nst = min(kTile, L - it * kTile);
+        if (nst == kTile) {
+            RnnFwdOpsH<D> ring[2];
+            load_ops(ring[0], it, 0);
+#pragma unroll
+            for (int tt = 0; tt < kTile; tt++) {
+                if (tt + 1 < kTile) load_ops(ring[(tt + 1) & 1], it, tt + 1);
+                compute(ring[tt & 1], it, tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                RnnFwdOpsH<D> o;
+                load_ops(o, it, tt);
+                compute(o, it, tt);
+            }
+        }
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    float *vd_rows = vdiff ? vdiff + seq * L * D : nullptr;
+    fetch(0);
+    for (int it = -1; it < ntile; it++) {     // the tile M works on; this wave is one ahead
+        if (it + 1 < ntile) {
+            if (it >= 0 && vd_rows) flush_tile<D>(M.vd, vd_rows, it * kTile, L, lane);
+            commit(it + 1);
+            if (it + 2 < ntile) fetch((it + 2) * kTile);
+            run_tile(it + 1);
+        }
+        __syncthreads();
+    }
+    if (vd_rows) flush_tile<D>(M.vd, vd_rows, (ntile - 1) * kTile, L, lane);
+}
+
+template <int D>
+__device__ __forceinline__ void rnn_fwd_pair_m(RnnFwdPairLds<D> &M, fwp_view z, float *__restrict__ W,
+                                               float *__restrict__ hstate, float *__restrict__ out,
+                                               float *__restrict__ ckpt, int H, int L, int chunk, int nchunk,
+                                               int64_t seq, int lane) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    const int col = lane / S, sl = lane % S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *zb = row(z, n, h, 0);
+
+    float Wc[R];  // W[reg_index(jj)][col]
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Wc[jj] = W[(seq * D + reg_index<D>(lane, jj)) * D + col];
+    float hcur = hstate[seq * D + col];
+
+    TileRegs<D> pz;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *zlane = zb + lrow * z.sL + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) pz.template fetch<true>(zlane, z.sL, t0, L, lane);
+        else pz.template fetch<false>(zlane, z.sL, t0, L, lane);
+    };
+    auto load_ops = [&](RnnFwdOpsM<D> &o, int it, int tt) {
+#pragma unroll
+        for (int p = 0; p < NP; p++) o.k[p] = M.k[it % 3][tt * D + 16 * p + per];
+        o.u = M.u[it & 1][tt * D + col];
+        o.z = M.z[it & 1][tt * D + col];
+    };
+    auto compute = [&](const RnnFwdOpsM<D> &o, int tt) {
+        // s = softmax(h_{t-1}) = e / sum(e); the read is done with e and scaled afterwards: the
+        // wave-wide sum then runs beside the read instead of ahead of it on the sequential path
+        const float mx = across_groups<S>(hcur, OpMax());
+        const float e = __expf(hcur - mx);
+        float s[NP];
+        to_periodic<D>(e, s, lane);
+        const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));
+        rank1_rot<D>(Wc, o.k, o.u);
+        hcur = fmaf(group_sum<S>(dot_rot<D>(Wc, s)), rsum, o.z);
+        hcur = pinned(hcur);
+        M.out[tt * D + col] = hcur;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    float *out_rows = out + seq * L * D;
+    fetch(0);
+    pz.commit(M.z[0], lane);
+    if (ntile > 1) fetch(kTile);
+    __syncthreads();
+    for (int it = 0; it < ntile; it++) {
+        const int t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        if (it + 1 < ntile) pz.commit(M.z[(it + 1) & 1], lane);
+        if (it > 0) flush_tile<D>(M.out, out_rows, t0 - kTile, L, lane);
+        if (it + 2 < ntile) fetch(t0 + 2 * kTile);
+        if (nst == kTile) {
+            RnnFwdOpsM<D> ring[2];
+            load_ops(ring[0], it, 0);
+#pragma unroll
+            for (int tt = 0; tt < kTile; tt++) {
+                if (tt + 1 < kTile) load_ops(ring[(tt + 1) & 1], it, tt + 1);
+                compute(ring[tt & 1], tt);
+            }
+        } else {  // ragged last tile: not pipelined
+            for (int tt = 0; tt < nst; tt++) {
+                RnnFwdOpsM<D> o;
+                load_ops(o, it, tt);
+                compute(o, tt);
+            }
+        }
+        const int t_end = t0 + nst;
+        if (ckpt && (t_end % chunk == 0 || t_end == L)) {
+            float *c = ckpt + (seq * nchunk + (t_end - 1) / chunk) * D * D;
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) c[reg_index<D>(lane, jj) * D + col] = Wc[jj];
+        }
+        __syncthreads();
+    }
+    flush_tile<D>(M.out, out_rows, (ntile - 1) * kTile, L, lane);
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) W[(seq * D + reg_index<D>(lane, jj)) * D + col] = Wc[jj];
+    if (sl == 0) hstate[seq * D + col] = hcur;
+}
+
+template <int D>
+__global__ __launch_bounds__(kWave * 4) void k_rnn_fwd_pair(fwp_view z, fwp_view k, fwp_view v, fwp_view beta,
+                                                            float *__restrict__ W, float *__restrict__ hstate,
+                                                            float *__restrict__ out, float *__restrict__ vdiff,
+                                                            float *__restrict__ ckpt, int H, int L, int chunk,
+                                                            int nchunk, int nseq) {
+    extern __shared__ __align__(16) unsigned char pair_lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
+    RnnFwdPairLds<D> &M = reinterpret_cast<RnnFwdPairLds<D> *>(pair_lds)[wave & 1];
+    if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
+        const int ntile = (L + kTile - 1) / kTile;
+        for (int it = ntile; it >= 0; it--) __syncthreads();
+        return;
+    }
+    if (wave < 2) rnn_fwd_pair_m<D>(M, z, W, hstate, out, ckpt, H, L, chunk, nchunk, seq, lane);
+    else rnn_fwd_pair_h<D>(M, k, v, beta, W, vdiff, H, L, seq, lane);
+}
+
 // ----------------------------------------------------------------- backward
 
 template <int D>
@@ -668,6 +880,9 @@ __global__ __launch_bounds__(kWave * 4) void k_rnn_bwd_pair(
 
 }  // namespace
 
+// up to this many sequences (one wave on each SIMD) the forward pass puts two waves on each
+constexpr int kFwdPairMaxSeq = 512;
+
 // The backward pass puts two waves on a sequence, except from 513 to 1024 sequences: there the
 // one-wave kernel has a SIMD for each wave and is as fast or a little faster (768 sequences of D = 32
 // over 256 steps: 130 against 136 us; 512: 131 against 101 us; 1280: 268 against 217 us).
@@ -678,6 +893,15 @@ bool reg_rnn_supported(int D) { return D == 16 || D == 32; }
 int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
+    if (nseq <= kFwdPairMaxSeq) {
+        auto launch = [&](auto kernel, size_t lds) {
+            hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, z, k, v, beta, W, h, out,
+                               vdiff, ckpt, H, L, chunk, nchunk, nseq);
+            return (int)hipGetLastError();
+        };
+        return D == 16 ? launch(k_rnn_fwd_pair<16>, 2 * sizeof(RnnFwdPairLds<16>))
+                       : launch(k_rnn_fwd_pair<32>, 2 * sizeof(RnnFwdPairLds<32>));
+    }
     if (D == 16)
         hipLaunchKernelGGL((k_rnn_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
                            k, v, beta, W, h, out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
