@@ -878,15 +878,355 @@ __global__ __launch_bounds__(kWave * 4) void k_rnn_bwd_pair(
         rnn_bwd_pair_y<D>(M, ckpt, gk, L, chunk, nchunk, seq, lane);
 }
 
+// ------------------------------------------- backward, three waves per sequence
+//
+// The same division taken one step further, for when there are SIMDs to spare: wave X keeps only the
+// sequential part (the gradient of h through W and the softmax; grad_z); wave A, one tile behind,
+// keeps G in column layout and computes r = G^T k, grad_v, grad_beta and a; wave Y, two tiles behind,
+// computes grad_k as before.  X loads the tiles into a ring of four slots (it fills the slot of tile
+// it - 1 while X, A and Y work on tiles it, it + 1 and it + 2).  A workgroup holds two sequences, six
+// waves on the four SIMDs of a CU.
+template <int D>
+struct RnnTriLds {
+    float k[4][kTile * D], u[4][kTile * D], s[4][kTile * D], d[4][kTile * D];
+    float b[4][kTile];
+    float go[2][kTile * D];
+    float g[3][kTile * D];      // X -> A, Y
+    float a[2][kTile * D];      // A -> Y
+    float pd[kTile * D];
+    float gk[kTile * D];
+};
+
+template <int D>
+struct RnnBwdOpsT {   // X of the three
+    float u[Geo<D>::NP];
+    float go_i, s_i, k_i;
+};
+template <int D>
+struct RnnBwdOpsA {
+    float s[Geo<D>::NP], k[Geo<D>::NP];
+    float g_i, d_i, b;
+};
+
+// Every role runs the same loop, so that the barriers' counts agree: in round j the role that is
+// LAG tiles behind works on tile ntile - 1 - (j - LAG), if there is such a tile.
+template <int LAG, typename F>
+__device__ __forceinline__ void tri_rounds(int ntile, F &&work) {
+    for (int j = 0; j < ntile + 2; j++) {
+        const int t = ntile - 1 - (j - LAG);
+        if (t >= 0 && t < ntile) work(t);
+        __syncthreads();
+    }
+}
+
+template <int D>
+__device__ __forceinline__ void rnn_bwd_tri_x(RnnTriLds<D> &M, fwp_view k, fwp_view beta,
+                                              const float *__restrict__ vdiff,
+                                              const float *__restrict__ out,
+                                              const float *__restrict__ h_init, fwp_view go,
+                                              const float *__restrict__ ckpt, float *__restrict__ gz, int H,
+                                              int L, int chunk, int nchunk, int64_t seq, int lane) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    const int i = lane / S, per = lane % 16;
+    const int n = (int)(seq / H), h = (int)(seq % H);
+    const float *kb = row(k, n, h, 0), *gob = row(go, n, h, 0), *bb = row(beta, n, h, 0);
+    const float *db = vdiff + seq * L * D, *ob = out + seq * L * D, *hib = h_init + seq * D;
+
+    float Wr[R], Wnext[R];   // Wr[jj] = W[i][reg_index(jj)]
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Wr[jj] = 0.f;
+    float dh_i = 0.f;   // gradient carried to the previous output, entry i
+
+    TileRegs<D> pk, pgo, pd, pu, ps;
+    float pb = 0.f;
+    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
+    const float *klane = kb + lrow * k.sL + 4 * lc4, *golane = gob + lrow * go.sL + 4 * lc4,
+                *dlane = db + lrow * D + 4 * lc4;
+    auto fetch = [&](int t0) {
+        if (t0 + kTile <= L) {
+            pk.template fetch<true>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<true>(golane, go.sL, t0, L, lane);
+            pd.template fetch<true>(dlane, D, t0, L, lane);
+        } else {
+            pk.template fetch<false>(klane, k.sL, t0, L, lane);
+            pgo.template fetch<false>(golane, go.sL, t0, L, lane);
+            pd.template fetch<false>(dlane, D, t0, L, lane);
+        }
+        float bs[NV4];
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            const int t = t0 + lrow + TileRegs<D>::kRowsPerLoad * x;
+            bs[x] = bb[(int64_t)min(t, L - 1) * beta.sL];
+            // row t of the delayed output is out[t-1], or the initial state for t = 0
+            const float *src = t == 0 ? hib + 4 * lc4 : ob + (int64_t)(min(t, L) - 1) * D + 4 * lc4;
+            ps.r[x] = *reinterpret_cast<const float4 *>(src);
+        }
+        pu = pd;
+        pu.scale_rows(bs);
+        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
+    };
+    auto commit = [&](int it) {
+        const int slot = it & 3;
+        pk.commit(M.k[slot], lane);
+        pu.commit(M.u[slot], lane);
+        pd.commit(M.d[slot], lane);
+        M.b[slot][per] = pb;
+        pgo.commit(M.go[it & 1], lane);
+        // softmax of each row of the delayed output, off the sequential path
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {
+            float4 &r = ps.r[x];
+            const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
+            r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
+            const float inv = fast_div(1.f, row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum()));
+            r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
+        }
+        ps.commit(M.s[slot], lane);
+    };
+    auto fetch_state = [&](int c) {
+        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
+    };
+    float *gz_rows = gz + seq * L * D;
+    auto load_ops = [&](RnnBwdOpsT<D> &o, int it, int tt) {
+        const int slot = it & 3, off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) o.u[p] = M.u[slot][off + 16 * p + per];
+        o.go_i = M.go[it & 1][off + i];
+        o.s_i = M.s[slot][off + i];
+        o.k_i = M.k[slot][off + i];
+    };
+    auto compute = [&](const RnnBwdOpsT<D> &o, float *hand, int tt) {
+        const float g_i = dh_i + o.go_i;                      // gradient of h_t = grad_z
+        float g[NP];
+        to_periodic<D>(g_i, g, lane);
+        // gradient of s_t = W_t g, through the softmax to h_{t-1}
+        const float ds_i = group_sum<S>(dot_rot<D>(Wr, g));
+        const float dot = across_groups<S>(ds_i * o.s_i, OpSum());
+        dh_i = o.s_i * (ds_i - dot);
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                   // W_{t-1}
+        hand[tt * D + i] = g_i;
+    };
+
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch((ntile - 1) * kTile);
+    commit(ntile - 1);
+    fetch_state(nchunk - 1);
+    if (ntile > 1) fetch((ntile - 2) * kTile);
+    __syncthreads();
+    tri_rounds<0>(ntile, [&](int it) {
+        const int t0 = it * kTile;
+        const int nst = min(kTile, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
+        }
+        if (it >= 1) commit(it - 1);
+        if (it + 1 < ntile) flush_tile<D>(M.g[(it + 1) % 3], gz_rows, t0 + kTile, L, lane);
+        if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
+        if (it >= 2) fetch(t0 - 2 * kTile);
+        float *hand = M.g[it % 3];
+        if (nst == kTile) {
+            RnnBwdOpsT<D> ring[2];
+            load_ops(ring[(kTile - 1) & 1], it, kTile - 1);
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], it, tt - 1);
+                compute(ring[tt & 1], hand, tt);
+            }
+        } else {  // ragged last tile (first in reverse): not pipelined
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                RnnBwdOpsT<D> o;
+                load_ops(o, it, tt);
+                compute(o, hand, tt);
+            }
+        }
+    });
+    flush_tile<D>(M.g[0], gz_rows, 0, L, lane);
+}
+
+template <int D>
+__device__ __forceinline__ void rnn_bwd_tri_a(RnnTriLds<D> &M, float *__restrict__ gv,
+                                              float *__restrict__ gbeta, int L, int64_t seq, int lane) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
+    const int i = lane / S, per = lane % 16;
+    float Gc[R];   // Gc[jj] = G[reg_index(jj)][i]
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Gc[jj] = 0.f;
+    float *gv_rows = gv + seq * L * D;
+    auto flush = [&](int ty) {   // what the work on tile ty left in LDS
+        const int t0 = ty * kTile, nst = min(kTile, L - t0);
+#pragma unroll
+        for (int x = 0; x < NV4; x++) {   // grad_v = -a
+            const int f = lane + kWave * x, rw = f / (D / 4), c4 = f % (D / 4);
+            const float4 a4 = *reinterpret_cast<const float4 *>(M.a[ty & 1] + 4 * f);
+            if (t0 + rw < L)
+                *reinterpret_cast<float4 *>(gv_rows + (int64_t)(t0 + rw) * D + 4 * c4) =
+                    make_float4(-a4.x, -a4.y, -a4.z, -a4.w);
+        }
+        const int tt = lane / 4, part = lane % 4;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < D / 4; j += 4) {
+            const float4 x = *reinterpret_cast<const float4 *>(&M.pd[tt * D + part * (D / 4) + j]);
+            acc += (x.x + x.y) + (x.z + x.w);
+        }
+        acc = group_sum<4>(acc);
+        if (tt < nst) gbeta[seq * L + t0 + tt] = acc;
+    };
+    auto load_ops = [&](RnnBwdOpsA<D> &o, int ty, int tt) {
+        const int slot = ty & 3, off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.s[p] = M.s[slot][off + 16 * p + per];
+            o.k[p] = M.k[slot][off + 16 * p + per];
+        }
+        o.g_i = M.g[ty % 3][off + i];
+        o.d_i = M.d[slot][off + i];
+        o.b = M.b[slot][tt];
+    };
+    auto compute = [&](const RnnBwdOpsA<D> &o, float *hand, int tt) {
+        // G' = G + s (x) g;  r = G'^T k
+        rank1_rot<D>(Gc, o.s, o.g_i);
+        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
+        const float a_i = -(o.b * r_i);                       // gradient w.r.t. v_old; grad_v = -a
+        M.pd[tt * D + i] = r_i * o.d_i;
+        rank1_rot<D>(Gc, o.k, a_i);
+        hand[tt * D + i] = pinned(a_i);
+    };
+    const int ntile = (L + kTile - 1) / kTile;
+    __syncthreads();
+    tri_rounds<1>(ntile, [&](int ty) {
+        const int nst = min(kTile, L - ty * kTile);
+        if (ty + 1 < ntile) flush(ty + 1);
+        float *hand = M.a[ty & 1];
+        if (nst == kTile) {
+            RnnBwdOpsA<D> ring[2];
+            load_ops(ring[(kTile - 1) & 1], ty, kTile - 1);
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], ty, tt - 1);
+                compute(ring[tt & 1], hand, tt);
+            }
+        } else {
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                RnnBwdOpsA<D> o;
+                load_ops(o, ty, tt);
+                compute(o, hand, tt);
+            }
+        }
+    });
+    flush(0);
+}
+
+template <int D>
+__device__ __forceinline__ void rnn_bwd_tri_y(RnnTriLds<D> &M, const float *__restrict__ ckpt,
+                                              float *__restrict__ gk, int L, int chunk, int nchunk,
+                                              int64_t seq, int lane) {
+    using G = Geo<D>;
+    constexpr int S = G::S, R = G::R, NP = G::NP;
+    const int i = lane / S, per = lane % 16;
+    // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)]
+    float Wr[R], Gr[R], Wnext[R];
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) Gr[jj] = Wr[jj] = 0.f;
+    auto fetch_state = [&](int c) {
+        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
+#pragma unroll
+        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
+    };
+    float *gk_rows = gk + seq * L * D;
+    auto load_ops = [&](RnnBwdOpsY<D> &o, int ty, int tt) {
+        const int slot = ty & 3, off = tt * D;
+#pragma unroll
+        for (int p = 0; p < NP; p++) {
+            o.g[p] = M.g[ty % 3][off + 16 * p + per];
+            o.a[p] = M.a[ty & 1][off + 16 * p + per];
+            o.u[p] = M.u[slot][off + 16 * p + per];
+        }
+        o.s_i = M.s[slot][off + i];
+        o.k_i = M.k[slot][off + i];
+    };
+    auto compute = [&](const RnnBwdOpsY<D> &o, int tt) {
+        rank1_rot<D>(Gr, o.g, o.s_i);                         // G' = G + s (x) g
+        float gk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
+        rank1_rot<D, true>(Wr, o.u, o.k_i);                   // W_{t-1}
+        gk_i = group_sum<S>(dot_rot<D>(Wr, o.a, gk_i));
+        rank1_rot<D>(Gr, o.a, o.k_i);
+        M.gk[tt * D + i] = pinned(gk_i);
+    };
+    const int ntile = (L + kTile - 1) / kTile;
+    fetch_state(nchunk - 1);
+    __syncthreads();
+    tri_rounds<2>(ntile, [&](int ty) {
+        const int t0 = ty * kTile;
+        const int nst = min(kTile, L - t0);
+        const int t_end = t0 + nst;
+        if (t_end % chunk == 0 || t_end == L) {
+#pragma unroll
+            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
+        }
+        if (ty + 1 < ntile) flush_tile<D>(M.gk, gk_rows, t0 + kTile, L, lane);
+        if (t0 % chunk == 0 && ty >= 1) fetch_state(t0 / chunk - 1);
+        if (nst == kTile) {
+            RnnBwdOpsY<D> ring[2];
+            load_ops(ring[(kTile - 1) & 1], ty, kTile - 1);
+#pragma unroll
+            for (int tt = kTile - 1; tt >= 0; tt--) {
+                if (tt > 0) load_ops(ring[(tt - 1) & 1], ty, tt - 1);
+                compute(ring[tt & 1], tt);
+            }
+        } else {
+            for (int tt = nst - 1; tt >= 0; tt--) {
+                RnnBwdOpsY<D> o;
+                load_ops(o, ty, tt);
+                compute(o, tt);
+            }
+        }
+    });
+    flush_tile<D>(M.gk, gk_rows, 0, L, lane);
+}
+
+// Waves 0..5 of a workgroup, which holds two sequences: X, X, Y, Y, A, A; the two A waves are the
+// fifth and sixth and share SIMDs with the two X waves (the lighter roles), each Y has one to itself.
+template <int D>
+__global__ __launch_bounds__(kWave * 6) void k_rnn_bwd_tri(
+    fwp_view k, fwp_view beta, const float *__restrict__ vdiff, const float *__restrict__ out,
+    const float *__restrict__ h_init, fwp_view go, const float *__restrict__ ckpt,
+    float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv,
+    float *__restrict__ gbeta, int H, int L, int chunk, int nchunk, int nseq) {
+    extern __shared__ __align__(16) unsigned char tri_lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+    const int lane = threadIdx.x % kWave;
+    const int role = wave >> 1;                                   // 0: X, 1: Y, 2: A
+    const int which = role == 2 ? 1 - (wave & 1) : wave & 1;      // A of the other X's sequence
+    const int64_t seq = (int64_t)blockIdx.x * 2 + which;
+    RnnTriLds<D> &M = reinterpret_cast<RnnTriLds<D> *>(tri_lds)[which];
+    if (seq >= nseq) {   // odd number of sequences: the spare waves only keep the barriers' count
+        const int ntile = (L + kTile - 1) / kTile;
+        for (int j = 0; j < ntile + 3; j++) __syncthreads();
+        return;
+    }
+    if (role == 0) rnn_bwd_tri_x<D>(M, k, beta, vdiff, out, h_init, go, ckpt, gz, H, L, chunk, nchunk, seq, lane);
+    else if (role == 1) rnn_bwd_tri_y<D>(M, ckpt, gk, L, chunk, nchunk, seq, lane);
+    else rnn_bwd_tri_a<D>(M, gv, gbeta, L, seq, lane);
+}
+
 }  // namespace
 
 // up to this many sequences (one wave on each SIMD) the forward pass puts two waves on each
 constexpr int kFwdPairMaxSeq = 512;
 
-// The backward pass puts two waves on a sequence, except from 513 to 1024 sequences: there the
-// one-wave kernel has a SIMD for each wave and is as fast or a little faster (768 sequences of D = 32
-// over 256 steps: 130 against 136 us; 512: 131 against 101 us; 1280: 268 against 217 us).
-inline bool rnn_bwd_pair(int nseq) { return nseq <= 512 || nseq > 1024; }
+// Up to this many sequences (one workgroup of two sequences on each CU) the backward pass puts three
+// waves on each; beyond it two, except from 513 to 1024 sequences: there the one-wave kernel has a
+// SIMD for each wave and is as fast or a little faster (D = 32 over 256 steps, 512 sequences: one wave
+// 131 us, two 98 us, three 79 us; 768: one 130, two 136 us; 1280: one 268, two 217 us).
+constexpr int kTriMaxSeq = 512;
+inline bool rnn_bwd_pair(int nseq) { return nseq > 1024; }
 
 bool reg_rnn_supported(int D) { return D == 16 || D == 32; }
 
@@ -915,18 +1255,20 @@ int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                 const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
                 float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
-    if (rnn_bwd_pair(nseq)) {
-        auto launch = [&](auto kernel, size_t lds) {
-            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
-                return (int)e;
-            hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, k, beta, vdiff, out,
-                               h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
-            return (int)hipGetLastError();
-        };
-        return D == 16 ? launch(k_rnn_bwd_pair<16>, 2 * sizeof(RnnPairLds<16>))
-                       : launch(k_rnn_bwd_pair<32>, 2 * sizeof(RnnPairLds<32>));
-    }
+    auto launch_on = [&](auto kernel, int waves, size_t lds) {
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+            return (int)e;
+        hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * waves), lds, s, k, beta, vdiff, out, h_init,
+                           go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
+        return (int)hipGetLastError();
+    };
+    if (nseq <= kTriMaxSeq)
+        return D == 16 ? launch_on(k_rnn_bwd_tri<16>, 6, 2 * sizeof(RnnTriLds<16>))
+                       : launch_on(k_rnn_bwd_tri<32>, 6, 2 * sizeof(RnnTriLds<32>));
+    if (rnn_bwd_pair(nseq))
+        return D == 16 ? launch_on(k_rnn_bwd_pair<16>, 4, 2 * sizeof(RnnPairLds<16>))
+                       : launch_on(k_rnn_bwd_pair<32>, 4, 2 * sizeof(RnnPairLds<32>));
     if (D == 16)
         hipLaunchKernelGGL((k_rnn_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, k,
                            beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,

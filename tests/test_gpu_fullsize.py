@@ -195,22 +195,22 @@ def test_rnn_full_size_properties(fwp):
 
 
 @pytest.mark.parametrize("D,T", [(32, 100), (16, 70)])
-def test_rnn_backward_one_and_two_waves_per_sequence(fwp, D, T):
-    """The backward pass of the Delta RNN puts two waves on a sequence up to 512 sequences and one
-    from there to 1024: 1024 sequences in one call against the same sequences in two calls of
-    512 and in calls of 511 (an odd count leaves a workgroup with one sequence) and 513.
-    Tolerance: |a - b| <= 1e-4 + 1e-3 |b|."""
-    z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(7, 128, 8, T, D, dtype=np.float32, w0=True))
+def test_rnn_one_two_and_three_waves_per_sequence(fwp, D, T):
+    """The Delta RNN puts several waves on a sequence while there are SIMDs to spare: forward two up
+    to 512 sequences, backward three up to 512, one from 513 to 1024, two beyond.  1100 sequences in
+    one call against the same sequences in calls of 600 and 500 and of 511 (an odd count leaves a
+    workgroup with one sequence) and 589.  Tolerance: |a - b| <= 1e-4 + 1e-3 |b|."""
+    NS = 1100
+    z, k, v, W0, beta, h0, go = (dev(a) for a in rnn_inputs(7, NS, 1, T, D, dtype=np.float32, w0=True))
 
-    def grads(sl):
-        fn = lambda t: fwp.fast_rnn_v2(t[0], t[1], t[2], W0.reshape(-1, 1, D, D)[sl].clone(), t[3],
-                                       h0.reshape(-1, 1, 1, D)[sl].clone())
-        flat = [x.reshape(-1, 1, T, x.shape[-1])[sl] for x in (z, k, v, beta)]
-        return grads_of(fn, flat, go.reshape(-1, 1, T, D)[sl])[1]
+    def run(sl):
+        ts = [x[sl].clone().requires_grad_(True) for x in (z, k, v, beta)]
+        out = fwp.fast_rnn_v2(ts[0], ts[1], ts[2], W0[sl].clone(), ts[3], h0[sl].clone())
+        return (out.detach(), *torch.autograd.grad(out, ts, go[sl]))
 
-    whole = grads(slice(0, 1024))
-    for cut in (512, 511):
-        parts = [grads(slice(0, cut)), grads(slice(cut, 1024))]
+    whole = run(slice(0, NS))
+    for cut in (600, 511):
+        parts = [run(slice(0, cut)), run(slice(cut, NS))]
         for i, w in enumerate(whole):
             got = torch.cat([parts[0][i], parts[1][i]], 0)
             assert torch.isfinite(got).all()
