@@ -27,8 +27,8 @@ PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
 # WRITE_SIZE (KiB per dispatch; FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by what the same counters read
 # for a 2 GiB device-to-device copy, `--copy-calibration`).
 MEASURED_TRAFFIC = {'delta': {'fwd': 84400000.0, 'bwd': 105900000.0}, 'delta_lm': {'fwd': 204700000.0, 'bwd': 271100000.0},
-                    'sum': {'fwd': 55100000.0, 'bwd': 91500000.0}, 'rnn': {'fwd': 97400000.0, 'bwd': 127900000.0}, 'rec': {'fwd': 131900000.0, 'bwd': 150700000.0},
-                    'lstm': {'fwd': 325200000.0, 'bwd': 382300000.0}}
+                    'sum': {'fwd': 55100000.0, 'bwd': 91500000.0}, 'rnn': {'fwd': 97500000.0, 'bwd': 127500000.0}, 'rec': {'fwd': 131900000.0, 'bwd': 150700000.0},
+                    'lstm': {'fwd': 325300000.0, 'bwd': 382500000.0}}
 
 # name -> (B, H, T, D, algorithmic flops per token-head = c*D^2, fwd bytes, bwd bytes per token-head)
 WORKLOADS = {
