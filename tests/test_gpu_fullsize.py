@@ -118,7 +118,7 @@ def test_sum_widest_states_blocked_against_generic_kernels(fwp, B, H, T, E, M):
         assert torch.allclose(x, y, atol=1e-4, rtol=1e-3), (i, float((x - y).abs().max()))
 
 
-@pytest.mark.parametrize("E,M", [(64, 32), (96, 16), (16, 64), (64, 64)])
+@pytest.mark.parametrize("E,M", [(64, 32), (96, 16), (16, 64), (64, 64), (32, 64), (96, 32)])
 def test_delta_rectangular_states_at_full_occupancy(fwp, E, M):
     """1024 sequences (several waves on every SIMD) of the rectangular state shapes: a split on a
     block boundary with the state carried over is the same computation bit for bit, two runs give
