@@ -469,8 +469,12 @@ __device__ __forceinline__ void rec_bwd_pair_y(RecPairLds<D> &M, float *__restri
         }
 }
 
-template <int D>
-__global__ __launch_bounds__(kWave * 4) void k_rec_bwd_pair(
+// NS sequences to a workgroup: waves 0 .. NS-1 carry the steps, waves NS .. 2 NS - 1 the sums.  The waves
+// of a workgroup go to the SIMDs in turn; with four sequences each SIMD of the CU gets one wave of
+// either kind, whereas two workgroups of two sequences on a CU both put their heavy waves on the same
+// two SIMDs.
+template <int D, int NS>
+__global__ __launch_bounds__(kWave * 2 * NS) void k_rec_bwd_pair(
     const float *__restrict__ q_act, const float *__restrict__ k_act,
     const float *__restrict__ beta_act, const float *__restrict__ vdiff,
     const float *__restrict__ out, const float *__restrict__ h_init, fwp_view go,
@@ -481,14 +485,14 @@ __global__ __launch_bounds__(kWave * 4) void k_rec_bwd_pair(
     extern __shared__ __align__(16) unsigned char pair_lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
-    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
-    RecPairLds<D> &M = reinterpret_cast<RecPairLds<D> *>(pair_lds)[wave & 1];
-    if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
+    const int64_t seq = (int64_t)blockIdx.x * NS + wave % NS;
+    RecPairLds<D> &M = reinterpret_cast<RecPairLds<D> *>(pair_lds)[wave % NS];
+    if (seq >= nseq) {   // the last workgroup's spare waves only keep the barriers' count
         const int ntile = (L + kTile - 1) / kTile;
         for (int it = ntile; it >= 0; it--) __syncthreads();
         return;
     }
-    if (wave < 2)
+    if (wave < NS)
         rec_bwd_pair_x<D>(M, q_act, k_act, beta_act, vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx, gkx, gvx,
                           gbx, H, L, chunk, nchunk, seq, lane);
     else
@@ -509,9 +513,17 @@ int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float 
                            qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
                            ckpt, H, L, chunk, nchunk, nseq);
     else
-        hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
-                           qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
-                           ckpt, H, L, chunk, nchunk, nseq);
+        // Two sequences to a workgroup, except from 513 to 1024: two-wave workgroups are placed on the SIMDs
+        // unevenly once a CU holds more than one (768 sequences of 256 steps: 219 us, four to a workgroup
+        // 166 us); four to a workgroup take 84 KB of LDS, one workgroup to a CU.
+        if (nseq > 512 && nseq <= 1024)
+            hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
+                               qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
+                               ckpt, H, L, chunk, nchunk, nseq);
+        else
+            hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
+                               qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
+                               ckpt, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
 
@@ -521,17 +533,21 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
                 float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
                 int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
-    auto launch = [&](auto kernel, size_t lds) {
+    auto launch = [&](auto kernel, int ns, size_t lds) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
             return (int)e;
-        hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, q_act, k_act, beta_act, vdiff,
-                           out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx, gkx, gvx, gbx, workspace, H, L, chunk,
+        hipLaunchKernelGGL(kernel, dim3((nseq + ns - 1) / ns), dim3(kWave * 2 * ns), lds, s, q_act, k_act, beta_act,
+                           vdiff, out, h_init, go, Rq, Rk, Rv, rb, ckpt, gqx, gkx, gvx, gbx, workspace, H, L, chunk,
                            nchunk, nseq);
         return (int)hipGetLastError();
     };
-    return D == 16 ? launch(k_rec_bwd_pair<16>, 2 * sizeof(RecPairLds<16>))
-                   : launch(k_rec_bwd_pair<32>, 2 * sizeof(RecPairLds<32>));
+    // up to 512 sequences two to a workgroup (one workgroup on each CU), beyond that four
+    if (nseq <= 512)
+        return D == 16 ? launch(k_rec_bwd_pair<16, 2>, 2, 2 * sizeof(RecPairLds<16>))
+                       : launch(k_rec_bwd_pair<32, 2>, 2, 2 * sizeof(RecPairLds<32>));
+    return D == 16 ? launch(k_rec_bwd_pair<16, 4>, 4, 4 * sizeof(RecPairLds<16>))
+                   : launch(k_rec_bwd_pair<32, 4>, 4, 4 * sizeof(RecPairLds<32>));
 }
 
 }  // namespace fwp

@@ -217,6 +217,36 @@ def test_rnn_one_two_and_three_waves_per_sequence(fwp, D, T):
             assert torch.allclose(got, w, atol=1e-4, rtol=1e-3), (cut, i, float((got - w).abs().max()))
 
 
+@pytest.mark.parametrize("D,T", [(32, 70), (16, 50)])
+def test_rec_workgroups_of_two_and_of_four_sequences(fwp, D, T):
+    """The Recurrent Delta Net's kernels put two sequences in a workgroup up to 512 sequences and four
+    beyond (forward: from 513 to 1024): 1100 sequences in one call against the same sequences in
+    calls of 600 and 500 and of 511 (an odd count leaves a workgroup with spare waves) and 589.  The
+    gradients of the recurrent weights are sums over the sequences, so the parts' are added.
+    Tolerance: |a - b| <= 1e-4 + 1e-3 |b| (1e-3 + 1e-3 |b| on those sums of 1100 terms)."""
+    NS = 1100
+    *x, go = (dev(a) for a in rec_inputs(9, NS, 1, T, D, dtype=np.float32, w0=True))
+    qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0 = x
+
+    def run(sl):
+        ts = [t[sl].clone().requires_grad_(True) for t in (qx, kx, vx, bx)]
+        rs = [t.clone().requires_grad_(True) for t in (R_q, R_k, R_v, r_b)]
+        out = fwp.rec_update_fwm_tanh(*ts, *rs, W0[sl].clone(), h0[sl].clone())
+        g = torch.autograd.grad(out, [*ts, *rs], go[sl])
+        return (out.detach(), *g[:4]), g[4:]
+
+    whole, whole_r = run(slice(0, NS))
+    for cut in (600, 511):
+        (a, ar), (b, br) = run(slice(0, cut)), run(slice(cut, NS))
+        for i, w in enumerate(whole):
+            got = torch.cat([a[i], b[i]], 0)
+            assert torch.isfinite(got).all()
+            assert torch.allclose(got, w, atol=1e-4, rtol=1e-3), (cut, i, float((got - w).abs().max()))
+        for i, w in enumerate(whole_r):
+            got = ar[i] + br[i]
+            assert torch.allclose(got, w, atol=1e-3, rtol=1e-3), (cut, "R", i, float((got - w).abs().max()))
+
+
 def test_rec_full_size_properties(fwp):
     *x, go = (dev(a) for a in rec_inputs(2, 64, 8, 256, 32, dtype=np.float32))
     qx, kx, vx, bx, R_q, R_k, R_v, r_b, W0, h0 = x
