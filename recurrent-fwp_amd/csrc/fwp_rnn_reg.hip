@@ -343,8 +343,11 @@ __device__ __forceinline__ void rnn_fwd_pair_m(RnnFwdPairLds<D> &M, fwp_view z, 
     if (sl == 0) hstate[seq * D + col] = hcur;
 }
 
-template <int D>
-__global__ __launch_bounds__(kWave * 4) void k_rnn_fwd_pair(fwp_view z, fwp_view k, fwp_view v, fwp_view beta,
+// NS sequences to a workgroup: waves 0 .. NS-1 are the M waves, NS .. 2 NS - 1 the H waves.  The waves of
+// a workgroup go to the SIMDs in turn; with four sequences each SIMD of the CU gets one wave of either
+// kind, whereas two workgroups of two sequences on a CU both put their M waves on the same two SIMDs.
+template <int D, int NS>
+__global__ __launch_bounds__(kWave * 2 * NS) void k_rnn_fwd_pair(fwp_view z, fwp_view k, fwp_view v, fwp_view beta,
                                                             float *__restrict__ W, float *__restrict__ hstate,
                                                             float *__restrict__ out, float *__restrict__ vdiff,
                                                             float *__restrict__ ckpt, int H, int L, int chunk,
@@ -352,234 +355,29 @@ __global__ __launch_bounds__(kWave * 4) void k_rnn_fwd_pair(fwp_view z, fwp_view
     extern __shared__ __align__(16) unsigned char pair_lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
-    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
-    RnnFwdPairLds<D> &M = reinterpret_cast<RnnFwdPairLds<D> *>(pair_lds)[wave & 1];
+    const int64_t seq = (int64_t)blockIdx.x * NS + wave % NS;
+    RnnFwdPairLds<D> &M = reinterpret_cast<RnnFwdPairLds<D> *>(pair_lds)[wave % NS];
     if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
         const int ntile = (L + kTile - 1) / kTile;
         for (int it = ntile; it >= 0; it--) __syncthreads();
         return;
     }
-    if (wave < 2) rnn_fwd_pair_m<D>(M, z, W, hstate, out, ckpt, H, L, chunk, nchunk, seq, lane);
+    if (wave < NS) rnn_fwd_pair_m<D>(M, z, W, hstate, out, ckpt, H, L, chunk, nchunk, seq, lane);
     else rnn_fwd_pair_h<D>(M, k, v, beta, W, vdiff, H, L, seq, lane);
-}
-
-// ----------------------------------------------------------------- backward
-
-template <int D>
-struct RnnBwdOps {
-    float k[Geo<D>::NP], u[Geo<D>::NP], s[Geo<D>::NP];
-    float go_i, s_i, k_i, d_i, b;
-};
-
-template <int D, int RING, int PF, int WPB>
-__global__ __launch_bounds__(kWave * WPB) void k_rnn_bwd_reg(
-    fwp_view k, fwp_view beta, const float *__restrict__ vdiff, const float *__restrict__ out,
-    const float *__restrict__ h_init, fwp_view go, const float *__restrict__ ckpt,
-    float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv,
-    float *__restrict__ gbeta, int H, int L, int chunk, int nchunk, int nseq) {
-    using G = Geo<D>;
-    constexpr int S = G::S, R = G::R, NP = G::NP, NV4 = G::NV4;
-    static_assert(kTile % RING == 0 && PF < RING, "ring must divide the tile");
-    __shared__ __align__(16) float sk_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sgo_[WPB][2][kTile * D];
-    __shared__ __align__(16) float sd_[WPB][2][kTile * D];
-    __shared__ __align__(16) float su_[WPB][2][kTile * D];
-    __shared__ __align__(16) float ss_[WPB][2][kTile * D];   // softmax of the delayed output
-    __shared__ __align__(16) float sb_[WPB][2][kTile];
-    __shared__ __align__(16) float spd_[WPB][kTile * D];
-    __shared__ __align__(16) float sgrad_[WPB][3][kTile * D + 16];   // staged gz, gk, gv tiles
-
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: lets the compiler branch on it in scalar code
-    const int lane = threadIdx.x % kWave, i = lane / S, sl = lane % S, per = lane % 16;
-    const int64_t seq = (int64_t)blockIdx.x * WPB + wave;
-    if (seq >= nseq) return;
-    const int n = (int)(seq / H), h = (int)(seq % H);
-    auto &sk = sk_[wave];
-    auto &sgo = sgo_[wave];
-    auto &sd = sd_[wave];
-    auto &su = su_[wave];
-    auto &ss = ss_[wave];
-    auto &sb = sb_[wave];
-    auto &spd = spd_[wave];
-    auto &sgrad = sgrad_[wave];
-    const float *kb = row(k, n, h, 0), *gob = row(go, n, h, 0), *bb = row(beta, n, h, 0);
-    const float *db = vdiff + seq * L * D, *ob = out + seq * L * D, *hib = h_init + seq * D;
-
-    // Wr[jj] = W[i][reg_index(jj)], Gr[jj] = G[i][reg_index(jj)], Gc[jj] = G[reg_index(jj)][i]
-    float Wr[R], Gr[R], Gc[R], Wnext[R];
-#pragma unroll
-    for (int jj = 0; jj < R; jj++) Gr[jj] = Gc[jj] = Wr[jj] = 0.f;
-    float dh_i = 0.f;   // gradient carried to the previous output, entry i
-
-    TileRegs<D> pk, pgo, pd, pu, ps;
-    float pb = 0.f;
-    const int lrow = lane / (D / 4), lc4 = lane % (D / 4);
-    const float *klane = kb + lrow * k.sL + 4 * lc4, *golane = gob + lrow * go.sL + 4 * lc4,
-                *dlane = db + lrow * D + 4 * lc4;
-    auto fetch = [&](int t0) {
-        if (t0 + kTile <= L) {
-            pk.template fetch<true>(klane, k.sL, t0, L, lane);
-            pgo.template fetch<true>(golane, go.sL, t0, L, lane);
-            pd.template fetch<true>(dlane, D, t0, L, lane);
-        } else {
-            pk.template fetch<false>(klane, k.sL, t0, L, lane);
-            pgo.template fetch<false>(golane, go.sL, t0, L, lane);
-            pd.template fetch<false>(dlane, D, t0, L, lane);
-        }
-        float bs[NV4];
-#pragma unroll
-        for (int x = 0; x < NV4; x++) {
-            const int t = t0 + lrow + TileRegs<D>::kRowsPerLoad * x;
-            bs[x] = bb[(int64_t)min(t, L - 1) * beta.sL];
-            // row t of the delayed output is out[t-1], or the initial state for t = 0
-            const float *src = t == 0 ? hib + 4 * lc4 : ob + (int64_t)(min(t, L) - 1) * D + 4 * lc4;
-            ps.r[x] = *reinterpret_cast<const float4 *>(src);
-        }
-        pu = pd;
-        pu.scale_rows(bs);
-        pb = bb[(int64_t)min(t0 + per, L - 1) * beta.sL];
-    };
-    auto commit = [&](int buf) {
-        pk.commit(sk[buf], lane);
-        pgo.commit(sgo[buf], lane);
-        pd.commit(sd[buf], lane);
-        pu.commit(su[buf], lane);
-        sb[buf][per] = pb;
-        // softmax of each row of the delayed output, off the sequential path
-#pragma unroll
-        for (int x = 0; x < NV4; x++) {
-            float4 &r = ps.r[x];
-            const float mx = row_reduce<D>(fmaxf(fmaxf(r.x, r.y), fmaxf(r.z, r.w)), OpMax());
-            r.x = __expf(r.x - mx); r.y = __expf(r.y - mx); r.z = __expf(r.z - mx); r.w = __expf(r.w - mx);
-            const float inv = fast_div(1.f, row_reduce<D>((r.x + r.y) + (r.z + r.w), OpSum()));
-            r.x *= inv; r.y *= inv; r.z *= inv; r.w *= inv;
-        }
-        ps.commit(ss[buf], lane);
-    };
-    auto fetch_state = [&](int c) {
-        const float *src = ckpt + ((seq * nchunk + c) * D + i) * D;
-#pragma unroll
-        for (int jj = 0; jj < R; jj++) Wnext[jj] = src[reg_index<D>(lane, jj)];
-    };
-
-    // S = 4: s=0 -> gz, s=1 -> gk, s=2,3 -> gv.   S = 2: s=0 -> gz, s=1 -> gk, and a second write for gv.
-    float *dst1 = sgrad[sl == 0 ? 0 : (sl == 1 ? 1 : 2)] + i;
-    float *dst2 = sgrad[2] + i;
-    float *gz_rows = gz + seq * L * D, *gk_rows = gk + seq * L * D, *gv_rows = gv + seq * L * D;
-
-    auto load_ops = [&](RnnBwdOps<D> &o, int buf, int tt) {
-        const int off = tt * D;
-#pragma unroll
-        for (int p = 0; p < NP; p++) {
-            o.k[p] = sk[buf][off + 16 * p + per];
-            o.u[p] = su[buf][off + 16 * p + per];
-            o.s[p] = ss[buf][off + 16 * p + per];
-        }
-        o.go_i = sgo[buf][off + i];
-        o.s_i = ss[buf][off + i];
-        o.k_i = sk[buf][off + i];
-        o.d_i = sd[buf][off + i];
-        o.b = sb[buf][tt];
-    };
-    auto compute = [&](const RnnBwdOps<D> &o, int tt) {
-        const float g_i = dh_i + o.go_i;                      // gradient of h_t = grad_z
-        float g[NP], a[NP];
-        to_periodic<D>(g_i, g, lane);
-        // G' = G + s (x) g (both layouts);  r = G'^T k
-        rank1_rot<D>(Gc, o.s, g_i);
-        const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
-        const float gv_i = o.b * r_i;
-        const float a_i = -gv_i;                              // gradient w.r.t. v_old
-        to_periodic<D>(a_i, a, lane);
-        spd[tt * D + i] = r_i * o.d_i;
-        rank1_rot<D>(Gr, g, o.s_i);
-        // gradient of s_t = W_t g, through the softmax to h_{t-1}
-        const float ds_i = group_sum<S>(dot_rot<D>(Wr, g));
-        const float dot = across_groups<S>(ds_i * o.s_i, OpSum());
-        dh_i = o.s_i * (ds_i - dot);
-        rank1_rot<D, true>(Wr, o.u, o.k_i);                   // W_{t-1}
-        rank1_rot<D>(Gc, o.k, a_i);
-        float gk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
-        gk_i = group_sum<S>(dot_rot<D>(Wr, a, gk_i));
-        rank1_rot<D>(Gr, a, o.k_i);
-        const float o_z = pinned(g_i), o_k = pinned(gk_i), o_v = pinned(gv_i);
-        if constexpr (S == 4) {
-            dst1[tt * D] = sl == 0 ? o_z : (sl == 1 ? o_k : o_v);
-        } else {
-            dst1[tt * D] = sl == 0 ? o_z : o_k;
-            dst2[tt * D] = o_v;
-        }
-    };
-    auto flush = [&](int t0, int nst) {
-        flush_tile<D>(sgrad[0], gz_rows, t0, L, lane);
-        flush_tile<D>(sgrad[1], gk_rows, t0, L, lane);
-        flush_tile<D>(sgrad[2], gv_rows, t0, L, lane);
-        const int tt = lane / 4, part = lane % 4;
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < D / 4; j += 4) {
-            const float4 x = *reinterpret_cast<const float4 *>(&spd[tt * D + part * (D / 4) + j]);
-            acc += (x.x + x.y) + (x.z + x.w);
-        }
-        acc = group_sum<4>(acc);
-        if (tt < nst) gbeta[seq * L + t0 + tt] = acc;
-    };
-
-    const int ntile = (L + kTile - 1) / kTile;
-    fetch((ntile - 1) * kTile);
-    commit((ntile - 1) & 1);
-    fetch_state(nchunk - 1);
-    if (ntile > 1) fetch((ntile - 2) * kTile);
-    RnnBwdOps<D> ring[RING];
-    bool primed = false;
-
-    for (int it = ntile - 1; it >= 0; it--) {
-        const int buf = it & 1, t0 = it * kTile;
-        const int nst = min(kTile, L - t0);
-        const int t_end = t0 + nst;
-        if (t_end % chunk == 0 || t_end == L) {  // first tile (in reverse) of a chunk: re-anchor W
-#pragma unroll
-            for (int jj = 0; jj < R; jj++) Wr[jj] = Wnext[jj];
-        }
-        if (it >= 1) commit(buf ^ 1);
-        if (it + 1 < ntile) flush(t0 + kTile, min(kTile, L - t0 - kTile));
-        if (it >= 1 && t0 % chunk == 0) fetch_state(t0 / chunk - 1);
-        if (it >= 2) fetch(t0 - 2 * kTile);
-        if (nst == kTile) {
-            if (!primed) {
-#pragma unroll
-                for (int p = 0; p < PF; p++) load_ops(ring[(kTile - 1 - p) % RING], buf, kTile - 1 - p);
-                primed = true;
-            }
-#pragma unroll
-            for (int tt = kTile - 1; tt >= 0; tt--) {
-                const int nt = tt - PF;
-                if (nt >= 0) load_ops(ring[nt % RING], buf, nt);
-                else load_ops(ring[(nt + kTile) % RING], buf ^ 1, nt + kTile);
-                compute(ring[tt % RING], tt);
-            }
-        } else {  // ragged last tile (first in reverse): not pipelined
-            for (int tt = nst - 1; tt >= 0; tt--) {
-                RnnBwdOps<D> o;
-                load_ops(o, buf, tt);
-                compute(o, tt);
-            }
-        }
-    }
-    flush(0, min(kTile, L));
 }
 
 // ------------------------------------------- backward, two waves per sequence
 //
-// One wave cannot issue the backward step's instructions any faster, and up to about a thousand
-// sequences there are SIMDs with nothing to do, so the step is divided between two waves.  Wave X
+// One wave cannot issue the backward step's 180 instructions as fast as two waves on two SIMDs, or
+// on one SIMD in turn, issue a half each, so the step is divided between two waves.  Wave X
 // keeps the sequential part: the gradient of h through W and the softmax, G = dL/dW in column
 // layout for r = G^T k, with it grad_z, grad_v, grad_beta and a = dL/dv_old.  Wave Y, one tile of 16
 // steps behind, takes g = grad_z and a from LDS, keeps G in row layout and a copy of W of its own,
 // and computes grad_k = G u + W_{t-1} a.  X also loads the tiles both need (k, beta * vdiff and the
 // softmax of the delayed output) into a ring of three slots: X fills the slot of tile it - 1 while it
-// works on tile it and Y on tile it + 1.  One workgroup barrier per tile; a workgroup holds two
-// sequences, that is four waves, one for each SIMD of a CU.
+// works on tile it and Y on tile it + 1.  One workgroup barrier per tile; a workgroup holds four
+// sequences, that is eight waves X X X X Y Y Y Y, which go to the SIMDs of a CU in turn: one wave of
+// either kind on each.
 template <int D>
 struct RnnPairLds {
     float k[3][kTile * D], u[3][kTile * D], s[3][kTile * D];
@@ -855,8 +653,8 @@ __device__ __forceinline__ void rnn_bwd_pair_y(RnnPairLds<D> &M, const float *__
     }
 }
 
-template <int D>
-__global__ __launch_bounds__(kWave * 4) void k_rnn_bwd_pair(
+template <int D, int NS>   // NS sequences to a workgroup: waves 0 .. NS-1 are X, NS .. 2 NS - 1 are Y
+__global__ __launch_bounds__(kWave * 2 * NS) void k_rnn_bwd_pair(
     fwp_view k, fwp_view beta, const float *__restrict__ vdiff, const float *__restrict__ out,
     const float *__restrict__ h_init, fwp_view go, const float *__restrict__ ckpt,
     float *__restrict__ gz, float *__restrict__ gk, float *__restrict__ gv,
@@ -864,14 +662,14 @@ __global__ __launch_bounds__(kWave * 4) void k_rnn_bwd_pair(
     extern __shared__ __align__(16) unsigned char pair_lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const int lane = threadIdx.x % kWave;
-    const int64_t seq = (int64_t)blockIdx.x * 2 + (wave & 1);
-    RnnPairLds<D> &M = reinterpret_cast<RnnPairLds<D> *>(pair_lds)[wave & 1];
+    const int64_t seq = (int64_t)blockIdx.x * NS + wave % NS;
+    RnnPairLds<D> &M = reinterpret_cast<RnnPairLds<D> *>(pair_lds)[wave % NS];
     if (seq >= nseq) {   // odd number of sequences: the two spare waves only keep the barriers' count
         const int ntile = (L + kTile - 1) / kTile;
         for (int it = ntile; it >= 0; it--) __syncthreads();
         return;
     }
-    if (wave < 2)
+    if (wave < NS)
         rnn_bwd_pair_x<D>(M, k, beta, vdiff, out, h_init, go, ckpt, gz, gv, gbeta, H, L, chunk, nchunk, seq,
                           lane);
     else
@@ -1223,25 +1021,30 @@ __global__ __launch_bounds__(kWave * 6) void k_rnn_bwd_tri(
 constexpr int kFwdPairMaxSeq = 1024;
 
 // Up to this many sequences (one workgroup of two sequences on each CU) the backward pass puts three
-// waves on each; beyond it two, except from 513 to 1024 sequences: there the one-wave kernel has a
-// SIMD for each wave and is as fast or a little faster (D = 32 over 256 steps, 512 sequences: one wave
-// 131 us, two 98 us, three 79 us; 768: one 130, two 136 us; 1280: one 268, two 217 us).
+// waves on each, beyond it two, four sequences to a workgroup (D = 32 over 256 steps, 512 sequences:
+// one wave 131 us, two 98 us, three 79 us; 768: one 130, two 115 us; 1024: one 143, two 123 us;
+// 2048: one 270, two 239 us).
 constexpr int kTriMaxSeq = 512;
-inline bool rnn_bwd_pair(int nseq) { return nseq > 1024; }
-
 bool reg_rnn_supported(int D) { return D == 16 || D == 32; }
 
 int reg_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out,
                 float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
     if (nseq <= kFwdPairMaxSeq) {
-        auto launch = [&](auto kernel, size_t lds) {
-            hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * 4), lds, s, z, k, v, beta, W, h, out,
-                               vdiff, ckpt, H, L, chunk, nchunk, nseq);
+        auto launch = [&](auto kernel, int ns, size_t lds) {
+            if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
+                return (int)e;
+            hipLaunchKernelGGL(kernel, dim3((nseq + ns - 1) / ns), dim3(kWave * 2 * ns), lds, s, z, k, v, beta, W, h,
+                               out, vdiff, ckpt, H, L, chunk, nchunk, nseq);
             return (int)hipGetLastError();
         };
-        return D == 16 ? launch(k_rnn_fwd_pair<16>, 2 * sizeof(RnnFwdPairLds<16>))
-                       : launch(k_rnn_fwd_pair<32>, 2 * sizeof(RnnFwdPairLds<32>));
+        // up to 512 sequences two to a workgroup (one workgroup on each CU), beyond that four
+        if (nseq <= 512)
+            return D == 16 ? launch(k_rnn_fwd_pair<16, 2>, 2, 2 * sizeof(RnnFwdPairLds<16>))
+                           : launch(k_rnn_fwd_pair<32, 2>, 2, 2 * sizeof(RnnFwdPairLds<32>));
+        return D == 16 ? launch(k_rnn_fwd_pair<16, 4>, 4, 4 * sizeof(RnnFwdPairLds<16>))
+                       : launch(k_rnn_fwd_pair<32, 4>, 4, 4 * sizeof(RnnFwdPairLds<32>));
     }
     if (D == 16)
         hipLaunchKernelGGL((k_rnn_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, z,
@@ -1256,29 +1059,19 @@ int reg_rnn_bwd(fwp_view k, fwp_view beta, const float *vdiff, const float *out,
                 const float *h_init, fwp_view go, const float *ckpt, float *gz, float *gk,
                 float *gv, float *gbeta, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
-    auto launch_on = [&](auto kernel, int waves, size_t lds) {
+    auto launch_on = [&](auto kernel, int waves, size_t lds, int ns = 2) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds))
             return (int)e;
-        hipLaunchKernelGGL(kernel, dim3((nseq + 1) / 2), dim3(kWave * waves), lds, s, k, beta, vdiff, out, h_init,
+        hipLaunchKernelGGL(kernel, dim3((nseq + ns - 1) / ns), dim3(kWave * waves), lds, s, k, beta, vdiff, out, h_init,
                            go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk, nseq);
         return (int)hipGetLastError();
     };
     if (nseq <= kTriMaxSeq)
         return D == 16 ? launch_on(k_rnn_bwd_tri<16>, 6, 2 * sizeof(RnnTriLds<16>))
                        : launch_on(k_rnn_bwd_tri<32>, 6, 2 * sizeof(RnnTriLds<32>));
-    if (rnn_bwd_pair(nseq))
-        return D == 16 ? launch_on(k_rnn_bwd_pair<16>, 4, 2 * sizeof(RnnPairLds<16>))
-                       : launch_on(k_rnn_bwd_pair<32>, 4, 2 * sizeof(RnnPairLds<32>));
-    if (D == 16)
-        hipLaunchKernelGGL((k_rnn_bwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s, k,
-                           beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
-                           nseq);
-    else
-        hipLaunchKernelGGL((k_rnn_bwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s, k,
-                           beta, vdiff, out, h_init, go, ckpt, gz, gk, gv, gbeta, H, L, chunk, nchunk,
-                           nseq);
-    return (int)hipGetLastError();
+    return D == 16 ? launch_on(k_rnn_bwd_pair<16, 4>, 8, 4 * sizeof(RnnPairLds<16>), 4)
+                   : launch_on(k_rnn_bwd_pair<32, 4>, 8, 4 * sizeof(RnnPairLds<32>), 4);
 }
 
 }  // namespace fwp

@@ -196,8 +196,8 @@ def test_rnn_full_size_properties(fwp):
 
 @pytest.mark.parametrize("D,T", [(32, 100), (16, 70)])
 def test_rnn_one_two_and_three_waves_per_sequence(fwp, D, T):
-    """The Delta RNN puts several waves on a sequence while there are SIMDs to spare: forward two up
-    to 1024 sequences, backward three up to 512, one from 513 to 1024, two beyond.  1100 sequences in
+    """The Delta RNN puts several waves on a sequence: forward two up to 1024 sequences (two sequences
+    to a workgroup up to 512, then four), one beyond; backward three up to 512, two beyond.  1100 sequences in
     one call against the same sequences in calls of 600 and 500 and of 511 (an odd count leaves a
     workgroup with one sequence) and 589.  Tolerance: |a - b| <= 1e-4 + 1e-3 |b|."""
     NS = 1100
