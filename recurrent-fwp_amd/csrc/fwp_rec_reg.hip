@@ -508,22 +508,16 @@ int reg_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float 
                 float *q_act, float *k_act, float *beta_act, float *vdiff, float *ckpt, int N,
                 int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, nseq = N * H;
-    if (D == 16)
-        hipLaunchKernelGGL((k_rec_fwd_reg<16, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                           qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
-                           ckpt, H, L, chunk, nchunk, nseq);
-    else
-        // Two sequences to a workgroup, except from 513 to 1024: two-wave workgroups are placed on the SIMDs
-        // unevenly once a CU holds more than one (768 sequences of 256 steps: 219 us, four to a workgroup
-        // 166 us); four to a workgroup take 84 KB of LDS, one workgroup to a CU.
-        if (nseq > 512 && nseq <= 1024)
-            hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 4>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                               qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
-                               ckpt, H, L, chunk, nchunk, nseq);
-        else
-            hipLaunchKernelGGL((k_rec_fwd_reg<32, 2, 1, 2>), dim3((nseq + 1) / 2), dim3(kWave * 2), 0, s,
-                               qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,
-                               ckpt, H, L, chunk, nchunk, nseq);
+    auto launch = [&](auto kernel, int wpb) {
+        hipLaunchKernelGGL(kernel, dim3((nseq + wpb - 1) / wpb), dim3(kWave * wpb), 0, s, qx, kx, vx, bx, Rq, Rk, Rv,
+                           rb, W, h, out, q_act, k_act, beta_act, vdiff, ckpt, H, L, chunk, nchunk, nseq);
+    };
+    // D = 32: two sequences to a workgroup, except from 513 to 1024 sequences: two-wave workgroups are
+    // placed on the SIMDs unevenly once a CU holds more than one (768 sequences of 256 steps: 219 us, four
+    // to a workgroup 166 us); four to a workgroup take 84 KB of LDS, one workgroup to a CU.
+    if (D == 16) launch(k_rec_fwd_reg<16, 2, 1, 4>, 4);
+    else if (nseq > 512 && nseq <= 1024) launch(k_rec_fwd_reg<32, 2, 1, 4>, 4);
+    else launch(k_rec_fwd_reg<32, 2, 1, 2>, 2);
     return (int)hipGetLastError();
 }
 
