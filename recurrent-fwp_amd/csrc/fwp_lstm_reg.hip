@@ -123,8 +123,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_lstm_fwd_reg(LstmGates g, float
         }
     };
     auto compute = [&](const LstmFwdOps<D> &o, int tt) {
-        const float mx = across_groups<S>(hcur, OpMax());
-        const float e = __expf(hcur - mx);
+        const float e = __expf(softmax_shifted<S>(hcur));
         // the reads below use e and are scaled by 1 / sum(e) afterwards: the wave-wide sum then runs
         // beside them instead of ahead of them on the sequential path
         float s[NP];
@@ -400,8 +399,7 @@ __device__ __forceinline__ void lstm_fwd_pair_m(LstmFwdPairLds<D> &M, const Lstm
         }
     };
     auto compute = [&](const LstmFwdOpsM<D> &o, int tt) {
-        const float mx = across_groups<S>(hcur, OpMax());
-        const float e = __expf(hcur - mx);
+        const float e = __expf(softmax_shifted<S>(hcur));
         // the reads below use e and are scaled by 1 / sum(e) afterwards: the wave-wide sum then runs
         // beside them instead of ahead of them on the sequential path
         float s[NP];

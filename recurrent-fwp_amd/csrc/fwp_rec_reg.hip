@@ -125,8 +125,8 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
         const float ka = o.kx + group_sum<S>(dot_rot<D>(Rkc, y));
         const float va = o.vx + group_sum<S>(dot_rot<D>(Rvc, y));
         const float b = fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum()));
-        const float eq = __expf(qa - across_groups<S>(qa, OpMax()));
-        const float ek = __expf(ka - across_groups<S>(ka, OpMax()));
+        const float eq = __expf(softmax_shifted<S>(qa));
+        const float ek = __expf(softmax_shifted<S>(ka));
         // The softmaxes are eq / sum(eq) and ek / sum(ek); the state is read and written with eq and
         // ek and the results are scaled afterwards: the wave-wide sums then run beside the reads
         // instead of ahead of them on the sequential path.

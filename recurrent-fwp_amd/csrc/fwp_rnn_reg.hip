@@ -96,8 +96,7 @@ __global__ __launch_bounds__(kWave * WPB) void k_rnn_fwd_reg(fwp_view z, fwp_vie
         // s = softmax(h_{t-1}) = e / sum(e); independent of the delta write below, which overlaps
         // its latency.  The read is done with e and scaled afterwards: the wave-wide sum then runs
         // beside the read instead of ahead of it on the sequential path.
-        const float mx = across_groups<S>(hcur, OpMax());
-        const float e = __expf(hcur - mx);
+        const float e = __expf(softmax_shifted<S>(hcur));
         float s[NP];
         to_periodic<D>(e, s, lane);
         const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));
@@ -291,8 +290,7 @@ __device__ __forceinline__ void rnn_fwd_pair_m(RnnFwdPairLds<D> &M, fwp_view z, 
     auto compute = [&](const RnnFwdOpsM<D> &o, int tt) {
         // s = softmax(h_{t-1}) = e / sum(e); the read is done with e and scaled afterwards: the
         // wave-wide sum then runs beside the read instead of ahead of it on the sequential path
-        const float mx = across_groups<S>(hcur, OpMax());
-        const float e = __expf(hcur - mx);
+        const float e = __expf(softmax_shifted<S>(hcur));
         float s[NP];
         to_periodic<D>(e, s, lane);
         const float rsum = fast_div(1.f, across_groups<S>(e, OpSum()));

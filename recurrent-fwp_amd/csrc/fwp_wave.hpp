@@ -88,4 +88,18 @@ __device__ __forceinline__ float across_groups(float x, Op op) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), 63));
 }
 
+// x - c for a softmax over the wave, where any c with max(x) - c of a few tens at most gives the same
+// result.  The exact maximum costs a wave-wide reduction on the sequential path; the first entry is
+// there for one v_readfirstlane, and max(x) - x[0] >= 0, so nothing that matters underflows.  Only
+// when an entry lies more than kSlack above it (exp() and the sums after it could overflow; NaN
+// also lands here) is the maximum taken after all.
+template <int S>
+__device__ __forceinline__ float softmax_shifted(float x) {
+    constexpr float kSlack = 60.f;
+    const float c = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+    float y = x - c;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(y <= kSlack)) != 0, 0)) y = x - across_groups<S>(x, OpMax());
+    return y;
+}
+
 }  // namespace fwp

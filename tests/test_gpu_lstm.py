@@ -116,3 +116,24 @@ def test_lstm_backward_one_and_four_waves_per_sequence(fwp, D, T):
         got = torch.cat([parts[0][i], parts[1][i]], 0)
         assert torch.isfinite(got).all()
         assert torch.allclose(got, w, atol=1e-4, rtol=1e-3), (i, float((got - w).abs().max()))
+
+
+@pytest.mark.parametrize("N,H,L,D", [(2, 3, 30, 32), (1, 2, 40, 16), (70, 8, 12, 32)])
+def test_lstm_softmax_of_entries_far_apart(fwp, N, H, L, D):
+    """The first entry of the output far below the others at every step (its candidate value is -80
+    and its input and output gates are open): the kernels shift the softmax by the first entry and
+    take the exact maximum only when an entry lies far above it, as here.  The last shape has more
+    than 512 sequences: one wave per sequence forward."""
+    Zs, Ks, Vs, Bs, Ws, h0, c0, go = lstm_inputs(31 + D, N, H, L, D, w0=True)
+    Zs[0][..., 0], Zs[1][..., 0], Zs[2][..., 0] = 10.0, -80.0, 10.0
+    h0[..., 0], c0[..., 0] = -80.0, -80.0
+    args, diff, states, h, c = op_args(Zs, Ks, Vs, Bs, Ws, h0, c0)
+    out, cell = fwp.fast_lstm_v4(*args)
+    ref = oracle.lstm_fwd(Zs, Ks, Vs, Bs, Ws, h0, c0)
+    check("out", out, ref[0])
+    check("cell", cell, ref[1])
+    out.backward(dev(go))
+    grads = oracle.lstm_bwd(Zs, Ks, Vs, Bs, Ws, h0, c0, go)
+    for a, gate in enumerate("iuo"):
+        for j, name in enumerate("z k v beta".split()):
+            check(f"grad_{name}_{gate}", diff[a][j].grad, grads[j][a])

@@ -221,6 +221,41 @@ def test_rec(fwp, N, H, L, D, w0):
         check("grad_" + name, t.grad, r)
 
 
+@pytest.mark.parametrize("N,H,L,D", [(2, 3, 40, 32), (1, 2, 50, 16), (130, 8, 20, 32)])
+def test_rnn_softmax_of_entries_far_apart(fwp, N, H, L, D):
+    """Outputs that differ by hundreds across the D entries: the kernels shift the softmax by the
+    first entry and take the exact maximum only when an entry lies far above it, which these inputs
+    make happen at most steps (the last shape has more than 1024 sequences: one wave per sequence)."""
+    z, k, v, W0, beta, h0, go = rnn_inputs(77 + D, N, H, L, D, w0=True)
+    z, h0 = z * 60.0, h0 * 60.0
+    tz, tk, tv, tb = (dev(x, True) for x in (z, k, v, beta))
+    W, h = dev(W0), dev(h0)
+    out = fwp.fast_rnn_v2(tz, tk, tv, W, tb, h)
+    ref_out, ref_W, ref_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("z k v beta".split(), (tz, tk, tv, tb), oracle.rnn_bwd(z, k, v, W0, beta, h0, go)):
+        check("grad_" + name, t.grad, r)
+
+
+@pytest.mark.parametrize("N,H,L,D", [(2, 3, 40, 32), (1, 2, 50, 16)])
+def test_rec_softmax_of_entries_far_apart(fwp, N, H, L, D):
+    """The same for the Recurrent Delta Net: query and key inputs that differ by hundreds."""
+    *x, go = rec_inputs(78 + D, N, H, L, D, w0=True)
+    x[0], x[1] = x[0] * 60.0, x[1] * 60.0
+    ts = [dev(a, True) for a in x[:8]]
+    W, h = dev(x[8]), dev(x[9])
+    out = fwp.rec_update_fwm_tanh(*ts, W, h)
+    ref_out, ref_W, ref_h = oracle.rec_fwd(*x)
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.backward(dev(go))
+    names = "qx kx vx bx R_q R_k R_v r_b".split()
+    for name, t, r in zip(names, ts, oracle.rec_bwd(*x, go)):
+        check("grad_" + name, t.grad, r)
+
+
 def test_rnn_and_rec_take_strided_views(fwp):
     # inputs as the layers pass them: [L,N,H,*] storage permuted to [N,H,L,*]
     def lnh(x):
