@@ -1,7 +1,8 @@
 // Register-state kernels of the Delta LSTM v4 for D in {16, 32}: three delta-rule memories (gate
 // order i, u, o), each held like the single memory of the Delta RNN kernels (fwp_rnn_reg.hip), read
 // with the softmax of the previous output; i = sigmoid, u linear, o = sigmoid, c = i u + (1 - i) c,
-// h = o c.  One wave64 per sequence.  Tiles of TL steps (8 at D = 32, 16 at D = 16) keep the LDS
+// h = o c.  One wave64 per sequence, or, while there are SIMDs to spare, two (forward) and four (backward)
+// that hand tiles over through LDS.  Tiles of TL steps (8 at D = 32, 16 at D = 16) keep the LDS
 // footprint of the nine (fifteen in backward) streamed tensors small enough for several waves per CU.
 //
 // Backward: what the cell needs per step is four coefficients, o, c o (1 - o), (u - c_prev) i (1 - i)

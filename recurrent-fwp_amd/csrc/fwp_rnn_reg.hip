@@ -5,6 +5,8 @@
 // and a sum over the whole wave (DPP row rotates, two row broadcasts and a lane read each) and then becomes a periodic
 // operand with one ds_bpermute per 16 entries.  In backward the softmax of the delayed output does
 // not sit on the sequential path: it is recomputed for a whole tile when the tile is committed.
+// Up to 1024 sequences the forward step is divided between two waves of a sequence, the backward step
+// between three (up to 512 sequences) or two, which hand tiles over through LDS.
 #include "fwp_reg.hpp"
 
 namespace fwp {
