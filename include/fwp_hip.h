@@ -48,7 +48,11 @@ enum {
     FWP_Q_VERSION = 0,
     FWP_Q_CHUNK_QUANTUM = 1, /* chunk must be a multiple of this */
     FWP_Q_DEFAULT_CHUNK = 2,
-    FWP_Q_MAX_STATE_FLOATS = 3 /* largest E*M (delta) the library accepts */
+    FWP_Q_MAX_STATE_FLOATS = 3, /* largest E*M (delta) the library accepts */
+    /* largest D of a call that saves for a backward pass (forward refuses larger ones up front) */
+    FWP_Q_MAX_D_RNN = 4,
+    FWP_Q_MAX_D_REC = 5,
+    FWP_Q_MAX_D_LSTM = 6
 };
 
 const char *fwp_strerror(int code);
@@ -65,6 +69,24 @@ int fwp_query(int what);
 enum { FWP_CFG_DELTA_KERNELS = 0 };
 enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2, FWP_DELTA_SPLIT = 3 };
 int fwp_config(int key, int value);
+
+/*
+ * Which kernels a delta-rule call with these views and dimensions takes under the current
+ * FWP_CFG_DELTA_KERNELS setting, assuming 16-byte aligned contiguous buffers: a pure function of its
+ * arguments, touches no device.  `backward` = 0: x is v; 1: x is grad_out.  Returns FWP_KIND_* or
+ * FWP_E_SHAPE.  The kernels that address a sequence with 32-bit offsets (FWP_KIND_SPLIT,
+ * FWP_KIND_CHUNKED, FWP_KIND_PHASE) are never chosen for a view that could exceed them.
+ * No counterpart in the reference (its one kernel per direction takes every call).
+ */
+enum {
+    FWP_KIND_LDS = 0,     /* state in LDS, any E, M */
+    FWP_KIND_SCAN = 1,    /* state in registers, step by step */
+    FWP_KIND_CHUNKED = 2, /* 16-step blocks on the matrix cores, one wave per sequence */
+    FWP_KIND_SPLIT = 3,   /* the same blocks, roles of a block on several waves */
+    FWP_KIND_PHASE = 4    /* blocks prepared in parallel by the waves of a workgroup, short chain */
+};
+int fwp_delta_kind(int backward, fwp_view q, fwp_view k, fwp_view x, fwp_view beta, int N, int H,
+                   int L, int E, int M);
 
 /* 0 if the current HIP device is a gfx950 part, FWP_E_ARCH otherwise. */
 int fwp_check_device(void);

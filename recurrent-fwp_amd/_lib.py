@@ -41,7 +41,8 @@ _SIGNATURES = {
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
 }
 EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
-                                       "fwp_delta_ckpt_floats"])
+                                       "fwp_delta_ckpt_floats", "fwp_delta_kind"])
+KIND_LDS, KIND_SCAN, KIND_CHUNKED, KIND_SPLIT, KIND_PHASE = 0, 1, 2, 3, 4
 CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT = 0, 0, 1, 2, 3
 
 _lib = None
@@ -68,6 +69,8 @@ def lib():
         handle.fwp_check_device.restype = ctypes.c_int
         handle.fwp_delta_ckpt_floats.argtypes = [ctypes.c_int] * 6
         handle.fwp_delta_ckpt_floats.restype = ctypes.c_longlong
+        handle.fwp_delta_kind.argtypes = [_I] + [_V] * 4 + [_I] * 5
+        handle.fwp_delta_kind.restype = ctypes.c_int
         handle.fwp_config.argtypes = [ctypes.c_int, ctypes.c_int]
         handle.fwp_config.restype = ctypes.c_int
         _lib = handle
@@ -84,6 +87,7 @@ def query(what):
 
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
+Q_MAX_D_RNN, Q_MAX_D_REC, Q_MAX_D_LSTM = 4, 5, 6
 
 
 _ckpt_floats_cache = {}
@@ -125,6 +129,15 @@ def require_device(t):
     with torch.cuda.device(dev):
         check(lib().fwp_check_device(), "device check")
     _checked_devices.add(dev)
+
+
+def same_device(ref, *others):
+    """Every tensor of a call lives on the first one's GPU: the kernels get raw addresses, and an
+    address of host memory or of another GPU would be a memory fault there, not an exception."""
+    dev = ref.device
+    for t in others:
+        if t.device != dev:
+            raise FwpError(f"all tensors of a call must be on the same device: got '{t.device}' beside '{dev}'")
 
 
 def rows(t):

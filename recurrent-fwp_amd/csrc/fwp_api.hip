@@ -3,6 +3,7 @@
 // LDS-state kernels (everything else).
 #include "fwp_common.hpp"
 
+#include <atomic>
 #include <initializer_list>
 #include <stdint.h>
 
@@ -23,7 +24,8 @@ int check_dims(int N, int H, int L, int E, int M, int chunk) {
 }
 
 // fwp_config(FWP_CFG_DELTA_KERNELS, .)
-int g_delta_kernels = FWP_DELTA_AUTO;
+// (a test and measurement switch: one word, read once per call, written by fwp_config only)
+std::atomic<int> g_delta_kernels{FWP_DELTA_AUTO};
 
 // Blocks on the matrix cores pay off from about two blocks on; single steps (stepwise inference)
 // stay on the scan kernel.
@@ -60,9 +62,28 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
     return (int64_t)N * H <= 1024;
 }
 
+// Which kernels a delta-rule call takes.  `x` is v for the forward pass and grad_out for the backward
+// pass (the views read 16 bytes at a time besides q and k); `aligned` says that every contiguous buffer
+// of the call is 16-byte aligned.  The kernels that read through buffer resources (split, chunked)
+// address a sequence with 32-bit byte offsets: views beyond them go to the scan or the LDS-state kernels,
+// which use 64-bit addresses, in both directions alike.
+int delta_kind(bool backward, bool aligned, const fwp_view &q, const fwp_view &k, const fwp_view &x,
+               const fwp_view &beta, int N, int H, int L, int E, int M) {
+    if (aligned && delta_split(!backward, N, H, L, E, M, {q, k, x}, beta)) return FWP_KIND_SPLIT;
+    if (aligned && reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x))
+        return delta_chunked(L) && in_range32(L, E, M, {q, k, x, beta}) ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
+    return FWP_KIND_LDS;
+}
+
 }  // namespace
 
 extern "C" {
+
+int fwp_delta_kind(int backward, fwp_view q, fwp_view k, fwp_view x, fwp_view beta, int N, int H, int L,
+                   int E, int M) {
+    if (check_dims(N, H, L, E, M, kDefaultChunk)) return FWP_E_SHAPE;
+    return delta_kind(backward != 0, true, q, k, x, beta, N, H, L, E, M);
+}
 
 int fwp_config(int key, int value) {
     if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_SPLIT) {
@@ -92,6 +113,9 @@ int fwp_query(int what) {
         case FWP_Q_CHUNK_QUANTUM: return kChunkQuantum;
         case FWP_Q_DEFAULT_CHUNK: return kDefaultChunk;
         case FWP_Q_MAX_STATE_FLOATS: return 16384;
+        case FWP_Q_MAX_D_RNN: return generic_max_dim(0);
+        case FWP_Q_MAX_D_REC: return generic_max_dim(1);
+        case FWP_Q_MAX_D_LSTM: return generic_max_dim(2);
         default: return -1;
     }
 }
@@ -119,14 +143,14 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(out);
-    if (aligned && delta_split(true, N, H, L, E, M, {q, k, v}, beta))
-        return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned) {
-        if (delta_chunked(L) && in_range32(L, E, M, {q, k, v, beta}))
-            return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
-                                  (hipStream_t)stream);
-        return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk,
-                             (hipStream_t)stream);
+    switch (delta_kind(false, aligned, q, k, v, beta, N, H, L, E, M)) {
+        case FWP_KIND_SPLIT:
+            return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
+        case FWP_KIND_CHUNKED:
+            return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+        case FWP_KIND_SCAN:
+            return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
+        default: break;
     }
     if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, M, chunk, (hipStream_t)stream)) return rc;
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
@@ -141,15 +165,17 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv);
-    if (aligned && delta_split(false, N, H, L, E, M, {q, k, grad_out}, beta))
-        return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
-                               (hipStream_t)stream);
-    if (reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(grad_out) && aligned) {
-        if (delta_chunked(L))
-            return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
-                                  chunk, (hipStream_t)stream);
-        return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E,
-                             chunk, (hipStream_t)stream);
+    switch (delta_kind(true, aligned, q, k, grad_out, beta, N, H, L, E, M)) {
+        case FWP_KIND_SPLIT:
+            return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
+                                   (hipStream_t)stream);
+        case FWP_KIND_CHUNKED:
+            return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, chunk,
+                                  (hipStream_t)stream);
+        case FWP_KIND_SCAN:
+            return reg_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, chunk,
+                                 (hipStream_t)stream);
+        default: break;
     }
     return generic_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
                              chunk, (hipStream_t)stream);

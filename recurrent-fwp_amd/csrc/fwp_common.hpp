@@ -61,6 +61,10 @@ int generic_rec_bwd(const float *q_act, const float *k_act, const float *beta_ac
 int reduce_rec_param_grads(const float *workspace, float *gRq, float *gRk, float *gRv,
                            float *grb, int N, int H, int D, hipStream_t s);
 
+// Largest D of a differentiated call of the recurrent operators on the LDS-state kernels
+// (op: 0 Delta RNN, 1 Recurrent Delta Net, 2 Delta LSTM).
+int generic_max_dim(int op);
+
 // Register-state kernels (one wave per sequence): E = M = D in {16, 32}, 16-byte aligned rows.
 bool reg_view_ok(const fwp_view &v);
 bool reg_delta_supported(int E, int M);

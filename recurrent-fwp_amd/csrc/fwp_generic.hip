@@ -637,6 +637,45 @@ __global__ void k_reduce_param_grads(const float *workspace, float *gRq, float *
     else grb[h * D + j - 3 * DD] = acc;
 }
 
+// The same sums when a head's 3 D^2 + D values are a whole number of 16-byte words: a workgroup takes
+// kRedCols words of one head, kRedSlices threads share a word's N terms (thread i the terms n = i,
+// i + kRedSlices, ... in ascending order) and one of them adds the kRedSlices partial sums in ascending
+// order: the order of the additions depends on N only, not on timing.  (One thread per value with all
+// N terms, as above, is a few dozen workgroups with long dependent chains of loads.)
+constexpr int kRedCols = 16, kRedSlices = 16;
+__global__ __launch_bounds__(kRedCols * kRedSlices) void k_reduce_param_grads_wide(
+    const float *__restrict__ workspace, float *__restrict__ gRq, float *__restrict__ gRk,
+    float *__restrict__ gRv, float *__restrict__ grb, int N, int H, int D) {
+    __shared__ float4 part[kRedSlices][kRedCols];
+    const int per4 = (3 * D * D + D) / 4;
+    const int col = threadIdx.x % kRedCols, slice = threadIdx.x / kRedCols;
+    const int j4 = blockIdx.x * kRedCols + col, h = blockIdx.y;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (j4 < per4) {
+        const float4 *src = reinterpret_cast<const float4 *>(workspace) + (int64_t)h * per4 + j4;
+        for (int n = slice; n < N; n += kRedSlices) {
+            const float4 x = src[(int64_t)n * H * per4];
+            acc.x += x.x, acc.y += x.y, acc.z += x.z, acc.w += x.w;
+        }
+    }
+    part[slice][col] = acc;
+    __syncthreads();
+    if (slice != 0 || j4 >= per4) return;
+    for (int i = 1; i < kRedSlices; i++) {
+        const float4 x = part[i][col];
+        acc.x += x.x, acc.y += x.y, acc.z += x.z, acc.w += x.w;
+    }
+    const int DD = D * D;
+    const float a[4] = {acc.x, acc.y, acc.z, acc.w};
+    for (int r = 0; r < 4; r++) {
+        const int j = 4 * j4 + r;
+        if (j < DD) gRq[h * DD + j] = a[r];
+        else if (j < 2 * DD) gRk[h * DD + j - DD] = a[r];
+        else if (j < 3 * DD) gRv[h * DD + j - 2 * DD] = a[r];
+        else grb[h * D + j - 3 * DD] = a[r];
+    }
+}
+
 template <typename K>
 int prepare(K kernel, size_t bytes) {
     if (bytes > kMaxLds) return FWP_E_TOO_LARGE;
@@ -656,6 +695,8 @@ int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *
                       float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
                       hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)E * pitch(M) + 2 * E + 2 * M);
+    // a backward pass will follow: refuse here what it could not take, before the states are touched
+    if (ckpt && sizeof(float) * ((size_t)2 * E * pitch(M) + 3 * E + 5 * M + 1) > kMaxLds) return FWP_E_TOO_LARGE;
     if (int rc = prepare(k_delta_fwd, bytes)) return rc;
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_delta_fwd, dim3(N * H), dim3(NT), bytes, s, q, k, v, beta, W, out, vdiff,
@@ -677,6 +718,8 @@ int generic_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff,
 int generic_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N,
                     int H, int L, int E, int M, int chunk, hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)E * pitch(M) + 2 * E + M);
+    // a backward pass will follow: refuse here what it could not take, before the states are touched
+    if (ckpt && sizeof(float) * ((size_t)2 * E * pitch(M) + 2 * E + 2 * M) > kMaxLds) return FWP_E_TOO_LARGE;
     if (int rc = prepare(k_sum_fwd, bytes)) return rc;
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_sum_fwd, dim3(N * H), dim3(NT), bytes, s, q, k, v, W, out, ckpt, H, L, E,
@@ -699,6 +742,8 @@ int generic_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W,
                     float *out, float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
                     hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)D * pitch(D) + 7 * D);
+    // a backward pass will follow: refuse here what it could not take, before the states are touched
+    if (ckpt && sizeof(float) * ((size_t)2 * D * pitch(D) + 12 * D + 1) > kMaxLds) return FWP_E_TOO_LARGE;
     if (int rc = prepare(k_rnn_fwd, bytes)) return rc;
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_rnn_fwd, dim3(N * H), dim3(NT), bytes, s, z, k, v, beta, W, h, out, vdiff,
@@ -722,6 +767,8 @@ int generic_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *
                      float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk,
                      hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)3 * D * pitch(D) + 16 * D);
+    // a backward pass will follow: refuse here what it could not take, before the states are touched
+    if (ckpt && sizeof(float) * ((size_t)6 * D * pitch(D) + 19 * D + 1) > kMaxLds) return FWP_E_TOO_LARGE;
     if (int rc = prepare(k_lstm_fwd, bytes)) return rc;
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_lstm_fwd, dim3(N * H), dim3(NT), bytes, s, g, h, c, out, cell, gates, vdiff,
@@ -746,6 +793,8 @@ int generic_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const fl
                     float *out, float *q_act, float *k_act, float *beta_act, float *vdiff,
                     float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)D * pitch(D) + 8 * D + 1);
+    // a backward pass will follow: refuse here what it could not take, before the states are touched
+    if (ckpt && sizeof(float) * ((size_t)2 * D * pitch(D) + 3 * D * D + 16 * D + 1) > kMaxLds) return FWP_E_TOO_LARGE;
     if (int rc = prepare(k_rec_fwd, bytes)) return rc;
     int nchunk = (L + chunk - 1) / chunk;
     hipLaunchKernelGGL(k_rec_fwd, dim3(N * H), dim3(NT), bytes, s, qx, kx, vx, bx, Rq, Rk, Rv, rb,
@@ -767,9 +816,27 @@ int generic_rec_bwd(const float *q_act, const float *k_act, const float *beta_ac
     return launched();
 }
 
+// Largest D whose differentiated call fits the LDS-state kernels (the backward pass is the larger one).
+int generic_max_dim(int op) {
+    int best = 0;
+    for (int D = 1; D <= 128; D++) {
+        const size_t floats = op == 0   ? (size_t)2 * D * pitch(D) + 12 * D + 1
+                              : op == 1 ? (size_t)2 * D * pitch(D) + 3 * D * D + 16 * D + 1
+                                        : (size_t)6 * D * pitch(D) + 19 * D + 1;
+        if (sizeof(float) * floats <= kMaxLds && (size_t)D * D <= 16384) best = D;
+    }
+    return best;
+}
+
 int reduce_rec_param_grads(const float *workspace, float *gRq, float *gRk, float *gRv,
                            float *grb, int N, int H, int D, hipStream_t s) {
-    int total = H * (3 * D * D + D);
+    const int per = 3 * D * D + D;
+    if (per % 4 == 0 && (reinterpret_cast<uintptr_t>(workspace) & 15) == 0) {
+        hipLaunchKernelGGL(k_reduce_param_grads_wide, dim3((per / 4 + kRedCols - 1) / kRedCols, H),
+                           dim3(kRedCols * kRedSlices), 0, s, workspace, gRq, gRk, gRv, grb, N, H, D);
+        return launched();
+    }
+    int total = H * per;
     hipLaunchKernelGGL(k_reduce_param_grads, dim3((total + 255) / 256), dim3(256), 0, s, workspace,
                        gRq, gRk, gRv, grb, N, H, D);
     return launched();

@@ -93,6 +93,15 @@ void require_device(const at::Tensor &t) {
     checked[idx] = true;
 }
 
+// Every tensor of a call lives on the first one's GPU: the kernels get raw addresses, and an address
+// of host memory or of another GPU would be a memory fault there, not an exception.
+void same_device(const at::Tensor &ref, std::initializer_list<at::Tensor> others) {
+    for (const at::Tensor &t : others)
+        if (t.defined() && t.device() != ref.device())
+            fail("all tensors of a call must be on the same device: got '" + t.device().str() + "' beside '" +
+                 ref.device().str() + "'");
+}
+
 void *stream_of(const at::Tensor &t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
 
 struct DeltaFn : torch::autograd::Function<DeltaFn> {
@@ -100,6 +109,7 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
                               const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &beta_in,
                               const at::Tensor &W, bool need_grad) {
         require_device(Q_in);
+        same_device(Q_in, {K_in, V_in, beta_in, W});
         if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
         const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
         if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}) ||
@@ -176,6 +186,7 @@ struct SumFn : torch::autograd::Function<SumFn> {
                               const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &W, bool exact,
                               bool need_grad) {
         require_device(Q_in);
+        same_device(Q_in, {K_in, V_in, W});
         if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
         const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
         if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}))
@@ -250,6 +261,7 @@ struct RnnFn : torch::autograd::Function<RnnFn> {
                               const at::Tensor &V_in, const at::Tensor &W, const at::Tensor &beta_in,
                               const at::Tensor &h0, bool need_grad) {
         require_device(Z_in);
+        same_device(Z_in, {K_in, V_in, W, beta_in, h0});
         require(Z_in.dim() == 4 && V_in.dim() == 4, "expected 4-D [N,H,L,D] tensors");
         const int64_t N = Z_in.size(0), H = Z_in.size(1), L = Z_in.size(2), D = V_in.size(3);
         require(same_shape(Z_in, {N, H, L, D}) && same_shape(K_in, {N, H, L, D}) && same_shape(V_in, {N, H, L, D}),
@@ -327,6 +339,7 @@ struct RecFn : torch::autograd::Function<RecFn> {
                               const at::Tensor &R_k, const at::Tensor &R_v, const at::Tensor &r_b, const at::Tensor &W,
                               const at::Tensor &h0, bool need_grad) {
         require_device(qx_in);
+        same_device(qx_in, {kx_in, vx_in, bx_in, R_q, R_k, R_v, r_b, W, h0});
         require(qx_in.dim() == 4 && vx_in.dim() == 4, "expected 4-D [N,H,L,D] tensors");
         const int64_t N = qx_in.size(0), H = qx_in.size(1), L = qx_in.size(2), E = qx_in.size(3), M = vx_in.size(3);
         require(E == M, "Current kernel only support this case.");
@@ -421,6 +434,7 @@ struct LstmFn : torch::autograd::Function<LstmFn> {
         const at::Tensor &bu, const at::Tensor &Wu, const at::Tensor &Zo, const at::Tensor &Ko, const at::Tensor &Vo,
         const at::Tensor &bo, const at::Tensor &Wo, const at::Tensor &h0, const at::Tensor &c0, bool need_grad) {
         require_device(Zi);
+        same_device(Zi, {Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0});
         if (Zi.dim() != 4 || Vi.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
         const int64_t N = Zi.size(0), H = Zi.size(1), L = Zi.size(2), D = Vi.size(3);
         const at::Tensor *Zs[3] = {&Zi, &Zu, &Zo}, *Ks[3] = {&Ki, &Ku, &Ko}, *Vs[3] = {&Vi, &Vu, &Vo},

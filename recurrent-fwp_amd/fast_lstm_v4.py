@@ -28,6 +28,7 @@ class FastLSTMv4(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0):
         _lib.require_device(Zi)
+        _lib.same_device(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0)
         N, H, L, _ = Zi.shape
         D = Vi.shape[-1]
         Zs, Ks, Vs, Bs, Ws = (Zi, Zu, Zo), (Ki, Ku, Ko), (Vi, Vu, Vo), (bi, bu, bo), (Wi, Wu, Wo)

@@ -24,6 +24,7 @@ class FastWeightSum(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q, K, V, W):
         _lib.require_device(Q)
+        _lib.same_device(Q, K, V, W)
         N, H, L, E = Q.shape
         M = V.shape[-1]
         if K.shape != (N, H, L, E) or V.shape != (N, H, L, M):

@@ -22,6 +22,7 @@ class DeltaFastWeight(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Q, K, V, beta, W):
         _lib.require_device(Q)
+        _lib.same_device(Q, K, V, beta, W)
         N, H, L, E = Q.shape
         M = V.shape[-1]
         if K.shape != (N, H, L, E) or V.shape != (N, H, L, M) or beta.shape != (N, H, L, 1):
@@ -66,6 +67,7 @@ class DeltaFastWeight(torch.autograd.Function):
         vdiff = saved.data_ptr()
         ckpt = vdiff + 4 * N * H * L * M
         qv, kv, bv = ctx.views
+        _lib.same_device(Q, grad_out)
         grad_out, gv_ = _lib.rows(grad_out)
         grad_Q = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)
         grad_K = torch.empty((N, H, L, E), device=Q.device, dtype=torch.float32)

@@ -18,6 +18,7 @@ class FastRNNv2(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Z, K, V, W, beta, h0):
         _lib.require_device(Z)
+        _lib.same_device(Z, K, V, W, beta, h0)
         N, H, L, _ = Z.shape
         D = V.shape[-1]
         # same preconditions as the reference (:54-57)

@@ -139,8 +139,13 @@ class DeltaNetLayer(nn.Module):
             q, k, v, beta = (t.permute(1, 2, 0, 3) for t in qkvb.split((D, D, D, 1), dim=-1))
             q, k, beta = sum_normalised_elu(q), sum_normalised_elu(k), torch.sigmoid(beta)
 
+        hip_op = self.fast_weight_op is fast_weight_delta
+        if hip_op and q.dtype != torch.float32:
+            # half or bf16 activations (autocast): the operator and its state are fp32, as the
+            # reference's kernel and its torch.zeros state are
+            q, k, v, beta = q.float(), k.float(), v.float(), beta.float()
         if mems is None:
-            W = torch.zeros(bsz, H, D, D, device=h.device, dtype=h.dtype)
+            W = torch.zeros(bsz, H, D, D, device=h.device, dtype=torch.float32 if hip_op else q.dtype)
         else:
             if not carry_over_fast_weight:
                 raise ValueError("mems are only meaningful with carry_over_fast_weight=True")
@@ -149,7 +154,7 @@ class DeltaNetLayer(nn.Module):
             W = mems[0][:bsz].clone()
 
         out = self.fast_weight_op(q, k, v, beta, W)                  # [bsz, H, slen, D]
-        out = (self.scale * out).permute(2, 0, 1, 3).reshape(slen, bsz, H * D)
+        out = (self.scale * out).permute(2, 0, 1, 3).reshape(slen, bsz, H * D).to(x.dtype)
         out = residual + self.drop(self.o_net(out))
         if not self.pre_lnorm:
             out = self.layer_norm(out)

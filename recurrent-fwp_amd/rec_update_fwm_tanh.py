@@ -19,6 +19,7 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
     @staticmethod
     def forward(ctx, qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0):
         _lib.require_device(qx)
+        _lib.same_device(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0)
         N, H, L, E = qx.shape
         M = vx.shape[-1]
         # same preconditions as the reference (:52-56)

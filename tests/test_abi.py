@@ -73,6 +73,53 @@ def test_ckpt_size_and_config_entry_points(fwp):
     assert lib.fwp_sum_bwd(v, v, v, v, p, None, p, p, p, 1, 1, 4, 16, 16, 24, None) == -3
 
 
+def test_delta_dispatch_keeps_32_bit_kernels_off_views_beyond_their_range(fwp):
+    """fwp_delta_kind is the dispatch of fwp_delta_fwd / fwp_delta_bwd as a pure function.  Views into
+    [T, B, H*D] storage with T = 8192 and B*H*D = 65536 pass 2 GiB along the sequence axis: the
+    kernels that address a sequence with 32-bit offsets must not get them, forward or backward."""
+    L = fwp._lib
+    lib = L.lib()
+    N, H, T, D = 128, 32, 8192, 16
+    small = L.View(4096, H * T * D, T * D, D)
+    huge = L.View(4096, H * D, D, N * H * D)          # permuted [T,N,H,D]: 256 KiB between steps
+    beta = L.View(4096, H * T, T, 1)
+    offsets32 = (L.KIND_CHUNKED, L.KIND_SPLIT, L.KIND_PHASE)
+    for setting in (L.DELTA_AUTO, L.DELTA_CHUNKED, L.DELTA_SPLIT):
+        L.config(L.CFG_DELTA_KERNELS, setting)
+        try:
+            for backward in (0, 1):
+                assert lib.fwp_delta_kind(backward, small, small, small, beta, 4, 8, 256, D, D) in offsets32
+                for views in ((huge, small, small), (small, huge, small), (small, small, huge)):
+                    kind = lib.fwp_delta_kind(backward, *views, beta, N, H, T, D, D)
+                    assert kind == L.KIND_SCAN, (setting, backward, kind)
+        finally:
+            L.config(L.CFG_DELTA_KERNELS, L.DELTA_AUTO)
+    # short sequences stay on the scan kernels, shapes without a fast kernel on the LDS kernels
+    assert lib.fwp_delta_kind(0, small, small, small, beta, 4, 8, 8, D, D) == L.KIND_SCAN
+    odd = L.View(4096, 8 * 64 * 24, 64 * 24, 24)
+    assert lib.fwp_delta_kind(1, odd, odd, odd, beta, 4, 8, 64, 24, 24) == L.KIND_LDS
+    assert lib.fwp_delta_kind(0, small, small, small, beta, 0, 8, 64, D, D) == -2
+
+
+def test_largest_state_of_a_differentiated_call_is_published(fwp):
+    L = fwp._lib
+    rnn, rec, lstm = (L.query(q) for q in (L.Q_MAX_D_RNN, L.Q_MAX_D_REC, L.Q_MAX_D_LSTM))
+    assert 64 <= lstm <= rec <= rnn <= 128
+
+
+def test_operators_refuse_tensors_on_different_devices(fwp):
+    """Only the first tensor being on the GPU is not enough: the others are passed by address."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("needs a machine without a GPU (the check itself is device independent)")
+    L = fwp._lib
+    meta = torch.zeros(1, 1, 2, 4, device="meta")
+    cpu = torch.zeros(1, 1, 2, 4)
+    with pytest.raises(L.FwpError, match="same device"):
+        L.same_device(meta, meta, cpu)
+    L.same_device(cpu, cpu, cpu)
+
+
 def test_operators_refuse_cpu_tensors(fwp):
     import torch
     q = torch.zeros(1, 1, 2, 4)

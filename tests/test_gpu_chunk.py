@@ -23,7 +23,9 @@ def run(fwp, arrays, chunk, fwd_kind, bwd_kind):
     view = lambda t: L_.View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
     W = W0.clone()
     out, vdiff = torch.empty_like(v), torch.empty_like(v)
-    ckpt = torch.empty(L_.delta_ckpt_floats(N, H, T, E, M, chunk), device="cuda", dtype=torch.float32)
+    # what a caching allocator may hand back after a blocked forward of the same shape: a header that
+    # says "per-block matrices follow" and stale matrices; every forward kind has to set it right
+    ckpt = torch.ones(L_.delta_ckpt_floats(N, H, T, E, M, chunk), device="cuda", dtype=torch.float32)
     gq, gk, gv, gb = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(beta)
     stream = L_.stream_of(q)
     try:
