@@ -1,0 +1,9 @@
+"""``fast_weight_rnn_v2``: the reference's module of this name (algorithmic/fast_weight_rnn_v2/__init__.py), served by the
+MI355X implementation: Delta RNN v2.  Imported as ``from fast_weight_rnn_v2 import fast_rnn_v2``
+(algorithmic/layers.py:7-10)."""
+from _fwp_dropin import package as _package
+
+FastRNNv2 = _package().FastRNNv2
+fast_rnn_v2 = _package().fast_rnn_v2
+
+__all__ = ["FastRNNv2", "fast_rnn_v2"]

@@ -1,0 +1,9 @@
+"""``torchbeast.rec_update_fwm_tanh``: the reference's module of this name (reinforcement_learning/torchbeast/rec_update_fwm_tanh/__init__.py), served by the
+MI355X implementation: Recurrent Delta Net update with tanh feedback.  Imported as ``from torchbeast.rec_update_fwm_tanh import rec_update_fwm_tanh``
+(reinforcement_learning/torchbeast/layer.py:7-10)."""
+from _fwp_dropin import package as _package
+
+FastWeightRecUpdateTanh = _package().FastWeightRecUpdateTanh
+rec_update_fwm_tanh = _package().rec_update_fwm_tanh
+
+__all__ = ["FastWeightRecUpdateTanh", "rec_update_fwm_tanh"]

@@ -1,0 +1,148 @@
+"""Parity at the benchmark sizes, whole tensors against the float64 C oracle, default dispatch.
+
+For every output, final state and gradient the achieved error is printed (run with -s) and written to
+gpurun_out/parity_<case>.json when that directory exists:
+  max_abs          max |got - want|
+  rel_scale        max_abs / max |want|                    (error relative to the tensor's scale)
+  rel_elem         max |got - want| / (|want| + 1e-6)      (the measure of the reference's own self-tests,
+                   algorithmic/fast_weight/__init__.py:107-111, taken there over a handful of values)
+  combined         max |got - want| / (1e-4 + 1e-3 |want|) (<= 1: every element within atol + rtol |want|)
+Asserted for every tensor: max_abs <= 1e-4 and rel_scale <= 1e-3, the two bounds separately, and
+`combined` <= 1.  rel_elem on its own cannot hold over millions of values, some of which are arbitrarily
+close to zero; it is reported, with the share of elements beyond 1e-3."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import delta_inputs, lstm_inputs, rec_inputs, rnn_inputs
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ATOL, RTOL = 1e-4, 1e-3
+
+def measures(got, want):
+    got = np.asarray(got, np.float64)
+    want = np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    rel = err / (np.abs(want) + 1e-6)
+    return {
+        "max_abs": float(err.max()),
+        "max_want": float(np.abs(want).max()),
+        "rel_scale": float(err.max() / max(np.abs(want).max(), 1e-30)),
+        "rel_elem": float(rel.max()),
+        "share_rel_elem_above_1e-3": float((rel > 1e-3).mean()),
+        "combined": float((err / (ATOL + RTOL * np.abs(want))).max()),
+    }
+
+
+def report(case, rows):
+    print(f"\n{case}")
+    print(f"  {'tensor':8s} {'max|want|':>10s} {'max_abs':>10s} {'rel_scale':>10s} {'rel_elem':>10s} {'>1e-3':>9s} {'combined':>9s}")
+    for name, m in rows.items():
+        print(f"  {name:8s} {m['max_want']:10.3e} {m['max_abs']:10.3e} {m['rel_scale']:10.3e} {m['rel_elem']:10.3e} "
+              f"{m['share_rel_elem_above_1e-3']:9.2e} {m['combined']:9.3f}", flush=True)
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, f"parity_{case}.json"), "w") as f:
+            json.dump(rows, f, indent=1)
+    for name, m in rows.items():
+        assert m["combined"] <= 1.0, f"{case} {name}: beyond {ATOL} + {RTOL}|want| ({m})"
+        assert m["rel_scale"] <= RTOL, f"{case} {name}: relative error {m['rel_scale']:.3e}"
+        assert m["max_abs"] <= ATOL, f"{case} {name}: max abs error {m['max_abs']:.3e}"
+
+
+def dev(a, grad=False):
+    t = torch.from_numpy(np.ascontiguousarray(a, np.float32)).cuda()
+    return t.requires_grad_(True) if grad else t
+
+
+def f64(arrays):
+    return [np.asarray(a, np.float64) for a in arrays]
+
+
+@pytest.mark.parametrize("case,shape", [("delta_B96H8T256D16", (96, 8, 256, 16)),
+                                        ("delta_B32H8T1024D32", (32, 8, 1024, 32))])
+def test_delta_rule_whole_batch_against_the_oracle(fwp, case, shape):
+    N, H, T, D = shape
+    q, k, v, beta, W0, go = delta_inputs(2, N, H, T, D, D, dtype=np.float32)
+    ts = [dev(a, True) for a in (q, k, v, beta)]
+    W = dev(W0)
+    out = fwp.fast_weight_delta(*ts, W)
+    out.backward(dev(go))
+    torch.cuda.synchronize()
+    q, k, v, beta, W0, go = f64((q, k, v, beta, W0, go))
+    want_out, want_W = oracle.delta_fwd(q, k, v, beta, W0)
+    want_g = oracle.delta_bwd(q, k, v, beta, W0, go)[:4]
+    rows = {"out": measures(out.detach().cpu().numpy(), want_out), "W": measures(W.cpu().numpy(), want_W)}
+    for name, t, w in zip(("gq", "gk", "gv", "gbeta"), ts, want_g):
+        rows[name] = measures(t.grad.cpu().numpy(), w)
+    report(case, rows)
+
+
+def test_delta_rnn_whole_batch_against_the_oracle(fwp):
+    N, H, T, D = 64, 8, 256, 32
+    z, k, v, W0, beta, h0, go = rnn_inputs(4, N, H, T, D, dtype=np.float32)
+    ts = [dev(a, True) for a in (z, k, v, beta)]
+    W, h = dev(W0), dev(h0)
+    out = fwp.fast_rnn_v2(ts[0], ts[1], ts[2], W, ts[3], h)
+    out.backward(dev(go))
+    torch.cuda.synchronize()
+    z, k, v, W0, beta, h0, go = f64((z, k, v, W0, beta, h0, go))
+    want_out, want_W, want_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+    want_g = oracle.rnn_bwd(z, k, v, W0, beta, h0, go)
+    rows = {"out": measures(out.detach().cpu().numpy(), want_out), "W": measures(W.cpu().numpy(), want_W),
+            "h": measures(h.cpu().numpy(), want_h)}
+    for name, t, w in zip(("gz", "gk", "gv", "gbeta"), ts, want_g):
+        rows[name] = measures(t.grad.cpu().numpy(), w)
+    report("rnn_B64H8T256D32", rows)
+
+
+def test_recurrent_delta_net_whole_batch_against_the_oracle(fwp):
+    N, H, T, D = 64, 8, 256, 32
+    *x, go = rec_inputs(3, N, H, T, D, dtype=np.float32)
+    ts = [dev(a, True) for a in x[:8]]
+    W, h = dev(x[8]), dev(x[9])
+    out = fwp.rec_update_fwm_tanh(*ts, W, h)
+    out.backward(dev(go))
+    torch.cuda.synchronize()
+    x = f64(x)
+    go = np.asarray(go, np.float64)
+    want_out, want_W, want_h = oracle.rec_fwd(*x)
+    want_g = oracle.rec_bwd(*x, go)
+    rows = {"out": measures(out.detach().cpu().numpy(), want_out), "W": measures(W.cpu().numpy(), want_W),
+            "h": measures(h.cpu().numpy(), want_h)}
+    for name, t, w in zip(("gqx", "gkx", "gvx", "gbx", "gRq", "gRk", "gRv", "grb"), ts, want_g):
+        rows[name] = measures(t.grad.cpu().numpy(), w)
+    report("rec_B64H8T256D32", rows)
+
+
+def test_delta_lstm_whole_batch_against_the_oracle(fwp):
+    N, H, T, D = 64, 8, 256, 32
+    Zs, Ks, Vs, Bs, Ws, h0, c0, go = lstm_inputs(5, N, H, T, D, dtype=np.float32)
+    tz, tk, tv, tb = ([dev(a, True) for a in xs] for xs in (Zs, Ks, Vs, Bs))
+    tw = [dev(a) for a in Ws]
+    h, c = dev(h0), dev(c0)
+    args = []
+    for a in range(3):
+        args += [tz[a], tk[a], tv[a], tb[a], tw[a]]
+    out, cell = fwp.fast_lstm_v4(*args, h, c)
+    out.backward(dev(go))
+    torch.cuda.synchronize()
+    Zs, Ks, Vs, Bs, Ws = (f64(xs) for xs in (Zs, Ks, Vs, Bs, Ws))
+    h0, c0, go = f64((h0, c0, go))
+    want_out, want_cell, want_W, want_h, want_c = oracle.lstm_fwd(Zs, Ks, Vs, Bs, Ws, h0, c0)
+    gZ, gK, gV, gB = oracle.lstm_bwd(Zs, Ks, Vs, Bs, Ws, h0, c0, go)
+    rows = {"out": measures(out.detach().cpu().numpy(), want_out),
+            "cell": measures(cell.detach().cpu().numpy(), want_cell),
+            "h": measures(h.cpu().numpy(), want_h), "c": measures(c.cpu().numpy(), want_c)}
+    for a, gate in enumerate("iuo"):
+        rows[f"W_{gate}"] = measures(tw[a].cpu().numpy(), want_W[a])
+        rows[f"gz_{gate}"] = measures(tz[a].grad.cpu().numpy(), gZ[a])
+        rows[f"gk_{gate}"] = measures(tk[a].grad.cpu().numpy(), gK[a])
+        rows[f"gv_{gate}"] = measures(tv[a].grad.cpu().numpy(), gV[a])
+        rows[f"gb_{gate}"] = measures(tb[a].grad.cpu().numpy(), gB[a])
+    report("lstm_B64H8T256D32", rows)

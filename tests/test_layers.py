@@ -213,6 +213,41 @@ def test_gpu_lm_against_loop_operator(pkg):
 
 
 @pytest.mark.gpu
+def test_gpu_lm_at_benchmark_size_against_loop_operator(pkg):
+    """The 16-layer language model of the benchmark (d_model 256, 8 heads of 32, FFN 1024, vocabulary
+    32768, 32 sequences of 1024 tokens drawn from Zipf(1.1), initialisation N(0, 0.02)): fp32 with the HIP
+    operator against float64 with the step loop as operator, same weights and tokens.  Per-token
+    losses within 1e-4 + 1e-3 |want|; every parameter gradient within 1e-3 of its largest entry."""
+    cfg = dict(n_token=32768, n_layer=16, n_head=8, d_model=256, d_head=32, d_inner=1024)
+    B, T = 32, 1024
+    torch.manual_seed(5)
+    ours = pkg.DeltaNetLM(init_std=0.02, **cfg).cuda()
+    ref = pkg.DeltaNetLM(fast_weight_op=loop_op, init_std=0.02, **cfg).to(device="cuda", dtype=torch.float64)
+    ref.load_state_dict({k: v.double() for k, v in ours.state_dict().items()})
+    p = np.arange(1, cfg["n_token"] + 1, dtype=np.float64) ** -1.1
+    cdf = np.cumsum(p / p.sum())
+    toks = np.minimum(np.searchsorted(cdf, np.random.default_rng(0).random((T + 1, B))), cfg["n_token"] - 1)
+    toks = torch.from_numpy(toks.astype(np.int64)).cuda()
+    data, target = toks[:-1], toks[1:]
+    (loss,) = ours(data, target)
+    loss.mean().backward()
+    (loss_ref,) = ref(data, target)
+    loss_ref.mean().backward()
+    torch.cuda.synchronize()
+    err = (loss.double() - loss_ref).abs()
+    print(f"\nLM at benchmark size: mean loss {float(loss_ref.mean()):.4f}, per-token loss max abs err "
+          f"{float(err.max()):.3e}", flush=True)
+    assert bool((err <= ATOL + RTOL * loss_ref.abs()).all()), f"loss: max abs err {float(err.max()):.3e}"
+    worst = 0.0
+    for (name, a), (_, b) in zip(ours.named_parameters(), ref.named_parameters()):
+        scale = float(b.grad.abs().max())
+        e = float((a.grad.double() - b.grad).abs().max())
+        worst = max(worst, e / max(scale, 1e-30))
+        assert e <= 1e-3 * scale + 1e-9, f"grad {name}: {e:.3e} (scale {scale:.3e})"
+    print(f"parameter gradients: worst error relative to the tensor's largest entry {worst:.3e}", flush=True)
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("D", [16, 32, 64])
 def test_gpu_fused_pre_step_against_the_pytorch_lines(pkg, D):
     from importlib import import_module
