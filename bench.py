@@ -482,7 +482,7 @@ def main():
     ap.add_argument("--workload", choices=sorted(WORKLOADS) + ["lm", "step"], default="delta")
     ap.add_argument("--cpu-reps", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--delta-kernels", choices=["auto", "scan", "chunked", "split"], default="auto",
+    ap.add_argument("--delta-kernels", choices=["auto", "scan", "chunked", "split", "phase"], default="auto",
                     help="delta-rule kernels for D=16/32: step-by-step register-state scan or 16-step blocks "
                          "on the matrix cores (default: the library's choice)")
     ap.add_argument("--graph", action="store_true",
@@ -512,7 +512,7 @@ def main():
     from __graft_entry__ import package
     pkg = package()
     pkg._lib.lib()                       # fails loudly if the HIP library is not built
-    pkg._lib.config(pkg._lib.CFG_DELTA_KERNELS, {"auto": 0, "scan": 1, "chunked": 2, "split": 3}[args.delta_kernels])
+    pkg._lib.config(pkg._lib.CFG_DELTA_KERNELS, {"auto": 0, "scan": 1, "chunked": 2, "split": 3, "phase": 4}[args.delta_kernels])
     name = args.workload
     if name == "lm":
         print(json.dumps(run_lm(args, pkg)))

@@ -64,10 +64,11 @@ int fwp_query(int what);
  * FWP_DELTA_AUTO (default: the fastest), FWP_DELTA_SCAN (step-by-step register-state
  * kernels), FWP_DELTA_CHUNKED (16-step blocks on the matrix cores, one wave per sequence),
  * FWP_DELTA_SPLIT (the same blocks, a sequence's work split over several waves; the sum rule
- * takes the one-wave blocks).  All give the same results within the fp32 tolerance.  Returns FWP_E_SHAPE for an unknown key or value.
+ * takes the one-wave blocks), FWP_DELTA_PHASE (16 x 16 states: the blocks of a sequence prepared in
+ * parallel, one product per block on the sequential chain; other shapes as FWP_DELTA_SPLIT).  All give the same results within the fp32 tolerance.  Returns FWP_E_SHAPE for an unknown key or value.
  */
 enum { FWP_CFG_DELTA_KERNELS = 0 };
-enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2, FWP_DELTA_SPLIT = 3 };
+enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2, FWP_DELTA_SPLIT = 3, FWP_DELTA_PHASE = 4 };
 int fwp_config(int key, int value);
 
 /*

@@ -43,7 +43,7 @@ _SIGNATURES = {
 EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
                                        "fwp_delta_ckpt_floats", "fwp_delta_kind"])
 KIND_LDS, KIND_SCAN, KIND_CHUNKED, KIND_SPLIT, KIND_PHASE = 0, 1, 2, 3, 4
-CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT = 0, 0, 1, 2, 3
+CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT, DELTA_PHASE = 0, 0, 1, 2, 3, 4
 
 _lib = None
 _checked_devices = set()

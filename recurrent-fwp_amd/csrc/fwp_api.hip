@@ -55,11 +55,18 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
     if (!in_range32(L, E, M, {beta}) || !in_range32(L, E, M, views)) return false;
     for (const fwp_view &v : views)      // rows read 16 bytes at a time
         if (!reg_view_ok(v)) return false;
-    if (g_delta_kernels == FWP_DELTA_SPLIT) return true;
+    if (g_delta_kernels == FWP_DELTA_SPLIT || g_delta_kernels == FWP_DELTA_PHASE) return true;
     if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
     if (L < 32) return false;
     return (int64_t)N * H <= 1024;
+}
+
+// Of the calls the several-wave kernels take (same views, same range of offsets), those that go to the
+// kernels that prepare the blocks of a sequence in parallel: 16 x 16 states, forward.
+bool delta_phase(bool backward, int L, int E, int M) {
+    if (backward || !phase_delta_dims(E, M)) return false;
+    return g_delta_kernels == FWP_DELTA_PHASE;
 }
 
 // Which kernels a delta-rule call takes.  `x` is v for the forward pass and grad_out for the backward
@@ -69,7 +76,8 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
 // which use 64-bit addresses, in both directions alike.
 int delta_kind(bool backward, bool aligned, const fwp_view &q, const fwp_view &k, const fwp_view &x,
                const fwp_view &beta, int N, int H, int L, int E, int M) {
-    if (aligned && delta_split(!backward, N, H, L, E, M, {q, k, x}, beta)) return FWP_KIND_SPLIT;
+    if (aligned && delta_split(!backward, N, H, L, E, M, {q, k, x}, beta))
+        return delta_phase(backward, L, E, M) ? FWP_KIND_PHASE : FWP_KIND_SPLIT;
     if (aligned && reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x))
         return delta_chunked(L) && in_range32(L, E, M, {q, k, x, beta}) ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
     return FWP_KIND_LDS;
@@ -86,7 +94,7 @@ int fwp_delta_kind(int backward, fwp_view q, fwp_view k, fwp_view x, fwp_view be
 }
 
 int fwp_config(int key, int value) {
-    if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_SPLIT) {
+    if (key == FWP_CFG_DELTA_KERNELS && value >= FWP_DELTA_AUTO && value <= FWP_DELTA_PHASE) {
         g_delta_kernels = value;
         return FWP_OK;
     }
@@ -144,6 +152,8 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(out);
     switch (delta_kind(false, aligned, q, k, v, beta, N, H, L, E, M)) {
+        case FWP_KIND_PHASE:
+            return phase_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, chunk, (hipStream_t)stream);
         case FWP_KIND_SPLIT:
             return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         case FWP_KIND_CHUNKED:

@@ -94,6 +94,11 @@ int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,
 int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                     const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                     int L, int E, int M, int chunk, hipStream_t s);
+// 16 x 16 states with the blocks of a sequence prepared in parallel by the waves of a workgroup and one
+// product per block on the sequential chain (same arguments, results and saved buffers as split_delta_fwd).
+bool phase_delta_dims(int E, int M);
+int phase_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
+                    float *ckpt, int N, int H, int L, int chunk, hipStream_t s);
 int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                    int L, int D, int chunk, hipStream_t s);

@@ -19,12 +19,14 @@ def fwp():
     return importlib.import_module("recurrent-fwp_amd")
 
 
-@pytest.fixture(params=["scan", "chunked", "split"])
+@pytest.fixture(params=["scan", "chunked", "split", "phase"])
 def delta_kernels(request, fwp):
     """The kinds of delta-rule kernels for D = 16/32: the step-by-step scan, 16-step blocks on the
-    matrix cores with one wave per sequence, and those blocks split over several waves.  The sum rule
+    matrix cores with one wave per sequence, those blocks split over several waves, and (16 x 16
+    states) the blocks of a sequence prepared in parallel with a one-product chain.  The sum rule
     has the first two; other shapes take the LDS kernels whatever the setting."""
     L_ = fwp._lib
-    L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT}[request.param])
+    L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT,
+                                      "phase": L_.DELTA_PHASE}[request.param])
     yield request.param
     L_.config(L_.CFG_DELTA_KERNELS, L_.DELTA_AUTO)

@@ -10,13 +10,13 @@ from helpers import delta_inputs, within, max_abs
 
 pytestmark = pytest.mark.gpu
 ATOL, RTOL = 1e-4, 1e-3
-KINDS = ("scan", "chunked", "split")
+KINDS = ("scan", "chunked", "split", "phase")
 
 
 def run(fwp, arrays, chunk, fwd_kind, bwd_kind):
     L_ = fwp._lib
     lib = L_.lib()
-    code = {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT}
+    code = {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT, "phase": L_.DELTA_PHASE}
     q, k, v, beta, W0, go = (torch.from_numpy(a).cuda() for a in arrays)
     N, H, T, E = q.shape
     M = v.shape[-1]
