@@ -41,7 +41,8 @@ enum {
     FWP_E_SHAPE = -2,     /* a dimension is < 1 or inconsistent */
     FWP_E_CHUNK = -3,     /* chunk is not a positive multiple of FWP_Q_CHUNK_QUANTUM */
     FWP_E_TOO_LARGE = -4, /* state does not fit the workgroup's LDS */
-    FWP_E_ARCH = -5       /* current device is not gfx950 */
+    FWP_E_ARCH = -5,      /* current device is not gfx950 */
+    FWP_E_SCRATCH = -6    /* fwp_rec_bwd_static: N*H*(3*D*D+D) exceeds FWP_Q_STATIC_SCRATCH_FLOATS */
 };
 
 enum {
@@ -52,7 +53,8 @@ enum {
     /* largest D of a call that saves for a backward pass (forward refuses larger ones up front) */
     FWP_Q_MAX_D_RNN = 4,
     FWP_Q_MAX_D_REC = 5,
-    FWP_Q_MAX_D_LSTM = 6
+    FWP_Q_MAX_D_LSTM = 6,
+    FWP_Q_STATIC_SCRATCH_FLOATS = 7 /* floats of scratch fwp_rec_bwd_static has per GPU */
 };
 
 const char *fwp_strerror(int code);
@@ -255,6 +257,25 @@ int fwp_rec_bwd(const float *q_act, const float *k_act, const float *beta_act,
                 float *gkx, float *gvx, float *gbx, float *gRq, float *gRk,
                 float *gRv, float *grb, float *workspace, int N, int H, int L,
                 int D, int chunk, void *stream);
+
+/*
+ * fwp_rec_bwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  Same arguments
+ * and results as fwp_rec_bwd without `workspace`: the per-sequence partial sums go to a fixed array
+ * inside the library (8 MiB on every GPU the library runs on, held until the process ends) and the
+ * call allocates and frees nothing.  Limit: N*H*(3*D*D+D) <= fwp_query(FWP_Q_STATIC_SCRATCH_FLOATS)
+ * (2 Mi floats; B=64 H=8 D=32 needs 1.6 Mi), else FWP_E_SCRATCH and nothing is launched.
+ * All calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads)
+ * race; calls on one stream are ordered and safe.  Nothing needs clearing between calls: every
+ * call overwrites the part it reads.  The array's address is looked up on a GPU's first call (or by
+ * fwp_check_device); make that call once before opening a graph capture.
+ */
+int fwp_rec_bwd_static(const float *q_act, const float *k_act, const float *beta_act,
+                       const float *vdiff, const float *out, const float *h_init,
+                       fwp_view grad_out, const float *Rq, const float *Rk, const float *Rv,
+                       const float *rb, const float *ckpt, float *gqx, float *gkx, float *gvx,
+                       float *gbx, float *gRq, float *gRk, float *gRv, float *grb, int N, int H,
+                       int L, int D, int chunk, void *stream);
 
 #ifdef __cplusplus
 }

@@ -39,6 +39,7 @@ _SIGNATURES = {
     "fwp_deltanet_prep_bwd": [_P] * 6 + [_I] * 4 + [_P],
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
+    "fwp_rec_bwd_static": [_P] * 6 + [_V] + [_P] * 13 + [_I] * 5 + [_P],
 }
 EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
                                        "fwp_delta_ckpt_floats", "fwp_delta_kind"])
@@ -87,7 +88,7 @@ def query(what):
 
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
-Q_MAX_D_RNN, Q_MAX_D_REC, Q_MAX_D_LSTM = 4, 5, 6
+Q_MAX_D_RNN, Q_MAX_D_REC, Q_MAX_D_LSTM, Q_STATIC_SCRATCH_FLOATS = 4, 5, 6, 7
 
 
 _ckpt_floats_cache = {}

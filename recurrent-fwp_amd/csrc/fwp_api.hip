@@ -109,6 +109,7 @@ const char *fwp_strerror(int code) {
         case FWP_E_CHUNK: return "chunk is not a positive multiple of the chunk quantum";
         case FWP_E_TOO_LARGE: return "the fast-weight state does not fit the workgroup's LDS";
         case FWP_E_ARCH: return "the current device is not a gfx950 (MI355X) part";
+        case FWP_E_SCRATCH: return "the call needs more scratch memory than the library's fixed scratch array holds";
         default: break;
     }
     if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -121,6 +122,7 @@ int fwp_query(int what) {
         case FWP_Q_CHUNK_QUANTUM: return kChunkQuantum;
         case FWP_Q_DEFAULT_CHUNK: return kDefaultChunk;
         case FWP_Q_MAX_STATE_FLOATS: return 16384;
+        case FWP_Q_STATIC_SCRATCH_FLOATS: return static_scratch_floats();
         case FWP_Q_MAX_D_RNN: return generic_max_dim(0);
         case FWP_Q_MAX_D_REC: return generic_max_dim(1);
         case FWP_Q_MAX_D_LSTM: return generic_max_dim(2);
@@ -140,7 +142,8 @@ int fwp_check_device(void) {
     hipDeviceProp_t p;
     e = hipGetDeviceProperties(&p, dev);
     if (e != hipSuccess) return (int)e;
-    return strncmp(p.gcnArchName, "gfx950", 6) == 0 ? FWP_OK : FWP_E_ARCH;
+    if (strncmp(p.gcnArchName, "gfx950", 6) != 0) return FWP_E_ARCH;
+    return static_scratch_init();        // per-device set-up of the entry point that allocates nothing
 }
 
 int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,

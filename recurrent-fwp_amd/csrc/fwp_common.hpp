@@ -65,6 +65,11 @@ int reduce_rec_param_grads(const float *workspace, float *gRq, float *gRk, float
 // (op: 0 Delta RNN, 1 Recurrent Delta Net, 2 Delta LSTM).
 int generic_max_dim(int op);
 
+// The fixed scratch array of fwp_rec_bwd_static: address lookup for the current device (once per
+// device; 0 or an error code) and its size in floats.
+int static_scratch_init();
+int static_scratch_floats();
+
 // Register-state kernels (one wave per sequence): E = M = D in {16, 32}, 16-byte aligned rows.
 bool reg_view_ok(const fwp_view &v);
 bool reg_delta_supported(int E, int M);
