@@ -35,6 +35,14 @@ typedef struct fwp_view {
     int64_t sN, sH, sL; /* strides in elements; last-axis stride is 1 */
 } fwp_view;
 
+/* An output tensor [N,H,L,M] that need not be contiguous: element strides of the N, H and L axes
+ * (last axis contiguous).  Lets fwp_delta_fwd_strided write rows where the caller's next operation
+ * wants them, e.g. [L,N,H*M] storage (sN = H*M, sH = M, sL = N*H*M). */
+typedef struct fwp_out_view {
+    float *ptr;
+    int64_t sN, sH, sL;
+} fwp_out_view;
+
 enum {
     FWP_OK = 0,
     FWP_E_NULL = -1,      /* a required pointer is NULL */
@@ -115,6 +123,16 @@ long long fwp_delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);
 int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,
                   float *out, float *vdiff, float *ckpt, int N, int H, int L,
                   int E, int M, int chunk, void *stream);
+
+/*
+ * fwp_delta_fwd with `out` given as a strided view.  The reference's layers permute and reshape the
+ * operator's [N,H,L,M] output to [L,N,H*M] right after the call
+ * (language_modeling/src/utils/cuda_fast_weight_layer.py:158-163, a copy there); written through a view
+ * of [L,N,H,M] storage that step is free.  Rows of the view must not overlap.
+ */
+int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,
+                          fwp_out_view out, float *vdiff, float *ckpt, int N, int H, int L,
+                          int E, int M, int chunk, void *stream);
 
 /*
  * Delta rule backward.  Replaces fast_weight_backward
@@ -215,17 +233,20 @@ int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff,
  * projection and its call of the operator
  * (language_modeling/src/utils/cuda_fast_weight_layer.py:108-125): from qkvb [T,B,H,3D+1]
  * (contiguous; per head q | k | v | beta logit) to the operator's inputs, contiguous [B,H,T,.]:
- *   q, k = (elu(x) + 1) / sum_D(elu(x) + 1)    v = copy    beta = sigmoid(logit)
- * D must be 16, 32 or 64 (FWP_E_SHAPE otherwise).
+ *   q = q_scale (elu(x) + 1) / sum_D(elu(x) + 1)    k likewise without the scale    v = copy
+ *   beta = sigmoid(logit)
+ * q_scale: the layer multiplies the operator's output by 1/sqrt(D) (:155-157); that output is linear
+ * in q, so passing the factor here gives the same result without a pass over the output (1 for the
+ * reference's q).  D must be 16, 32 or 64 (FWP_E_SHAPE otherwise).
  */
 int fwp_deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta,
-                          int T, int B, int H, int D, void *stream);
+                          int T, int B, int H, int D, float q_scale, void *stream);
 
 /* Adjoint of fwp_deltanet_prep_fwd: gradients of q, k, v, beta ([B,H,T,.] contiguous) to the
  * gradient of qkvb [T,B,H,3D+1] (every element written). */
 int fwp_deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
                           const float *gbeta, float *gqkvb, int T, int B, int H, int D,
-                          void *stream);
+                          float q_scale, void *stream);
 
 /*
  * Recurrent Delta Net forward.  Replaces rec_update_fwm_tanh_forward

@@ -20,6 +20,12 @@ class View(ctypes.Structure):
                 ("sL", ctypes.c_int64)]
 
 
+class OutView(ctypes.Structure):
+    """struct fwp_out_view: a strided [N,H,L,M] output."""
+    _fields_ = [("ptr", ctypes.c_void_p), ("sN", ctypes.c_int64), ("sH", ctypes.c_int64),
+                ("sL", ctypes.c_int64)]
+
+
 class FwpError(RuntimeError):
     pass
 
@@ -35,8 +41,9 @@ _SIGNATURES = {
     "fwp_rnn_bwd": [_V, _V, _P, _P, _P, _V, _P] + [_P] * 4 + [_I] * 5 + [_P],
     "fwp_lstm_fwd": [_VP] * 4 + [_P] * 8 + [_I] * 5 + [_P],
     "fwp_lstm_bwd": [_VP] * 2 + [_P] * 6 + [_V] + [_P] * 5 + [_I] * 5 + [_P],
-    "fwp_deltanet_prep_fwd": [_P] * 5 + [_I] * 4 + [_P],
-    "fwp_deltanet_prep_bwd": [_P] * 6 + [_I] * 4 + [_P],
+    "fwp_deltanet_prep_fwd": [_P] * 5 + [_I] * 4 + [ctypes.c_float, _P],
+    "fwp_deltanet_prep_bwd": [_P] * 6 + [_I] * 4 + [ctypes.c_float, _P],
+    "fwp_delta_fwd_strided": [_V] * 4 + [_P, OutView] + [_P] * 2 + [_I] * 6 + [_P],
     "fwp_rec_fwd": [_V] * 4 + [_P] * 12 + [_I] * 5 + [_P],
     "fwp_rec_bwd": [_P] * 6 + [_V] + [_P] * 14 + [_I] * 5 + [_P],
     "fwp_rec_bwd_static": [_P] * 6 + [_V] + [_P] * 13 + [_I] * 5 + [_P],

@@ -118,7 +118,7 @@ const char *fwp_strerror(int code) {
 
 int fwp_query(int what) {
     switch (what) {
-        case FWP_Q_VERSION: return 1;
+        case FWP_Q_VERSION: return 2;
         case FWP_Q_CHUNK_QUANTUM: return kChunkQuantum;
         case FWP_Q_DEFAULT_CHUNK: return kDefaultChunk;
         case FWP_Q_MAX_STATE_FLOATS: return 16384;
@@ -146,14 +146,16 @@ int fwp_check_device(void) {
     return static_scratch_init();        // per-device set-up of the entry point that allocates nothing
 }
 
-int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
-                  float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
-                  void *stream) {
-    if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(beta) || !W || !out)
+int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
+                          float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
+                          void *stream) {
+    if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(beta) || !W || !out.ptr)
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(out);
+    // the output view takes part in the choice of kernels like an input read 16 bytes at a time
+    const fwp_view ov = {out.ptr, out.sN, out.sH, out.sL};
+    const bool aligned = aligned16(vdiff) && aligned16(ckpt) && reg_view_ok(ov) && in_range32(L, E, M, {ov});
     switch (delta_kind(false, aligned, q, k, v, beta, N, H, L, E, M)) {
         case FWP_KIND_PHASE:
             return phase_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, chunk, (hipStream_t)stream);
@@ -168,6 +170,14 @@ int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, f
     if (int rc = delta_aux_invalidate(ckpt, N, H, L, E, M, chunk, (hipStream_t)stream)) return rc;
     return generic_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk,
                              (hipStream_t)stream);
+}
+
+int fwp_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+                  float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
+                  void *stream) {
+    if (!out) return FWP_E_NULL;
+    return fwp_delta_fwd_strided(q, k, v, beta, W, contiguous_out(out, H, L, M), vdiff, ckpt, N, H, L, E, M,
+                                 chunk, stream);
 }
 
 int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view grad_out,
@@ -311,17 +321,18 @@ int fwp_lstm_bwd(const fwp_view *k, const fwp_view *beta, const float *vdiff, co
 }
 
 int fwp_deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B,
-                          int H, int D, void *stream) {
+                          int H, int D, float q_scale, void *stream) {
     if (!qkvb || !q || !k || !v || !beta) return FWP_E_NULL;
     if (T < 1 || B < 1 || H < 1 || !prep_supported(D)) return FWP_E_SHAPE;
-    return deltanet_prep_fwd(qkvb, q, k, v, beta, T, B, H, D, (hipStream_t)stream);
+    return deltanet_prep_fwd(qkvb, q, k, v, beta, T, B, H, D, q_scale, (hipStream_t)stream);
 }
 
 int fwp_deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
-                          const float *gbeta, float *gqkvb, int T, int B, int H, int D, void *stream) {
+                          const float *gbeta, float *gqkvb, int T, int B, int H, int D, float q_scale,
+                          void *stream) {
     if (!qkvb || !gq || !gk || !gv || !gbeta || !gqkvb) return FWP_E_NULL;
     if (T < 1 || B < 1 || H < 1 || !prep_supported(D)) return FWP_E_SHAPE;
-    return deltanet_prep_bwd(qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, D, (hipStream_t)stream);
+    return deltanet_prep_bwd(qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, D, q_scale, (hipStream_t)stream);
 }
 
 int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq,

@@ -17,6 +17,11 @@ __device__ __forceinline__ const float *row(const fwp_view &v, int n, int h, int
     return v.ptr + (int64_t)n * v.sN + (int64_t)h * v.sH + (int64_t)t * v.sL;
 }
 
+// A contiguous [N,H,L,M] output as the view the delta-rule forward kernels write through.
+inline fwp_out_view contiguous_out(float *p, int H, int L, int M) {
+    return fwp_out_view{p, (int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
+}
+
 // Per-gate arguments of the Delta LSTM kernels, gate order i (input), u (update), o (output).
 struct LstmGates {
     fwp_view z[3], k[3], v[3], beta[3];
@@ -24,7 +29,7 @@ struct LstmGates {
 };
 
 // Launchers of the LDS-state kernels (any E, M that fit the LDS).
-int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                       float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
                       hipStream_t s);
 int generic_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
@@ -73,14 +78,14 @@ int static_scratch_floats();
 // Register-state kernels (one wave per sequence): E = M = D in {16, 32}, 16-byte aligned rows.
 bool reg_view_ok(const fwp_view &v);
 bool reg_delta_supported(int E, int M);
-int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                   float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
 int reg_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                   const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                   int L, int D, int chunk, hipStream_t s);
 
 // Chunked delta-rule forward on the matrix cores (same arguments and results as reg_delta_fwd).
-int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s);
 
 // Size of the delta rule's checkpoint buffer: the states, plus (shapes of the blocked kernels) a header and one
@@ -94,7 +99,7 @@ float *delta_aux_of(const float *ckpt, int N, int H, int L, int E, int M, int ch
 // arguments, results and auxiliary buffer as mfma_delta_fwd / mfma_delta_bwd).
 bool split_delta_supported(int L);
 bool split_delta_dims(int E, int M);      // E = 16 NE, M = 16 NM for the instantiated (NE, NM)
-int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                     float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s);
 int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                     const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
@@ -102,7 +107,7 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
 // 16 x 16 states with the blocks of a sequence prepared in parallel by the waves of a workgroup and one
 // product per block on the sequential chain (same arguments, results and saved buffers as split_delta_fwd).
 bool phase_delta_dims(int E, int M);
-int phase_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
+int phase_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out, float *vdiff,
                     float *ckpt, int N, int H, int L, int chunk, hipStream_t s);
 int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
@@ -157,9 +162,9 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
 // Fused pre-step of the Delta-Net layer and its adjoint (D in {16, 32, 64}).
 bool prep_supported(int D);
 int deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B, int H,
-                      int D, hipStream_t s);
+                      int D, float q_scale, hipStream_t s);
 int deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
-                      const float *gbeta, float *gqkvb, int T, int B, int H, int D, hipStream_t s);
+                      const float *gbeta, float *gqkvb, int T, int B, int H, int D, float q_scale, hipStream_t s);
 
 // Largest dynamic LDS allocation the LDS-state kernels ask for (bytes).
 constexpr size_t kMaxLds = 160 * 1024 - 1024;

@@ -58,7 +58,7 @@ struct FwdLds {
 template <int NE, int NM>   // state E = 16 NE by M = 16 NM
 __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, fwp_view k, fwp_view v,
                                                        fwp_view beta, float *__restrict__ W,
-                                                       float *__restrict__ out,
+                                                       fwp_out_view out,
                                                        float *__restrict__ vdiff,
                                                        float *__restrict__ ckpt,
                                                        float *__restrict__ aux, int nseq, int H,
@@ -85,15 +85,16 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
         kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
         vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
         bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
-        ob(out + seq * L * M, (uint32_t)(L * M * 4)),
+        ob(out.ptr + n * out.sN + h * out.sH, (uint32_t)(((L - 1) * out.sL + M) * 4)),
         db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0),
         tb(aux ? aux + kAuxHeader + seq * nblk * 256 : nullptr, aux ? (uint32_t)(nblk * 1024) : 0);
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
-                   m_step = (unsigned)(kBlk * M * 4);
+                   m_step = (unsigned)(kBlk * M * 4), out_step = (unsigned)(kBlk * out.sL * 4);
     const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
                    o_bc = (unsigned)(c * beta.sL) * 4;
-    const unsigned o_vt = (unsigned)(c * v.sL + 4 * g) * 4, o_out = (unsigned)(c * M + 4 * g) * 4;
+    const unsigned o_vt = (unsigned)(c * v.sL + 4 * g) * 4, o_out = (unsigned)(c * out.sL + 4 * g) * 4,
+                   o_dt = (unsigned)(c * M + 4 * g) * 4;
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     // A block past the end is read at index nblk: every row beyond the buffers, all zeros.
     auto load = [&](FwdRaw<NE, NM> &w, int ib) {
@@ -182,7 +183,7 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
 #pragma unroll
             for (int eb = 0; eb < NE; eb++) S[eb][mb] = tn(Kc[eb], U, S[eb][mb]);
             const v4f O = tn(U, Rm, Ot);          // register r = O[t0 + c][16 mb + 4g + r]
-            ob.st4(O, o_out + 64 * mb, ib * m_step);
+            ob.st4(O, o_out + 64 * mb, ib * out_step);
             if (vdiff) {
                 // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division
                 // where the block's betas allow it
@@ -198,7 +199,7 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
                     Dd = X - tn(Gu, U, zero);
                 }
                 tr[2].put_t(p, Dd);        // leaves like O
-                db.st4(tr[2].get(lane), o_out + 64 * mb, ib * m_step);
+                db.st4(tr[2].get(lane), o_dt + 64 * mb, ib * m_step);
             }
         }
         if (ckpt && ib < nblk && (chunk_of.closes(ib) || ib + 1 == nblk)) {
@@ -502,7 +503,7 @@ int delta_aux_invalidate(float *ckpt, int N, int H, int L, int E, int M, int chu
     return (int)hipGetLastError();
 }
 
-int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                    float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     float *aux = delta_aux_of(ckpt, N, H, L, D, D, chunk);

@@ -50,7 +50,7 @@ struct PhaseKeep {
 
 __global__ __launch_bounds__(64 * kPhWaves) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void k_delta_fwd_phase(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *__restrict__ W,
-                       float *__restrict__ out, float *__restrict__ vdiff, float *__restrict__ ckpt,
+                       fwp_out_view out, float *__restrict__ vdiff, float *__restrict__ ckpt,
                        float *__restrict__ aux, int H, int L, int chunk, int nchunk) {
     constexpr int E = 16, M = 16;
     // per block of the span: P^T; B, and once the chain has passed the block its starting state
@@ -66,18 +66,18 @@ void k_delta_fwd_phase(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float 
         kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
         vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
         bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4));
-    const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4)),
+    const RowBuf ob(out.ptr + n * out.sN + h * out.sH, (uint32_t)(((L - 1) * out.sL + M) * 4)),
         db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0);
     const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
                    v_step = (unsigned)(kBlk * v.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
-                   m_step = (unsigned)(kBlk * M * 4);
+                   m_step = (unsigned)(kBlk * M * 4), out_step = (unsigned)(kBlk * out.sL * 4);
     const int nblk = (L + kBlk - 1) / kBlk;
     const RowBuf tb(aux ? aux + kAuxHeader + seq * nblk * 256 : nullptr, aux ? (uint32_t)(nblk * 1024) : 0);
     // row c of a block, columns 4g .. 4g + 3: one 16-byte load per lane gives the transposed matrix
     // in the accumulator layout
     const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
                    o_vt = (unsigned)(c * v.sL + 4 * g) * 4, o_bc = (unsigned)(c * beta.sL) * 4;
-    const unsigned o_out = (unsigned)(c * M + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + c) * 4;
+    const unsigned o_out = (unsigned)(c * out.sL + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + c) * 4;
     const v4f zero = {0.f, 0.f, 0.f, 0.f};
     v4f ident;
 #pragma unroll
@@ -200,7 +200,7 @@ void k_delta_fwd_phase(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float 
             const v4f U = tn(keep[j].nWt, S0, keep[j].Uh);        // Uh - W S
             v4f Ot = tn(S0, keep[j].Qt, zero);                    // O^T = S^T Q^T + U^T lower(Q K^T)^T
             Ot = tn(U, keep[j].Rm, Ot);                           // register r = O[t0 + c][4g + r]
-            ob.st4(Ot, o_out, ib * m_step);
+            ob.st4(Ot, o_out, ib * out_step);
             if (vdiff) {
                 // U = diag(beta)(v - v_old): a division where the block's betas allow it
                 v4f Dd;
@@ -238,7 +238,7 @@ void k_delta_fwd_phase(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float 
 
 bool phase_delta_dims(int E, int M) { return E == 16 && M == 16; }
 
-int phase_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
+int phase_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out, float *vdiff,
                     float *ckpt, int N, int H, int L, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     float *aux = delta_aux_of(ckpt, N, H, L, 16, 16, chunk);

@@ -52,7 +52,7 @@ struct FwdOps {
 template <int D, int RING, int PF, int WPB, bool SUM = false>
 __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_view k, fwp_view v,
                                                          fwp_view beta, float *__restrict__ W,
-                                                         float *__restrict__ out,
+                                                         fwp_out_view out,
                                                          float *__restrict__ vdiff,
                                                          float *__restrict__ ckpt, int H, int L,
                                                          int chunk, int nchunk, int nseq) {
@@ -122,10 +122,10 @@ __global__ __launch_bounds__(kWave * WPB) void k_delta_fwd_reg(fwp_view q, fwp_v
     // memory operations in flight when a tile is committed are at least a tile old.
     const bool store_d = !SUM && (sl & 1);
     float *stage = sout[store_d ? 1 : 0] + col;
-    float *out_rows = out + seq * L * D;
+    float *out_rows = out.ptr + n * out.sN + h * out.sH;
     float *vd_rows = vdiff ? vdiff + seq * L * D : nullptr;
     auto flush = [&](int t0) {
-        flush_tile<D>(sout[0], out_rows, t0, L, lane);
+        flush_tile<D>(sout[0], out_rows, t0, L, lane, out.sL);
         if (vd_rows) flush_tile<D>(sout[1], vd_rows, t0, L, lane);
     };
 
@@ -433,7 +433,7 @@ bool reg_view_ok(const fwp_view &v) {
 
 bool reg_delta_supported(int E, int M) { return E == M && (E == 16 || E == 32); }
 
-int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int reg_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                   float *vdiff, float *ckpt, int N, int H, int L, int D, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     const int nseq = N * H;
@@ -468,10 +468,10 @@ int reg_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
     const fwp_view none = {nullptr, 0, 0, 0};
     if (D == 16)
         hipLaunchKernelGGL((k_delta_fwd_reg<16, 4, 2, 4, true>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                           q, k, v, none, W, out, nullptr, ckpt, H, L, chunk, nchunk, nseq);
+                           q, k, v, none, W, contiguous_out(out, H, L, D), nullptr, ckpt, H, L, chunk, nchunk, nseq);
     else
         hipLaunchKernelGGL((k_delta_fwd_reg<32, 2, 1, 4, true>), dim3((nseq + 3) / 4), dim3(kWave * 4), 0, s,
-                           q, k, v, none, W, out, nullptr, ckpt, H, L, chunk, nchunk, nseq);
+                           q, k, v, none, W, contiguous_out(out, H, L, D), nullptr, ckpt, H, L, chunk, nchunk, nseq);
     return (int)hipGetLastError();
 }
 

@@ -63,7 +63,7 @@ struct OutRaw {
 template <int NE, int NM, int PF, bool OUT>   // E = 16 NE, M = 16 NM, PF = blocks in flight
 __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void k_delta_fwd_split(fwp_view q, fwp_view k, fwp_view v,
                                                                   fwp_view beta, float *__restrict__ W,
-                                                                  float *__restrict__ out,
+                                                                  fwp_out_view out,
                                                                   float *__restrict__ vdiff,
                                                                   float *__restrict__ ckpt,
                                                                   float *__restrict__ aux, int H, int L,
@@ -194,7 +194,9 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
         return;
     }
 
-    const unsigned m_step = (unsigned)(kBlk * M * 4);
+    const unsigned m_step = (unsigned)(kBlk * M * 4), out_step = (unsigned)(kBlk * out.sL * 4);
+    float *const out_rows = out.ptr + n * out.sN + h * out.sH;
+    const uint32_t out_bytes = (uint32_t)(((L - 1) * out.sL + M) * 4);
     if (OUT && wave == NM + 2) {       // the wave that fills the workgroup up to four
         for (int r = 0; r < nblk + 2; r++) lds_barrier();
         return;
@@ -202,8 +204,8 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
     if (OUT && wave == NM + 1) {
         // ------------------------------------------------ output wave, one block behind
         using Raw = OutRaw<NE, !kPrepQK>;
-        const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4));
-        const unsigned o_out = (unsigned)(c * M + 4 * g) * 4;
+        const RowBuf ob(out_rows, out_bytes);
+        const unsigned o_out = (unsigned)(c * out.sL + 4 * g) * 4;
         auto load = [&](Raw &w, int ib) {
             const unsigned ks = ib * k_step, qs = ib * q_step;
 #pragma unroll
@@ -230,7 +232,7 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
 #pragma unroll
                 for (int eb = 0; eb < NE; eb++) Ot = tn(from[eb].get(lane), w.Qt[eb], Ot);   // O^T, state part
                 const v4f O = tn(from[OUT ? NE : 0].get(lane), Rm, Ot);   // register r = O[t0 + c][16 mb + 4g + r]
-                ob.st4(O, o_out + 64 * mb, ib * m_step);
+                ob.st4(O, o_out + 64 * mb, ib * out_step);
             }
         };
         lds_barrier();      // the preparing wave's block 0
@@ -271,8 +273,8 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
 #pragma unroll
         for (int r = 0; r < 4; r++) S[eb][r] = W[(seq * E + 16 * eb + 4 * g + r) * M + 16 * mb + c];
     const ChunkOf chunk_of(chunk);
-    const RowBuf ob(out + seq * L * M, (uint32_t)(L * M * 4)), db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0);
-    const unsigned o_out = (unsigned)(c * M + 16 * mb + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + 16 * mb + c) * 4;
+    const RowBuf ob(out_rows, out_bytes), db(vdiff ? vdiff + seq * L * M : nullptr, vdiff ? (uint32_t)(L * M * 4) : 0);
+    const unsigned o_out = (unsigned)(c * out.sL + 16 * mb + 4 * g) * 4, o_vd = (unsigned)(4 * g * M + 16 * mb + c) * 4;
     const RowBuf tb(aux && mb == 0 ? aux + kAuxHeader + seq * nblk * 256 : nullptr,
                     aux && mb == 0 ? (uint32_t)(nblk * 1024) : 0);
     auto block = [&](int ib, const StateRaw &cur) {
@@ -310,7 +312,7 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
                 for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
             }
             const v4f O = tn(U, Rm, Ot);             // register r = O[t0 + c][16 mb + 4g + r]
-            ob.st4(O, o_out, ib * m_step);
+            ob.st4(O, o_out, ib * out_step);
         }
         if (vdiff) {
             // v - v_old = X - strict_lower(K K^T) U, and U = diag(beta)(v - v_old): a division where
@@ -1028,7 +1030,7 @@ constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
 // 768 / 1024 sequences of 256 steps: 12.5 / 15.0 / 18.2 / 20.7 us with it, 14.8 / 17.4 / 18.2 / 21.7 us
 // without; D = 32, 256 sequences of 1024 steps: 54 against 62 us).
 template <int NE, int NM>
-void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out, float *vdiff,
+void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out, float *vdiff,
                 float *ckpt, float *aux, int nseq, int H, int L, int chunk, int nchunk, hipStream_t s) {
     if constexpr (NM <= 2) {
         if (NM == 1 || (int64_t)nseq * (NM + 2) <= 1536) {
@@ -1054,7 +1056,7 @@ void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_v
 // the (NE, NM) pairs of split_delta_dims
 #define FWP_SPLIT_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2)
 
-int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                     float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk;
     float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);

@@ -70,7 +70,7 @@ __device__ __forceinline__ float dot_lds(const float *a, const float *b, int D) 
 // ---------------------------------------------------------------- delta rule
 
 __global__ __launch_bounds__(NT) void k_delta_fwd(fwp_view q, fwp_view k, fwp_view v,
-                                                  fwp_view beta, float *W, float *out,
+                                                  fwp_view beta, float *W, fwp_out_view out,
                                                   float *vdiff, float *ckpt, int H, int L, int E,
                                                   int M, int chunk, int nchunk) {
     extern __shared__ float lds[];
@@ -95,7 +95,7 @@ __global__ __launch_bounds__(NT) void k_delta_fwd(fwp_view q, fwp_view k, fwp_vi
         rank1(sW, lda, sk, su, E, M, 1.f);
         __syncthreads();
         for (int m = threadIdx.x; m < M; m += NT)
-            out[(seq * L + t) * M + m] = col_dot(sW, lda, sq, E, m);
+            out.ptr[n * out.sN + h * out.sH + t * out.sL + m] = col_dot(sW, lda, sq, E, m);
         if (ckpt && ((t + 1) % chunk == 0 || t == L - 1))
             store_state(ckpt + (seq * nchunk + t / chunk) * E * M, sW, lda, E, M);
     }
@@ -691,7 +691,7 @@ inline int launched() { return (int)hipGetLastError(); }
 
 }  // namespace
 
-int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, float *out,
+int generic_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                       float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk,
                       hipStream_t s) {
     size_t bytes = sizeof(float) * ((size_t)E * pitch(M) + 2 * E + 2 * M);

@@ -2,6 +2,8 @@
 // cuda_fast_weight_layer.py:108-125): from the layer's one projection qkvb[T,B,H,3D+1] straight to
 // the operator's inputs in [B,H,T,.] order,
 //     q, k = (elu(x) + 1) / sum_D(elu(x) + 1)      v = copy      beta = sigmoid
+// (q times a constant on request: the operator's output is linear in q, so the 1/sqrt(D) the layer
+// applies to that output can be applied here, to D values per token instead of a pass of its own)
 // and its adjoint: one pass over the data each way instead of the dozen elementwise, reduction
 // and copy kernels the same lines cost in stock PyTorch.  D lanes per (t, b, h) row; sums over the
 // row are butterfly shuffles inside the wave.
@@ -22,7 +24,7 @@ __device__ __forceinline__ float feature(float x) { return x > 0.f ? x + 1.f : _
 template <int D>
 __global__ __launch_bounds__(256) void k_prep_fwd(const float *__restrict__ qkvb, float *__restrict__ q,
                                                   float *__restrict__ k, float *__restrict__ v,
-                                                  float *__restrict__ beta, int T, int B, int H) {
+                                                  float *__restrict__ beta, int T, int B, int H, float q_scale) {
     constexpr int RPB = 256 / D;                       // rows per block
     const int j = threadIdx.x % D;
     const int64_t r = (int64_t)blockIdx.x * RPB + threadIdx.x / D;     // row in (t, b, h) order
@@ -35,7 +37,7 @@ __global__ __launch_bounds__(256) void k_prep_fwd(const float *__restrict__ qkvb
     const float sq = row_sum<D>(fq), sk = row_sum<D>(fk);
     if (!ok) return;
     const int64_t o = (((int64_t)b * H + h) * T + t) * D + j;
-    q[o] = fq / sq;
+    q[o] = fq / sq * q_scale;
     k[o] = fk / sk;
     v[o] = src[2 * D + j];
     if (j == 0) beta[((int64_t)b * H + h) * T + t] = 1.f / (1.f + __expf(-src[3 * D]));
@@ -47,7 +49,7 @@ __global__ __launch_bounds__(256) void k_prep_bwd(const float *__restrict__ qkvb
                                                   const float *__restrict__ gk,
                                                   const float *__restrict__ gv,
                                                   const float *__restrict__ gbeta,
-                                                  float *__restrict__ gqkvb, int T, int B, int H) {
+                                                  float *__restrict__ gqkvb, int T, int B, int H, float q_scale) {
     constexpr int RPB = 256 / D;
     const int j = threadIdx.x % D;
     const int64_t r = (int64_t)blockIdx.x * RPB + threadIdx.x / D;
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(256) void k_prep_bwd(const float *__restrict__ qkvb
     const float xq = src[j], xk = src[D + j];
     const float fq = feature(xq), fk = feature(xk);
     const float sq = row_sum<D>(fq), sk = row_sum<D>(fk);
-    const float dq = gq[o], dk = gk[o];
+    const float dq = gq[o] * q_scale, dk = gk[o];
     const float cq = row_sum<D>(dq * fq) / sq, ck = row_sum<D>(dk * fk) / sk;      // sum(dy y)
     if (!ok) return;
     dst[j] = (dq - cq) / sq * (xq > 0.f ? 1.f : fq);
@@ -79,27 +81,27 @@ __global__ __launch_bounds__(256) void k_prep_bwd(const float *__restrict__ qkvb
 bool prep_supported(int D) { return D == 16 || D == 32 || D == 64; }
 
 int deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B, int H,
-                      int D, hipStream_t s) {
+                      int D, float q_scale, hipStream_t s) {
     const int64_t rows = (int64_t)T * B * H;
     const int rpb = 256 / D;
     const dim3 grid((unsigned)((rows + rpb - 1) / rpb));
-    if (D == 16) hipLaunchKernelGGL(k_prep_fwd<16>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H);
-    else if (D == 32) hipLaunchKernelGGL(k_prep_fwd<32>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H);
-    else hipLaunchKernelGGL(k_prep_fwd<64>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H);
+    if (D == 16) hipLaunchKernelGGL(k_prep_fwd<16>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H, q_scale);
+    else if (D == 32) hipLaunchKernelGGL(k_prep_fwd<32>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H, q_scale);
+    else hipLaunchKernelGGL(k_prep_fwd<64>, grid, dim3(256), 0, s, qkvb, q, k, v, beta, T, B, H, q_scale);
     return (int)hipGetLastError();
 }
 
 int deltanet_prep_bwd(const float *qkvb, const float *gq, const float *gk, const float *gv,
-                      const float *gbeta, float *gqkvb, int T, int B, int H, int D, hipStream_t s) {
+                      const float *gbeta, float *gqkvb, int T, int B, int H, int D, float q_scale, hipStream_t s) {
     const int64_t rows = (int64_t)T * B * H;
     const int rpb = 256 / D;
     const dim3 grid((unsigned)((rows + rpb - 1) / rpb));
     if (D == 16)
-        hipLaunchKernelGGL(k_prep_bwd<16>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H);
+        hipLaunchKernelGGL(k_prep_bwd<16>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, q_scale);
     else if (D == 32)
-        hipLaunchKernelGGL(k_prep_bwd<32>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H);
+        hipLaunchKernelGGL(k_prep_bwd<32>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, q_scale);
     else
-        hipLaunchKernelGGL(k_prep_bwd<64>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H);
+        hipLaunchKernelGGL(k_prep_bwd<64>, grid, dim3(256), 0, s, qkvb, gq, gk, gv, gbeta, gqkvb, T, B, H, q_scale);
     return (int)hipGetLastError();
 }
 

@@ -157,14 +157,15 @@ struct TileRegs {
 };
 
 // A tile of outputs staged in LDS goes to HBM with 16-byte stores (rows beyond L are dropped).
+// `pitch`: floats between consecutive rows of the destination (D for a contiguous tensor).
 template <int D, int TL = kTile>
 __device__ __forceinline__ void flush_tile(const float *tile, float *dst_rows, int t0, int L,
-                                           int lane) {
+                                           int lane, int64_t pitch = D) {
 #pragma unroll
     for (int i = 0; i < Geo<D, TL>::NV4; i++) {
         const int f = lane + kWave * i, rw = f / (D / 4), c4 = f % (D / 4);
         const float4 x = *reinterpret_cast<const float4 *>(tile + 4 * f);
-        if (t0 + rw < L) *reinterpret_cast<float4 *>(dst_rows + (int64_t)(t0 + rw) * D + 4 * c4) = x;
+        if (t0 + rw < L) *reinterpret_cast<float4 *>(dst_rows + (int64_t)(t0 + rw) * pitch + 4 * c4) = x;
     }
 }
 

@@ -16,6 +16,7 @@
 #include <c10/hip/HIPStream.h>
 
 #include <mutex>
+#include <optional>
 #include <stdexcept>
 #include <string>
 #include <tuple>
@@ -107,7 +108,7 @@ void *stream_of(const at::Tensor &t) { return c10::hip::getCurrentHIPStream(t.ge
 struct DeltaFn : torch::autograd::Function<DeltaFn> {
     static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Q_in,
                               const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &beta_in,
-                              const at::Tensor &W, bool need_grad) {
+                              const at::Tensor &W, bool need_grad, int64_t time_major) {
         require_device(Q_in);
         same_device(Q_in, {K_in, V_in, beta_in, W});
         if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
@@ -118,11 +119,18 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
                  " beta" + shape_of(beta_in));
         if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
             fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+        // out follows Q's memory order unless told otherwise: steps outermost for a permuted view of
+        // [L,N,H,E] storage (the reference's layers), so that their reshape to [L,N,H*M] is a view
+        if (time_major < 0) {
+            const int64_t sN = Q_in.stride(0), sH = Q_in.stride(1), sL = Q_in.stride(2);
+            time_major = L > 1 && (N > 1 || H > 1) && (N <= 1 || sL > sN) && (H <= 1 || sL > sH);
+        }
         fwp_view qv, kv, vv, bv;
         const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), V = rows(V_in, vv), beta = rows(beta_in, bv);
         const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
         const auto opts = Q.options();
-        at::Tensor out = at::empty({N, H, L, M}, opts), saved;
+        at::Tensor out = time_major ? at::empty({L, N, H, M}, opts).permute({1, 2, 0, 3}) : at::empty({N, H, L, M}, opts), saved;
+        const fwp_out_view ov = {out.data_ptr<float>(), out.stride(0), out.stride(1), out.stride(2)};
         float *vdiff = nullptr, *ckpt = nullptr;
         if (need_grad) {
             // v - v_old [N,H,L,M] and the checkpoints behind it, one allocation
@@ -135,9 +143,9 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
         {
             c10::OptionalDeviceGuard guard;
             if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
-            check(fwp_delta_fwd(qv, kv, vv, bv, W.data_ptr<float>(), out.data_ptr<float>(), vdiff, ckpt, (int)N,
-                                (int)H, (int)L, (int)E, (int)M, chunk, stream_of(Q)),
-                  "fwp_delta_fwd");
+            check(fwp_delta_fwd_strided(qv, kv, vv, bv, W.data_ptr<float>(), ov, vdiff, ckpt, (int)N, (int)H,
+                                        (int)L, (int)E, (int)M, chunk, stream_of(Q)),
+                  "fwp_delta_fwd_strided");
         }
         if (need_grad) {
             ctx->save_for_backward({Q, K, beta, saved});
@@ -151,7 +159,7 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
     static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
                                                  torch::autograd::tensor_list grads) {
         const at::Tensor none;
-        if (!grads[0].defined()) return {none, none, none, none, none, none};
+        if (!grads[0].defined()) return {none, none, none, none, none, none, none};
         const auto saved = ctx->get_saved_variables();
         if (saved.size() != 4) fail("backward of a forward pass that kept nothing for it");
         const at::Tensor &Q = saved[0], &K = saved[1], &beta = saved[2], &buf = saved[3];
@@ -175,7 +183,7 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
                                 (int)M, chunk, stream_of(Q)),
                   "fwp_delta_bwd");
         }
-        return {gq, gk, gv, gb, none, none};
+        return {gq, gk, gv, gb, none, none, none};
     }
 };
 
@@ -546,12 +554,13 @@ at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::T
     return SumFn::apply(Q, K, V, W, exact, need_grad);
 }
 
+// time_major: None = out's memory follows Q's, True = [L,N,H,M] storage, False = contiguous [N,H,L,M]
 at::Tensor fast_weight_delta(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V,
-                             const at::Tensor &beta, const at::Tensor &W) {
+                             const at::Tensor &beta, const at::Tensor &W, std::optional<bool> time_major) {
     // decided here: forward itself runs with gradient mode switched off
     const bool need_grad = at::GradMode::is_enabled() &&
                            (Q.requires_grad() || K.requires_grad() || V.requires_grad() || beta.requires_grad());
-    return DeltaFn::apply(Q, K, V, beta, W, need_grad);
+    return DeltaFn::apply(Q, K, V, beta, W, need_grad, time_major.has_value() ? (int64_t)*time_major : (int64_t)-1);
 }
 
 void set_error_class(py::object cls) {
@@ -571,7 +580,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
             PyErr_SetString(PyExc_AssertionError, e.what());
         }
     });
-    m.def("fast_weight_delta", &fast_weight_delta,
+    m.def("fast_weight_delta", &fast_weight_delta, py::arg("Q"), py::arg("K"), py::arg("V"), py::arg("beta"),
+          py::arg("W"), py::arg("time_major") = py::none(),
           "out = fast_weight_delta(Q, K, V, beta, W): delta-rule fast weight memory; W is updated in place");
     m.def("fast_weight_sum", &fast_weight_sum,
           "out = fast_weight_sum(Q, K, V, W, exact): sum-rule fast weight memory; W is updated in place");

@@ -10,6 +10,15 @@ def _nchunk(L, chunk):
     return (L + chunk - 1) // chunk
 
 
+def rows_lead(t):
+    """Is this 4-D [N,H,L,D] tensor a view of storage laid out [L,N,H,...] (the steps outermost), as
+    the reference's layers hand their inputs over (permuted views of a [len, bsz, ...] projection)?"""
+    N, H, L, _ = t.shape
+    sN, sH, sL, _ = t.stride()
+    others = ([sN] if N > 1 else []) + ([sH] if H > 1 else [])
+    return L > 1 and bool(others) and all(sL > s for s in others)
+
+
 class DeltaFastWeight(torch.autograd.Function):
     """``out = fast_weight_delta(Q, K, V, beta, W)``.
 
@@ -17,10 +26,16 @@ class DeltaFastWeight(torch.autograd.Function):
     initial state on entry and the state after the last step on return (in place).
     Gradients flow to Q, K, V and beta; W gets none, as in the reference (:92).
     Unlike the reference, backward leaves W untouched.
+
+    ``out`` has the reference's shape ``[N,H,L,M]``; its memory follows Q's: when Q is a permuted
+    view of ``[L,N,H,E]`` storage, as in the reference's layers, out is a permuted view of
+    ``[L,N,H,M]`` storage, so that their ``transpose(1, 2).reshape(bsz, slen, H * D).transpose(0, 1)``
+    right after the call (cuda_fast_weight_layer.py:158-163) is a view and not a copy.  A sixth
+    argument forces either layout (``True``: steps outermost, ``False``: contiguous ``[N,H,L,M]``).
     """
 
     @staticmethod
-    def forward(ctx, Q, K, V, beta, W):
+    def forward(ctx, Q, K, V, beta, W, time_major=None):
         _lib.require_device(Q)
         _lib.same_device(Q, K, V, beta, W)
         N, H, L, E = Q.shape
@@ -30,13 +45,19 @@ class DeltaFastWeight(torch.autograd.Function):
                                 f"V{tuple(V.shape)} beta{tuple(beta.shape)}")
         if W.shape != (N, H, E, M) or not W.is_contiguous() or W.dtype != torch.float32:
             raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
+        need_grad = any(ctx.needs_input_grad[:4])
+        chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
+        if time_major is None:
+            time_major = rows_lead(Q)
         Q, qv = _lib.rows(Q)
         K, kv = _lib.rows(K)
         V, vv = _lib.rows(V)
         beta, bv = _lib.rows(beta)
-        need_grad = any(ctx.needs_input_grad[:4])
-        chunk = _lib.query(_lib.Q_DEFAULT_CHUNK)
-        out = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
+        if time_major:
+            out = torch.empty((L, N, H, M), device=Q.device, dtype=torch.float32).permute(1, 2, 0, 3)
+        else:
+            out = torch.empty((N, H, L, M), device=Q.device, dtype=torch.float32)
+        ov = _lib.OutView(out.data_ptr(), out.stride(0), out.stride(1), out.stride(2))
         saved = vdiff = ckpt = None
         if need_grad:
             # v - v_old [N,H,L,M] and the checkpoints behind it, one allocation (L*M is a multiple
@@ -47,10 +68,10 @@ class DeltaFastWeight(torch.autograd.Function):
             vdiff = saved.data_ptr()
             ckpt = vdiff + 4 * n_vdiff
         with _lib.on_device(Q):
-            rc = _lib.lib().fwp_delta_fwd(qv, kv, vv, bv, _lib.ptr(W), _lib.ptr(out), vdiff, ckpt,
-                                          N, H, L, E, M, chunk, _lib.stream_of(Q))
+            rc = _lib.lib().fwp_delta_fwd_strided(qv, kv, vv, bv, _lib.ptr(W), ov, vdiff, ckpt,
+                                                  N, H, L, E, M, chunk, _lib.stream_of(Q))
         if rc:
-            _lib.check(rc, "fwp_delta_fwd")
+            _lib.check(rc, "fwp_delta_fwd_strided")
         if need_grad:
             ctx.save_for_backward(Q, K, beta, saved)
             ctx.dims = (N, H, L, E, M, chunk)
@@ -61,7 +82,7 @@ class DeltaFastWeight(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         if grad_out is None:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
         Q, K, beta, saved = ctx.saved_tensors
         N, H, L, E, M, chunk = ctx.dims
         vdiff = saved.data_ptr()
@@ -80,7 +101,7 @@ class DeltaFastWeight(torch.autograd.Function):
                 _lib.stream_of(Q))
         if rc:
             _lib.check(rc, "fwp_delta_bwd")
-        return grad_Q, grad_K, grad_V, grad_beta, None
+        return grad_Q, grad_K, grad_V, grad_beta, None, None
 
 
 def _native():

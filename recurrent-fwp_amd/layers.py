@@ -55,11 +55,12 @@ def sum_normalised_elu(x):
 
 
 class DeltaNetPrep(torch.autograd.Function):
-    """``q, k, v, beta = DeltaNetPrep.apply(qkvb, n_head, d_head)``: the lines between the layer's
+    """``q, k, v, beta = DeltaNetPrep.apply(qkvb, n_head, d_head[, q_scale])``: the lines between the layer's
     projection and the operator (cuda_fast_weight_layer.py:108-125) as one HIP kernel each way.
     ``qkvb`` is the contiguous ``[len, bsz, n_head * (3 d_head + 1)]`` projection; the results are
     contiguous ``[bsz, n_head, len, .]``: q, k through :func:`sum_normalised_elu`, v copied, beta
-    through a sigmoid."""
+    through a sigmoid.  ``q_scale`` multiplies q: the operator's output is linear in q, so the
+    ``1/sqrt(d_head)`` the layer applies to that output (:155-157) can ride here for free."""
 
     @staticmethod
     def supported(qkvb, d_head):
@@ -67,7 +68,7 @@ class DeltaNetPrep(torch.autograd.Function):
                 and d_head in (16, 32, 64))
 
     @staticmethod
-    def forward(ctx, qkvb, n_head, d_head):
+    def forward(ctx, qkvb, n_head, d_head, q_scale=1.0):
         _lib.require_device(qkvb)
         T, B, _ = qkvb.shape
         H, D = n_head, d_head
@@ -76,24 +77,25 @@ class DeltaNetPrep(torch.autograd.Function):
         beta = torch.empty((B, H, T, 1), **f32)
         with _lib.on_device(qkvb):
             rc = _lib.lib().fwp_deltanet_prep_fwd(qkvb.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                                  beta.data_ptr(), T, B, H, D, _lib.stream_of(qkvb))
+                                                  beta.data_ptr(), T, B, H, D, float(q_scale),
+                                                  _lib.stream_of(qkvb))
         _lib.check(rc, "fwp_deltanet_prep_fwd")
         ctx.save_for_backward(qkvb)
-        ctx.dims = (T, B, H, D)
+        ctx.dims = (T, B, H, D, float(q_scale))
         return q, k, v, beta
 
     @staticmethod
     def backward(ctx, gq, gk, gv, gbeta):
         (qkvb,) = ctx.saved_tensors
-        T, B, H, D = ctx.dims
+        T, B, H, D, q_scale = ctx.dims
         gq, gk, gv, gbeta = (g.contiguous() for g in (gq, gk, gv, gbeta))
         gqkvb = torch.empty_like(qkvb)
         with _lib.on_device(qkvb):
             rc = _lib.lib().fwp_deltanet_prep_bwd(qkvb.data_ptr(), gq.data_ptr(), gk.data_ptr(), gv.data_ptr(),
-                                                  gbeta.data_ptr(), gqkvb.data_ptr(), T, B, H, D,
+                                                  gbeta.data_ptr(), gqkvb.data_ptr(), T, B, H, D, q_scale,
                                                   _lib.stream_of(qkvb))
         _lib.check(rc, "fwp_deltanet_prep_bwd")
-        return gqkvb, None, None
+        return gqkvb, None, None, None
 
 
 class DeltaNetLayer(nn.Module):
@@ -132,14 +134,17 @@ class DeltaNetLayer(nn.Module):
         residual = x
 
         qkvb = self.qkvb_net(x)
-        if self.fast_weight_op is fast_weight_delta and DeltaNetPrep.supported(qkvb, D):
-            q, k, v, beta = DeltaNetPrep.apply(qkvb, H, D)       # one fused kernel each way
+        hip_op = self.fast_weight_op is fast_weight_delta
+        fused = hip_op and DeltaNetPrep.supported(qkvb, D)
+        if fused:
+            # one fused kernel each way; q carries the 1/sqrt(D) of the read-out (the operator is
+            # linear in q), and the operator writes [len, bsz, H, D] storage: no pass over its output
+            q, k, v, beta = DeltaNetPrep.apply(qkvb, H, D, self.scale)
         else:
             qkvb = qkvb.view(slen, bsz, H, 3 * D + 1)
             q, k, v, beta = (t.permute(1, 2, 0, 3) for t in qkvb.split((D, D, D, 1), dim=-1))
             q, k, beta = sum_normalised_elu(q), sum_normalised_elu(k), torch.sigmoid(beta)
 
-        hip_op = self.fast_weight_op is fast_weight_delta
         if hip_op and q.dtype != torch.float32:
             # half or bf16 activations (autocast): the operator and its state are fp32, as the
             # reference's kernel and its torch.zeros state are
@@ -153,8 +158,12 @@ class DeltaNetLayer(nn.Module):
             # operator overwrites its state argument, so it gets storage of its own.
             W = mems[0][:bsz].clone()
 
-        out = self.fast_weight_op(q, k, v, beta, W)                  # [bsz, H, slen, D]
-        out = (self.scale * out).permute(2, 0, 1, 3).reshape(slen, bsz, H * D).to(x.dtype)
+        if fused:
+            out = fast_weight_delta(q, k, v, beta, W, True)          # [bsz, H, slen, D] over [slen, bsz, H, D] storage
+            out = out.permute(2, 0, 1, 3).reshape(slen, bsz, H * D)  # a view
+        else:
+            out = self.fast_weight_op(q, k, v, beta, W)              # [bsz, H, slen, D]
+            out = (self.scale * out).permute(2, 0, 1, 3).reshape(slen, bsz, H * D).to(x.dtype)
         out = residual + self.drop(self.o_net(out))
         if not self.pre_lnorm:
             out = self.layer_norm(out)

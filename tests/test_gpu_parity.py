@@ -297,3 +297,69 @@ def test_rejects_cpu_tensors_and_bad_shapes(fwp):
         fwp.fast_weight_delta(dev(q), dev(k[:, :, :3]), dev(v), dev(beta), dev(W0))
     with pytest.raises(AssertionError):
         fwp.fast_rnn_v2(dev(v), dev(k), dev(v), dev(W0), dev(beta), dev(v[:, :, :1, :3]))
+
+
+# ------------------------------------------------------------------ output layout
+
+TIME_MAJOR_SHAPES = [
+    (2, 3, 130, 16, 16),     # blocked kernels, ragged last block
+    (2, 2, 256, 32, 32),
+    (1, 2, 1, 16, 16),       # single step: scan kernels
+    (2, 3, 20, 16, 16),      # short: scan kernels
+    (2, 2, 37, 32, 97),      # LDS-state kernels, rows of 97 floats
+    (1, 1, 20, 5, 3),
+    (2, 3, 80, 96, 16),      # rectangular state on the several-wave kernels
+]
+
+
+@pytest.mark.parametrize("N,H,L,E,M", TIME_MAJOR_SHAPES)
+def test_delta_output_with_steps_outermost(fwp, delta_kernels, N, H, L, E, M):
+    """The operator writes its [N,H,L,M] result into [L,N,H,M] storage on request, and by itself when Q
+    is a view of storage laid out that way (the reference's layers: cuda_fast_weight_layer.py:108-116
+    hand over permuted views and reshape the result to [L,N,H*M], :158-163)."""
+    q, k, v, beta, W0, go = delta_inputs(900 + L + E + M, N, H, L, E, M, w0=True)
+    ref_out, ref_W = oracle.delta_fwd(q, k, v, beta, W0)
+    ref_g = oracle.delta_bwd(q, k, v, beta, W0, go)
+    # asked for
+    ts = [dev(x, True) for x in (q, k, v, beta)]
+    W = dev(W0)
+    out = fwp.fast_weight_delta(*ts, W, True)
+    assert out.shape == (N, H, L, M) and out.permute(2, 0, 1, 3).is_contiguous()
+    check("out", out, ref_out)
+    check("W", W, ref_W)
+    out.permute(2, 0, 1, 3).reshape(L, N, H * M).backward(
+        dev(np.ascontiguousarray(np.transpose(go, (2, 0, 1, 3))).reshape(L, N, H * M)))
+    for name, t, r in zip("q k v beta".split(), ts, ref_g):
+        check("grad_" + name, t.grad, r)
+    # following Q: views of [L,N,H,*] storage in, a view of [L,N,H,M] storage out; contiguous in, contiguous out
+    lead = [dev(np.ascontiguousarray(np.transpose(x, (2, 0, 1, 3)))) for x in (q, k, v, beta)]
+    out2 = fwp.fast_weight_delta(*(t.permute(1, 2, 0, 3) for t in lead), dev(W0))
+    if L > 1 and N * H > 1:
+        assert out2.permute(2, 0, 1, 3).is_contiguous()
+    check("out (views in)", out2, ref_out)
+    out3 = fwp.fast_weight_delta(*(dev(x) for x in (q, k, v, beta)), dev(W0))
+    assert out3.is_contiguous()
+    out4 = fwp.fast_weight_delta(*(t.permute(1, 2, 0, 3) for t in lead), dev(W0), False)
+    assert out4.is_contiguous()
+    check("out (views in, contiguous out)", out4, ref_out)
+
+
+@pytest.mark.parametrize("N,H,L,D", [(2, 3, 100, 16), (2, 2, 70, 32), (1, 2, 9, 32), (2, 2, 40, 24)])
+def test_delta_forward_through_the_c_abi_into_a_wider_buffer(fwp, delta_kernels, N, H, L, D):
+    """fwp_delta_fwd_strided: rows of the result land inside a wider [N,H,L,D+16] buffer whose other
+    columns stay as they were."""
+    L_ = fwp._lib
+    lib = L_.lib()
+    q, k, v, beta, W0, _ = delta_inputs(950 + L + D, N, H, L, D, D, dtype=np.float32, w0=True)
+    want, want_W = oracle.delta_fwd(*(a.astype(np.float64) for a in (q, k, v, beta, W0)))
+    tq, tk, tv, tb, W = (torch.from_numpy(a).cuda() for a in (q, k, v, beta, W0))
+    wide = torch.full((N, H, L, D + 16), -7.0, device="cuda")
+    view = lambda t: L_.View(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
+    window = wide[..., 8:8 + D]          # 32-byte offset: rows stay 16-byte aligned
+    ov = L_.OutView(window.data_ptr(), window.stride(0), window.stride(1), window.stride(2))
+    L_.check(lib.fwp_delta_fwd_strided(view(tq), view(tk), view(tv), view(tb), L_.ptr(W), ov, None, None,
+                                       N, H, L, D, D, L_.query(L_.Q_DEFAULT_CHUNK), L_.stream_of(tq)), "fwd")
+    torch.cuda.synchronize()
+    check("out", window, want)
+    check("W", W, want_W)
+    assert bool((wide[..., :8] == -7.0).all()) and bool((wide[..., 8 + D:] == -7.0).all())

@@ -248,18 +248,19 @@ def test_gpu_lm_at_benchmark_size_against_loop_operator(pkg):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("scale", [1.0, 0.25])
 @pytest.mark.parametrize("D", [16, 32, 64])
-def test_gpu_fused_pre_step_against_the_pytorch_lines(pkg, D):
+def test_gpu_fused_pre_step_against_the_pytorch_lines(pkg, D, scale):
     from importlib import import_module
     layers = import_module(pkg.__name__ + ".layers")
     T, B, H = 37, 3, 5
     torch.manual_seed(D)
     qkvb = (torch.randn(T, B, H * (3 * D + 1), device="cuda") * 2).requires_grad_(True)
     ref_in = qkvb.detach().double().requires_grad_(True)
-    got = pkg.DeltaNetPrep.apply(qkvb, H, D)
+    got = pkg.DeltaNetPrep.apply(qkvb, H, D, scale)
     x = ref_in.view(T, B, H, 3 * D + 1)
     q, k, v, beta = (t.permute(1, 2, 0, 3) for t in x.split((D, D, D, 1), dim=-1))
-    want = (layers.sum_normalised_elu(q), layers.sum_normalised_elu(k), v, torch.sigmoid(beta))
+    want = (scale * layers.sum_normalised_elu(q), layers.sum_normalised_elu(k), v, torch.sigmoid(beta))
     gs = [torch.randn_like(w) for w in want]
     for name, a, b in zip("q k v beta".split(), got, want):
         assert a.is_contiguous() and a.shape == b.shape

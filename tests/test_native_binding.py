@@ -28,17 +28,18 @@ def test_binding_refuses_what_the_python_function_refuses(fwp):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("N,H,L,E,M", [(2, 2, 64, 16, 16), (2, 3, 130, 32, 32), (1, 2, 37, 24, 8), (1, 2, 1, 16, 16)])
-def test_same_as_python_function(fwp, N, H, L, E, M):
+@pytest.mark.parametrize("time_major", [None, True, False])
+def test_same_as_python_function(fwp, N, H, L, E, M, time_major):
     q, k, v, beta, W0, go = (torch.from_numpy(a).cuda() for a in delta_inputs(3, N, H, L, E, M, dtype=np.float32))
     results = []
     for f in (native(fwp).fast_weight_delta, fwp.DeltaFastWeight.apply):
         ins = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
         W = W0.clone()
-        out = f(*ins, W)
+        out = f(*ins, W) if time_major is None else f(*ins, W, time_major)
         grads = torch.autograd.grad(out, ins, go)
         results.append([out, W, *grads])
     for a, b in zip(*results):
-        assert torch.equal(a, b)
+        assert torch.equal(a, b) and a.stride() == b.stride()
 
 
 @pytest.mark.gpu
