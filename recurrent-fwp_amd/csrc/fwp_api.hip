@@ -80,6 +80,11 @@ int delta_kind(bool backward, bool aligned, const fwp_view &q, const fwp_view &k
         return delta_phase(backward, L, E, M) ? FWP_KIND_PHASE : FWP_KIND_SPLIT;
     if (aligned && reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x))
         return delta_chunked(L) && in_range32(L, E, M, {q, k, x, beta}) ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
+    // keys of 128 features: the one-wave blocked kernels at any length (their only alternative is the
+    // LDS-state kernels)
+    if (aligned && wide_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x) &&
+        in_range32(L, E, M, {q, k, x, beta}))
+        return FWP_KIND_CHUNKED;
     return FWP_KIND_LDS;
 }
 
@@ -162,6 +167,8 @@ int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, flo
         case FWP_KIND_SPLIT:
             return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         case FWP_KIND_CHUNKED:
+            if (wide_delta_dims(E, M))
+                return mfma_delta_wide_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
         case FWP_KIND_SCAN:
             return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
@@ -193,6 +200,9 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
             return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
                                    (hipStream_t)stream);
         case FWP_KIND_CHUNKED:
+            if (wide_delta_dims(E, M))
+                return mfma_delta_wide_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
+                                           chunk, (hipStream_t)stream);
             return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, chunk,
                                   (hipStream_t)stream);
         case FWP_KIND_SCAN:

@@ -116,4 +116,61 @@ def _native():
 
 
 _fwp_torch = _native()
-fast_weight_delta = _fwp_torch.fast_weight_delta if _fwp_torch is not None else DeltaFastWeight.apply
+_operator = _fwp_torch.fast_weight_delta if _fwp_torch is not None else DeltaFastWeight.apply
+
+# Value widths the blocked kernels take for a given key width (fwp_delta_kind names the kernels).
+_FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16,)}
+_plans = {}
+
+
+def column_plan(E, M):
+    """How a state of E x M is run when no fast kernel takes it whole: ``None`` (run it as it is) or a
+    list of ``(first, last, width)``: value columns [first, last) run as a state of E x width, zero
+    padded when width > last - first.  The columns of the delta rule's state never mix -
+    v_old[m], the written value, W[:, m] and out[m] depend on column m and on the shared q, k, beta
+    only (fast_weight_cuda.cu:101-143) - so the operator on a slice of V, W is exact, the gradients of
+    Q, K, beta are the sums over the slices, and a padded column (v = 0, W = 0) stays zero."""
+    key = (E, M)
+    if key not in _plans:
+        widths = _FAST_WIDTHS.get(E)
+        plan = None
+        if widths is not None and not (M in widths):
+            plan, first = [], 0
+            while first < M:
+                left = M - first
+                fits = [w for w in widths if w <= left]
+                width = max(fits) if fits else min(w for w in widths if w >= left)
+                last = min(M, first + width)
+                plan.append((first, last, width))
+                first = last
+        _plans[key] = plan
+    return _plans[key]
+
+
+def fast_weight_delta(Q, K, V, beta, W, time_major=None):
+    """``out = fast_weight_delta(Q, K, V, beta, W)``, the reference's operator
+    (algorithmic/fast_weight/__init__.py:96).  Key widths of 16, 32, 64, 96 and 128 with value widths
+    the blocked kernels do not take whole (M = 3 D + 1 of the Delta-Delta layer, M = 128 of the
+    Delta-MLP layer: cuda_fast_weight_layer.py:1474-1492,1605-1610) run on them by slices of value
+    columns, see :func:`column_plan`; every other call goes straight to the autograd function."""
+    plan = column_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
+    if plan is None:
+        return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
+    if W.dim() != 4 or W.shape[-1] != V.shape[-1]:
+        raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
+    outs = []
+    for first, last, width in plan:
+        pad = width - (last - first)
+        Vs, Ws = V[..., first:last], W.detach()[..., first:last]
+        if pad:
+            Vs, Ws = torch.nn.functional.pad(Vs, (0, pad)), torch.nn.functional.pad(Ws, (0, pad))
+        else:
+            Ws = Ws.contiguous()
+        out = _operator(Q, K, Vs, beta, Ws, False)
+        with torch.no_grad():
+            W[..., first:last] = Ws[..., :last - first]         # the state after the last step, in place
+        outs.append(out[..., :last - first] if pad else out)
+    out = torch.cat(outs, -1)
+    if time_major or (time_major is None and rows_lead(Q)):
+        out = out.permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
+    return out

@@ -101,6 +101,31 @@ def test_delta_dispatch_keeps_32_bit_kernels_off_views_beyond_their_range(fwp):
     assert lib.fwp_delta_kind(0, small, small, small, beta, 0, 8, 64, D, D) == -2
 
 
+def test_value_columns_are_sliced_onto_the_blocked_kernels(fwp):
+    """Shapes of the reference's call sites that no kernel takes whole are run by slices of value
+    columns, every slice a state shape the blocked kernels take (checked against fwp_delta_kind)."""
+    import importlib
+    fw = importlib.import_module(fwp.__name__ + ".fast_weight")
+    L = fwp._lib
+    lib = L.lib()
+    assert fw.column_plan(32, 32) is None and fw.column_plan(96, 16) is None and fw.column_plan(128, 16) is None
+    assert fw.column_plan(24, 8) is None and fw.column_plan(5, 3) is None          # no fast kernel for these keys
+    assert fw.column_plan(32, 97) == [(0, 64, 64), (64, 96, 32), (96, 97, 16)]
+    assert fw.column_plan(32, 128) == [(0, 64, 64), (64, 128, 64)]
+    assert fw.column_plan(128, 32) == [(0, 16, 16), (16, 32, 16)]
+    assert fw.column_plan(96, 48) == [(0, 32, 32), (32, 48, 16)]
+    for E, M in ((32, 97), (32, 128), (128, 32), (96, 48), (64, 100), (16, 1)):
+        plan = fw.column_plan(E, M)
+        assert plan[0][0] == 0 and plan[-1][1] == M and all(a[1] == b[0] for a, b in zip(plan, plan[1:]))
+        for first, last, width in plan:
+            assert 0 < last - first <= width
+            qv = L.View(4096, 8 * 64 * E, 64 * E, E)
+            vv = L.View(4096, 8 * 64 * width, 64 * width, width)
+            bv = L.View(4096, 8 * 64, 64, 1)
+            for backward in (0, 1):
+                assert lib.fwp_delta_kind(backward, qv, qv, vv, bv, 4, 8, 64, E, width) in (L.KIND_SPLIT, L.KIND_CHUNKED)
+
+
 def test_largest_state_of_a_differentiated_call_is_published(fwp):
     L = fwp._lib
     rnn, rec, lstm = (L.query(q) for q in (L.Q_MAX_D_RNN, L.Q_MAX_D_REC, L.Q_MAX_D_LSTM))

@@ -33,7 +33,11 @@ DELTA_SHAPES = [
     (2, 3, 130, 16, 16, True),    # ragged tail chunk, carried-in state
     (2, 2, 256, 32, 32, True),
     (1, 2, 1, 16, 16, True),      # single step (RL-style stepping)
-    (2, 2, 37, 32, 97, True),     # E != M (Delta-Delta layer: M = 3D+1)
+    (2, 2, 37, 32, 97, True),     # E != M (Delta-Delta layer: M = 3D+1): slices of 64, 32 and a padded 1 value columns
+    (2, 2, 70, 32, 128, True),    # Delta-MLP layer, wide side as values: two slices of 64 value columns
+    (2, 2, 70, 128, 32, True),    # ... as keys: one-wave blocked kernels with 8 key tiles, two slices of 16 value columns
+    (1, 3, 40, 128, 16, True),    # Performer with 64 random features
+    (1, 2, 50, 96, 48, True),     # 96 keys take values of 16 or 32: slices of 32 and 16
     (1, 3, 70, 24, 8, False),     # E != M, M smaller
     (1, 1, 20, 5, 3, True),       # odd sizes
 ]
