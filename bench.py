@@ -25,10 +25,56 @@ PEAK_HBM = 8.0e12        # MI355X HBM3E, B/s
 
 # HBM bytes per launch of the forward / backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch; FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 by what the same counters read
-# for a 2 GiB device-to-device copy, `--copy-calibration`).
-MEASURED_TRAFFIC = {'delta': {'fwd': 84400000.0, 'bwd': 105900000.0}, 'delta_lm': {'fwd': 204700000.0, 'bwd': 271100000.0},
-                    'sum': {'fwd': 55100000.0, 'bwd': 91500000.0}, 'rnn': {'fwd': 97500000.0, 'bwd': 127500000.0}, 'rec': {'fwd': 131900000.0, 'bwd': 150700000.0},
-                    'lstm': {'fwd': 325300000.0, 'bwd': 382500000.0}}
+# for a 2 GiB device-to-device copy, `--copy-calibration`).  They live in profiles/hbm_traffic.txt, which
+# `bench.py --workload W --traffic-from FETCH_DIR WRITE_DIR` rewrites from the output directories of the
+# two counter runs; a workload without an entry there reports traffic null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.txt")
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def measured_traffic():
+    try:
+        with open(TRAFFIC_FILE) as f:
+            return json.load(f)["bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        return {}
+
+
+def update_traffic(workload, fetch_dir, write_dir):
+    """Average FETCH_SIZE / WRITE_SIZE per dispatch of the library's forward and backward kernels in the
+    two rocprofv3 output directories -> bytes per launch of that workload in profiles/hbm_traffic.txt."""
+    import glob
+    import sqlite3
+
+    def per_kernel(directory, counter):
+        dbs = glob.glob(os.path.join(directory, "**", "*.db"), recursive=True)
+        if not dbs:
+            sys.exit(f"bench.py: no rocprofv3 database under {directory}")
+        con = sqlite3.connect(dbs[0])
+        tables = [r[0] for r in con.execute("select name from sqlite_master where type in ('table','view')")]
+        table = [t for t in tables if t.startswith("counters_collection")][0]
+        rows = con.execute(f"select kernel_name, avg(value) from {table} where counter_name = ? "
+                           "group by kernel_name", (counter,)).fetchall()
+        out = {}
+        for kernel, kib in rows:
+            if "fwp" not in kernel or "reduce_param" in kernel or "prep" in kernel:
+                continue
+            out["fwd" if "fwd" in kernel else "bwd"] = kib * 1024.0
+        return out
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    entry = {d: round(fetch[d] * FETCH_SCALE + write[d] * WRITE_SCALE, -5) for d in ("fwd", "bwd")}
+    table = measured_traffic()
+    table[workload] = entry
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump({"what": "HBM bytes per launch of the forward / backward kernel of a bench.py workload: "
+                           "rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB per dispatch; the factors are "
+                           "what the counters read for a 2 GiB copy, bench.py --copy-calibration)",
+                   "rewritten_by": "python3 bench.py --workload W --traffic-from FETCH_DIR WRITE_DIR",
+                   "bytes_per_launch": table}, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({workload: entry}))
+
 
 # name -> (B, H, T, D, algorithmic flops per token-head = c*D^2, fwd bytes, bwd bytes per token-head)
 WORKLOADS = {
@@ -490,7 +536,13 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run five device-to-device copies of 2 GiB (a kernel of known traffic for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
+    ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="rewrite this workload's entry of profiles/hbm_traffic.txt from the output directories "
+                         "of `rocprofv3 --pmc FETCH_SIZE` and `rocprofv3 --pmc WRITE_SIZE` runs of it, and exit")
     args = ap.parse_args()
+    if args.traffic_from:
+        update_traffic(args.workload, *args.traffic_from)
+        return
     if args.steps is None:
         args.steps = 200 if args.workload == "lm" else 2000
     if args.warmup is None:
@@ -541,8 +593,10 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps
 
-    eager_s = timed_steps(step)
+    # the per-kernel leg first: with few timed steps (the default command of a fresh box times a
+    # millisecond of work) the step would otherwise be measured while the GPU is still waking up
     t_f, t_b, abi_step = kernel_times(name, pkg, arrays, max(20, min(args.steps, 100)))
+    eager_s = timed_steps(step)
     launch = "eager calls of the autograd Function"
     step_s = eager_s
     if args.graph:
@@ -577,7 +631,7 @@ def main():
         "config": {"workload": w["label"], "B": B, "H": H, "T": T, "D": D, "launch": launch},
         "roofline": {"bound": "hbm", "kernel": f"{name} {dom}", "achieved": dom_bytes / dom_t / 1e9,
                      "peak": PEAK_HBM / 1e9, "unit": "GB/s", "frac": dom_bytes / dom_t / PEAK_HBM,
-                     "traffic": MEASURED_TRAFFIC.get(name, {}).get(dom)},
+                     "traffic": measured_traffic().get(name, {}).get(dom)},
         "kernels": {"fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
                     "fwd_GBps": fwd_bytes / t_f / 1e9, "bwd_GBps": bwd_bytes / t_b / 1e9,
                     "kernel_only_tokens_per_s": tokens / kernel_s,

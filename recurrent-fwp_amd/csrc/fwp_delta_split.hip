@@ -79,6 +79,7 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
     // state wave mb to the output wave, blocks of even and odd index alternately: its columns of
     // the state before the block (NE tiles) and of U
     __shared__ LdsMat hx[OUT ? 2 : 1][OUT ? NM : 1][OUT ? NE + 1 : 1];
+    __shared__ LdsMat fill_rm[2];        // the fourth wave (one state wave) to the output wave: lower(Q K^T)^T
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
     const int lane = threadIdx.x % 64;
     const Geo16 p(lane);
@@ -197,13 +198,38 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
     const unsigned m_step = (unsigned)(kBlk * M * 4), out_step = (unsigned)(kBlk * out.sL * 4);
     float *const out_rows = out.ptr + n * out.sN + h * out.sH;
     const uint32_t out_bytes = (uint32_t)(((L - 1) * out.sL + M) * 4);
-    if (OUT && wave == NM + 2) {       // the wave that fills the workgroup up to four
-        for (int r = 0; r < nblk + 2; r++) lds_barrier();
+    // With one state wave a fourth wave fills the workgroup up to four (one SIMD each); it forms
+    // lower(Q K^T)^T for the output wave, in the round in which the state wave does the block
+    constexpr bool kFillQK = OUT && NM == 1;
+    if (OUT && wave == NM + 2) {
+        if constexpr (kFillQK) {
+            using Raw = PrepQk<NE>;
+            auto load = [&](Raw &w, int ib) {
+#pragma unroll
+                for (int b = 0; b < NE; b++) {
+                    w.Kt[b] = kb.f4(o_kt + 64 * b, ib * k_step);
+                    w.Qt[b] = qb.f4(o_qt + 64 * b, ib * q_step);
+                }
+            };
+            auto block = [&](int ib, const Raw &w) {
+                v4f R = zero, Rm;
+#pragma unroll
+                for (int eb = 0; eb < NE; eb++) R = tn(w.Kt[eb], w.Qt[eb], R);       // K Q^T  [s][t]
+#pragma unroll
+                for (int r = 0; r < 4; r++) Rm[r] = (p.up[r] || p.di[r]) ? R[r] : 0.f;
+                fill_rm[ib & 1].put(lane, Rm);
+            };
+            lds_barrier();      // the preparing wave's block 0
+            ring_loop<PF, Raw>(nblk, load, block);
+            lds_barrier();      // the output wave's last block
+        } else {
+            for (int r = 0; r < nblk + 2; r++) lds_barrier();
+        }
         return;
     }
     if (OUT && wave == NM + 1) {
         // ------------------------------------------------ output wave, one block behind
-        using Raw = OutRaw<NE, !kPrepQK>;
+        using Raw = OutRaw<NE, !kPrepQK && !kFillQK>;
         const RowBuf ob(out_rows, out_bytes);
         const unsigned o_out = (unsigned)(c * out.sL + 4 * g) * 4;
         auto load = [&](Raw &w, int ib) {
@@ -211,13 +237,15 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
 #pragma unroll
             for (int b = 0; b < NE; b++) {
                 w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
-                if constexpr (!kPrepQK) w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                if constexpr (!kPrepQK && !kFillQK) w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
             }
         };
         auto block = [&](int ib, const Raw &w) {
             v4f Rm;
             if constexpr (kPrepQK) {
                 Rm = rmat[(ib / kGrp) & 1][ib % kGrp].get(lane);
+            } else if constexpr (kFillQK) {
+                Rm = fill_rm[ib & 1].get(lane);
             } else {
                 v4f R = zero;
 #pragma unroll
