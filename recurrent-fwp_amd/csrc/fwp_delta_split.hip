@@ -716,7 +716,7 @@ struct QuadG {
 
 template <int NE, int NM, int WR>
 constexpr int quad_lds_mats() {
-    return 2 * (NM + NE * NM) + 3 * (2 + 2 * NM) + 2 * (NE * NM + NM) + 2 * NE + 2 * NM + WR;
+    return 2 * (NM + NE * NM) + 3 * (2 + 2 * NM + (NE <= 2 ? 2 * NE + NM : 0)) + 2 * (NE * NM + NM) + 2 * NE + 2 * NM + WR;
 }
 
 // PW = 2: P on two waves, one with the products of Pm, one with the others.
@@ -729,8 +729,16 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
     constexpr int E = 16 * NE, M = 16 * NM, NEW = NE / WR;
     static_assert(NE % WR == 0, "key tiles divide evenly over the waves of a role");
     __shared__ LdsMat pc[2][NM + NE * NM];     // P -> C: Pm^T dO per mb, then Q^T dO per (eb, mb)
-    __shared__ LdsMat pg[3][2 + 2 * NM];       // P -> G, R: dPm, dPm^T, d^T per mb, dO^T per mb
-    __shared__ float pb[3][16];                // P -> G, R: beta[t0 + c]
+    // With narrow keys P reads the block's rows for everybody: it hands K (transposed on the way) to C,
+    // R and G, Q to G, v - v_old (transposed) to R, and beta to C and R through the slots they read
+    // anyway, so that G loads nothing, R only the checkpointed state and C only K^T and T.  A CU's
+    // address unit takes one vector memory instruction per 16 cycles whatever its width, and the roles'
+    // loads of the same rows in the layouts each wants were most of what it did (K alone: 14 per block).
+    constexpr bool kShareG = NE <= 2;
+    constexpr int kGK = 2 + 2 * NM, kGQ = kGK + NE, kGD = kGQ + NE;
+    // P -> C, G, R: dPm, dPm^T, d^T per mb, dO^T per mb (and K, Q per eb, d per mb)
+    __shared__ LdsMat pg[3][2 + 2 * NM + (kShareG ? 2 * NE + NM : 0)];
+    __shared__ __align__(16) float pb[3][16];  // P -> C, G, R: beta[t0 + c]
     __shared__ LdsMat cg[2][NE * NM + NM];     // C -> G, R: dS^T per (eb, mb) before the block's update, dY^T per mb
     __shared__ LdsMat rg[2][NE];               // R -> G: -dX S0^T per eb, transposed like g_k
     __shared__ LdsMat inv[NM][2];              // the inverse inside C where forward left none
@@ -805,6 +813,10 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
                 for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
 #pragma unroll
                 for (int mb = 0; mb < NM; mb++) pc[e & 1][mb].put(lane, tn(Pm, w.Oc[mb], zero));
+                if constexpr (kShareG) {
+#pragma unroll
+                    for (int b = 0; b < NE; b++) pg[third(e)][kGK + b].put_t(p, w.Kt[b]);     // read back as K[4g + r][c]
+                }
             }
             if (with_rest) {
                 v4f Z = zero;
@@ -818,12 +830,17 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
                         pc[e & 1][NM + eb * NM + mb].put(lane, tn(w.Qc[eb], w.Oc[mb], zero));
                     to[2 + mb].put(lane, w.Dt[mb]);
                     to[2 + NM + mb].put(lane, w.Ot[mb]);
+                    if constexpr (kShareG) to[kGD + mb].put_t(p, w.Dt[mb]);      // read back as d[4g + r][c]
                 }
                 v4f dPm;
 #pragma unroll
                 for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
                 to[0].put(lane, dPm);
                 to[1].put_t(p, dPm);
+                if constexpr (kShareG) {
+#pragma unroll
+                    for (int b = 0; b < NE; b++) to[kGQ + b].put(lane, w.Qc[b]);
+                }
                 if (g == 0) pb[s3][c] = w.bcol;
             }
         };
@@ -840,39 +857,70 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
         const bool have_T = aux && aux[0] == 1.f;
         const RowBuf tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0);
-        const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4;
+        const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4, o_tt = (unsigned)(c * 16 + 4 * g) * 4;
         v4f ident;
 #pragma unroll
         for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
         auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
             if (have_T) {
+                if constexpr (kShareG) {
+                    w.T = tb.f4(o_tt, ib * 1024);       // rows of T, one load: T^T in the accumulator layout
+                } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
+                    for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
+                }
             }
             const unsigned ks = ib * k_step, bs = ib * b_step;
-            w.bcol = bb.f(o_bc, bs);
+            if constexpr (!kShareG) {
+                w.bcol = bb.f(o_bc, bs);
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
+                for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
+            } else if (!have_T) {
+                w.bcol = bb.f(o_bc, bs);
+            }
 #pragma unroll
             for (int b = 0; b < NE; b++) {
                 w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
+                if constexpr (!kShareG) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+                    for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
+                }
             }
         };
         v4f dS[NE];           // register r = dS[16 eb + 4g + r][16 mb + c]
 #pragma unroll
         for (int eb = 0; eb < NE; eb++) dS[eb] = zero;
         auto block = [&](int e, const Raw &w) {
+            // beta[t0 + 4g + r] and K[t0 + 4g + r][.]: loaded, or from what P left a round ago
+            float brow[4];
+            v4f Kc[NE];
+            if constexpr (kShareG) {
+                const float4 b4 = *reinterpret_cast<const float4 *>(&pb[third(e)][4 * g]);
+                brow[0] = b4.x, brow[1] = b4.y, brow[2] = b4.z, brow[3] = b4.w;
+#pragma unroll
+                for (int b = 0; b < NE; b++) Kc[b] = pg[third(e)][kGK + b].get(lane);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) brow[r] = w.brow[r];
+#pragma unroll
+                for (int b = 0; b < NE; b++) Kc[b] = w.Kc[b];
+            }
             v4f T = w.T;
-            if (!have_T) {
+            if (have_T) {
+                if constexpr (kShareG) {      // loaded as T^T: turned round through the wave's own LDS
+                    inv[mb][0].put_t(p, w.T);
+                    __builtin_amdgcn_wave_barrier();
+                    T = inv[mb][0].get(lane);
+                    __builtin_amdgcn_wave_barrier();
+                }
+            } else {
                 v4f G = zero, A, At;
 #pragma unroll
                 for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
-                    A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
+                    A[r] = p.lo[r] ? brow[r] * G[r] : 0.f;
                     At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
                 }
                 T = inv_unit_triangular_lds(At, A, ident, inv[mb], p, lane);      // (I + A)^-1
@@ -889,9 +937,9 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
             to[NE * NM + mb].put_t(p, dY);
             v4f ndX;
 #pragma unroll
-            for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
+            for (int r = 0; r < 4; r++) ndX[r] = -(brow[r] * dY[r]);
 #pragma unroll
-            for (int eb = 0; eb < NE; eb++) dS[eb] = tn(w.Kc[eb], ndX, dS[eb] + from[NM + eb * NM + mb].get(lane));
+            for (int eb = 0; eb < NE; eb++) dS[eb] = tn(Kc[eb], ndX, dS[eb] + from[NM + eb * NM + mb].get(lane));
         };
         lds_barrier();
         ring_loop<PF, Raw>(nblk, load, block);
@@ -910,16 +958,20 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
         auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
             const unsigned cs = chunk_of(ib) * (E * M * 4), ks = ib * k_step, bs = ib * b_step, ds = ib * d_step;
+            if constexpr (!kShareG) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
+                for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
 #pragma unroll
-            for (int b = 0; b < NEW; b++)
+                for (int b = 0; b < NEW; b++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
+                    for (int r = 0; r < 4; r++) w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
+            }
 #pragma unroll
             for (int mb = 0; mb < NM; mb++) {
+                if constexpr (!kShareG) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.Dc[mb][r] = db.f(o_dr[r] + 64 * mb, ds);
+                    for (int r = 0; r < 4; r++) w.Dc[mb][r] = db.f(o_dr[r] + 64 * mb, ds);
+                }
 #pragma unroll
                 for (int b = 0; b < NEW; b++)      // register r = S[16 eb + c][16 mb + 4g + r]
                     w.Sck[mb][b] = cb.f4(o_dt + (16 * (eb0 + b) * M + 16 * mb) * 4, cs);
@@ -935,21 +987,35 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
             const int s3 = third(e);
             const float bcol = pb[s3][c];
             const v4f dPmt = pg[s3][1].get(lane);
+            float brow[4];
+            v4f Kc[NEW];
+            if constexpr (kShareG) {
+                const float4 b4 = *reinterpret_cast<const float4 *>(&pb[s3][4 * g]);
+                brow[0] = b4.x, brow[1] = b4.y, brow[2] = b4.z, brow[3] = b4.w;
+#pragma unroll
+                for (int b = 0; b < NEW; b++) Kc[b] = pg[s3][kGK + eb0 + b].get(lane);
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++) brow[r] = w.brow[r];
+#pragma unroll
+                for (int b = 0; b < NEW; b++) Kc[b] = w.Kc[b];
+            }
             v4f gQt[NEW], part[NEW];
 #pragma unroll
-            for (int b = 0; b < NEW; b++) gQt[b] = tn(w.Kc[b], dPmt, zero), part[b] = zero;
+            for (int b = 0; b < NEW; b++) gQt[b] = tn(Kc[b], dPmt, zero), part[b] = zero;
 #pragma unroll
             for (int mb = 0; mb < NM; mb++) {
+                const v4f Dc = kShareG ? pg[s3][kShareG ? kGD + mb : 0].get(lane) : w.Dc[mb];
                 v4f nU;
 #pragma unroll
-                for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[mb][r]);
+                for (int r = 0; r < 4; r++) nU[r] = -(brow[r] * Dc[r]);
                 const v4f Ot = pg[s3][2 + NM + mb].get(lane);
                 const v4f dXt = bcol * cg[e & 1][NE * NM + mb].get(lane);
                 gvb.st4(dXt, o_dt + 64 * mb, ib * d_step);      // register r = g_v[t0 + c][16 mb + 4g + r]
 #pragma unroll
                 for (int b = 0; b < NEW; b++) {
                     if (chunk_of.closes(ib) || ib + 1 == nblk) St[mb][b] = w.Sck[mb][b];   // the state after the block is checkpointed
-                    St[mb][b] = tn(nU, w.Kc[b], St[mb][b]);     // S0^T = S'^T - U^T K
+                    St[mb][b] = tn(nU, Kc[b], St[mb][b]);       // S0^T = S'^T - U^T K
                     gQt[b] = tn(St[mb][b], Ot, gQt[b]);
                     part[b] = tn(St[mb][b], -dXt, part[b]);
                 }
@@ -972,15 +1038,17 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
     const RowBuf gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
         gbb(j == 0 ? gbeta + seq * L : nullptr, j == 0 ? (uint32_t)(L * 4) : 0);
     auto load = [&](Raw &w, int e) {
-        const int ib = nblk - 1 - e;
-        const unsigned ks = ib * k_step, qs = ib * q_step;
+        if constexpr (!kShareG) {
+            const int ib = nblk - 1 - e;
+            const unsigned ks = ib * k_step, qs = ib * q_step;
 #pragma unroll
-        for (int b = 0; b < NEW; b++)
+            for (int b = 0; b < NEW; b++)
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
-                w.Qc[b][r] = qb.f(o_qr[r] + 64 * (eb0 + b), qs);
-            }
+                for (int r = 0; r < 4; r++) {
+                    w.Kc[b][r] = kb.f(o_kr[r] + 64 * (eb0 + b), ks);
+                    w.Qc[b][r] = qb.f(o_qr[r] + 64 * (eb0 + b), qs);
+                }
+        }
     };
     v4f gKt[NEW];             // of the block before, still without R's term
 #pragma unroll
@@ -1019,16 +1087,22 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
 #pragma unroll
         for (int r = 0; r < 4; r++) nM[r] = p.lo[r] ? -Mx[r] : 0.f;
         own[j].put_t(p, nM);
+        v4f Kc[NEW], Qc[NEW];
 #pragma unroll
         for (int b = 0; b < NEW; b++) {
-            gKt[b] = tn(w.Qc[b], dPm, zero);
+            Kc[b] = kShareG ? pg[s3][kShareG ? kGK + eb0 + b : 0].get(lane) : w.Kc[b];
+            Qc[b] = kShareG ? pg[s3][kShareG ? kGQ + eb0 + b : 0].get(lane) : w.Qc[b];
+        }
+#pragma unroll
+        for (int b = 0; b < NEW; b++) {
+            gKt[b] = tn(Qc[b], dPm, zero);
 #pragma unroll
             for (int mb = 0; mb < NM; mb++) gKt[b] = tn(cg[e & 1][(eb0 + b) * NM + mb].get(lane), Ut[mb], gKt[b]);
         }
         __builtin_amdgcn_wave_barrier();
         const v4f nMs = nM + own[j].get(lane);
 #pragma unroll
-        for (int b = 0; b < NEW; b++) gKt[b] = tn(w.Kc[b], nMs, gKt[b]);
+        for (int b = 0; b < NEW; b++) gKt[b] = tn(Kc[b], nMs, gKt[b]);
     };
     lds_barrier();
     lds_barrier();

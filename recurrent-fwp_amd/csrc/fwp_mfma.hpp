@@ -156,21 +156,29 @@ struct SolveRow {
             be[4 * a] = b4.x, be[4 * a + 1] = b4.y, be[4 * a + 2] = b4.z, be[4 * a + 3] = b4.w;
         }
     }
-    // columns HI down to LO of the row (the columns above HI done before)
+    // columns HI down to LO of the row (the columns above HI done before).  Column j needs the row's
+    // entries i > j; only the newest of them, i = j + 1, has just been computed, so the terms i >= j + 2
+    // are summed first, in two chains that do not wait for it, and the newest term is added last: the
+    // dependent path through the row is two operations per column instead of a chain of up to fifteen.
     template <int HI, int LO>
     __device__ __forceinline__ void columns(const SolveLds &s, const Geo16 &p) {
         const float4 *gq = s.gm[p.g];
 #pragma unroll
         for (int jj = HI; jj >= LO; jj--) {
-            float acc = p.c == jj ? 1.f : 0.f;
+            float far0 = p.c == jj ? 1.f : 0.f, far1 = 0.f, near = 0.f;
 #pragma unroll
             for (int a = (jj + 1) / 4; a < 4; a++) {
                 const float4 g4 = gq[16 * a + jj];          // G[4a .. 4a + 3][jj]
                 const float gg[4] = {g4.x, g4.y, g4.z, g4.w};
 #pragma unroll
-                for (int x = 0; x < 4; x++)
-                    if (4 * a + x > jj) acc = fmaf(Wn[4 * a + x], gg[x], acc);
+                for (int x = 0; x < 4; x++) {
+                    const int i = 4 * a + x;
+                    if (i == jj + 1) near = gg[x];
+                    else if (i > jj + 1 && (i & 1)) far1 = fmaf(Wn[i], gg[x], far1);
+                    else if (i > jj + 1) far0 = fmaf(Wn[i], gg[x], far0);
+                }
             }
+            const float acc = jj < 15 ? fmaf(Wn[jj < 15 ? jj + 1 : 15], near, far0 + far1) : far0;
             T[jj] = acc;
             Wn[jj] = -(acc * be[jj]);
         }
