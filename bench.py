@@ -179,6 +179,39 @@ def gpu_step_fn(name, pkg, arrays):
     return step, diff
 
 
+def stream_floor(name):
+    """What the step's algorithmic HBM bytes cost at this size when nothing is computed: copies of one
+    [B,H,T,D] array into another (each launch reads and writes B*H*T*D*4 bytes), back to back between two
+    events like the kernel timings; forward and backward floors = their algorithmic bytes at that rate."""
+    import torch
+    w = WORKLOADS[name]
+    B, H, T, D = w["B"], w["H"], w["T"], w["D"]
+    n = B * H * T * D
+    src = [torch.randn(n, device="cuda:0") for _ in range(4)]
+    dst = [torch.empty(n, device="cuda:0") for _ in range(4)]
+
+    def sweep():
+        for a, b in zip(src, dst):
+            b.copy_(a)
+    for _ in range(20):
+        sweep()
+    torch.cuda.synchronize()
+    reps = 200
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        sweep()
+    e1.record()
+    torch.cuda.synchronize()
+    per_copy_s = e0.elapsed_time(e1) * 1e-3 / (reps * 4)
+    rate = 2 * n * 4 / per_copy_s
+    token_heads = B * H * T
+    fwd_b, bwd_b = w["fwd_bytes"](D) * token_heads, w["bwd_bytes"](D) * token_heads
+    return {"workload": w["label"], "copy_bytes": 2 * n * 4, "copy_us": per_copy_s * 1e6, "copy_GBps": rate / 1e9,
+            "fwd_floor_us": fwd_b / rate * 1e6, "bwd_floor_us": bwd_b / rate * 1e6,
+            "step_floor_us": (fwd_b + bwd_b) / rate * 1e6}
+
+
 def kernel_times(name, pkg, arrays, iters):
     """Average duration (s) of the forward and of the backward launch, timed with HIP
     events on the stream the kernels are launched on (direct C-ABI calls, buffers preallocated)."""
@@ -536,6 +569,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run five device-to-device copies of 2 GiB (a kernel of known traffic for "
                          "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
+    ap.add_argument("--stream-floor", action="store_true",
+                    help="only time plain device-to-device copies of one of the workload's [B,H,T,D] arrays, back to "
+                         "back like the kernels (what moving the step's algorithmic bytes costs at this size), and exit")
     ap.add_argument("--traffic-from", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="rewrite this workload's entry of profiles/hbm_traffic.txt from the output directories "
                          "of `rocprofv3 --pmc FETCH_SIZE` and `rocprofv3 --pmc WRITE_SIZE` runs of it, and exit")
@@ -555,6 +591,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_read": src.numel() * 4, "copy_bytes_written": src.numel() * 4}))
+        return
+    if args.stream_floor:
+        print(json.dumps(stream_floor(args.workload if args.workload in WORKLOADS else "delta")))
         return
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (sequences are independent; "
