@@ -510,8 +510,9 @@ def lm_cpu_baseline(pkg):
 
 def run_single_steps(args, pkg):
     """Stepwise inference: one call per time step (T = 1, no gradient, state carried in W and h), as an
-    actor or a decoder makes them.  Launch- and host-bound; reported per operator, through the package's
-    default entry point and through the Python autograd.Function."""
+    actor or a decoder makes them.  Reported per operator: through the package's default entry point (the
+    single-step kernels), the same with those kernels switched off (the kernels written for sequences), and
+    through the Python autograd.Function."""
     import numpy as np
     import torch
     from helpers import delta_inputs, rec_inputs, rnn_inputs
@@ -531,7 +532,9 @@ def run_single_steps(args, pkg):
     out = {}
     with torch.no_grad():
         for name, (call, default, python) in calls.items():
-            for label, f in (("default", default), ("python_function", python)):
+            for label, f in (("default", default), ("sequence_kernels", default), ("python_function", python)):
+                # "sequence_kernels": the same calls with the single-step kernels switched off
+                pkg._lib.config(pkg._lib.CFG_STEP_KERNELS, int(label != "sequence_kernels"))
                 for _ in range(args.warmup):
                     call(f)
                 torch.cuda.synchronize()
@@ -540,6 +543,14 @@ def run_single_steps(args, pkg):
                     call(f)
                 torch.cuda.synchronize()
                 out.setdefault(name, {})[label + "_us"] = (time.perf_counter() - t0) / n * 1e6
+                if label != "python_function":
+                    # what a caller that needs each step's result before the next sees: call + wait
+                    m = max(n // 10, 1)
+                    t0 = time.perf_counter()
+                    for _ in range(m):
+                        call(f)
+                        torch.cuda.synchronize()
+                    out[name][label + "_waited_us"] = (time.perf_counter() - t0) / m * 1e6
     lat = out["fast_weight_delta"]["default_us"] * 1e-6
     return {"metric": "stepwise inference tokens/s (one forward call per time step, no gradient), 1 GPU",
             "value": B / lat, "unit": "tokens/s", "n_gpus": 1, "steps": n, "warmup": args.warmup,

@@ -62,7 +62,8 @@ enum {
     FWP_Q_MAX_D_RNN = 4,
     FWP_Q_MAX_D_REC = 5,
     FWP_Q_MAX_D_LSTM = 6,
-    FWP_Q_STATIC_SCRATCH_FLOATS = 7 /* floats of scratch fwp_rec_bwd_static has per GPU */
+    FWP_Q_STATIC_SCRATCH_FLOATS = 7, /* floats of scratch fwp_rec_bwd_static has per GPU */
+    FWP_Q_STEP_LAUNCHES = 8 /* calls so far that the single-step kernels took (modulo 2^31) */
 };
 
 const char *fwp_strerror(int code);
@@ -75,9 +76,14 @@ int fwp_query(int what);
  * kernels), FWP_DELTA_CHUNKED (16-step blocks on the matrix cores, one wave per sequence),
  * FWP_DELTA_SPLIT (the same blocks, a sequence's work split over several waves; the sum rule
  * takes the one-wave blocks), FWP_DELTA_PHASE (16 x 16 states: the blocks of a sequence prepared in
- * parallel, one product per block on the sequential chain; other shapes as FWP_DELTA_SPLIT).  All give the same results within the fp32 tolerance.  Returns FWP_E_SHAPE for an unknown key or value.
+ * parallel, one product per block on the sequential chain; other shapes as FWP_DELTA_SPLIT).  All give the same results within the fp32 tolerance.
+ * FWP_CFG_STEP_KERNELS: 1 (default) sends forward calls of one step (L = 1) that save nothing for a
+ * backward pass - stepwise inference, state carried from call to call - to kernels that do exactly
+ * one step (every operator; E in {16,32,64,96,128} x M in {16,32,64,128} for the delta and sum rules,
+ * D in {16,32} for the others); 0 leaves them on the kernels written for sequences.
+ * Returns FWP_E_SHAPE for an unknown key or value.
  */
-enum { FWP_CFG_DELTA_KERNELS = 0 };
+enum { FWP_CFG_DELTA_KERNELS = 0, FWP_CFG_STEP_KERNELS = 1 };
 enum { FWP_DELTA_AUTO = 0, FWP_DELTA_SCAN = 1, FWP_DELTA_CHUNKED = 2, FWP_DELTA_SPLIT = 3, FWP_DELTA_PHASE = 4 };
 int fwp_config(int key, int value);
 

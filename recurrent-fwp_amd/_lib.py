@@ -52,6 +52,7 @@ EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_de
                                        "fwp_delta_ckpt_floats", "fwp_delta_kind"])
 KIND_LDS, KIND_SCAN, KIND_CHUNKED, KIND_SPLIT, KIND_PHASE = 0, 1, 2, 3, 4
 CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT, DELTA_PHASE = 0, 0, 1, 2, 3, 4
+CFG_STEP_KERNELS = 1
 
 _lib = None
 _checked_devices = set()
@@ -96,6 +97,12 @@ def query(what):
 
 Q_VERSION, Q_CHUNK_QUANTUM, Q_DEFAULT_CHUNK, Q_MAX_STATE_FLOATS = 0, 1, 2, 3
 Q_MAX_D_RNN, Q_MAX_D_REC, Q_MAX_D_LSTM, Q_STATIC_SCRATCH_FLOATS = 4, 5, 6, 7
+Q_STEP_LAUNCHES = 8
+
+
+def step_launches():
+    """Calls so far that went to the single-step kernels (a running count, never cached)."""
+    return int(lib().fwp_query(Q_STEP_LAUNCHES))
 
 
 _ckpt_floats_cache = {}

@@ -11,6 +11,6 @@ common=(--offload-arch=gfx950 -O3 -std=c++17 -fPIC -Xclang -target-feature -Xcla
 wide="$(mktemp -d)/fwp_sum_wide.o"
 "$HIPCC" "${common[@]}" -c "$here"/fwp_sum_wide.hip -o "$wide" "$@"
 "$HIPCC" "${common[@]}" -shared -mllvm -amdgpu-mfma-vgpr-form "$wide" \
-    "$here"/fwp_api.hip "$here"/fwp_generic.hip "$here"/fwp_delta_reg.hip "$here"/fwp_delta_mfma.hip "$here"/fwp_delta_split.hip "$here"/fwp_delta_phase.hip "$here"/fwp_rnn_reg.hip "$here"/fwp_lstm_reg.hip "$here"/fwp_rec_reg.hip "$here"/fwp_layer.hip "$here"/fwp_static.hip \
+    "$here"/fwp_api.hip "$here"/fwp_generic.hip "$here"/fwp_delta_reg.hip "$here"/fwp_delta_mfma.hip "$here"/fwp_delta_split.hip "$here"/fwp_delta_phase.hip "$here"/fwp_rnn_reg.hip "$here"/fwp_lstm_reg.hip "$here"/fwp_rec_reg.hip "$here"/fwp_layer.hip "$here"/fwp_static.hip "$here"/fwp_step.hip \
     -o "$out" "$@"
 echo "built $out"

@@ -27,6 +27,14 @@ int check_dims(int N, int H, int L, int E, int M, int chunk) {
 // (a test and measurement switch: one word, read once per call, written by fwp_config only)
 std::atomic<int> g_delta_kernels{FWP_DELTA_AUTO};
 
+// fwp_config(FWP_CFG_STEP_KERNELS, .): single steps that save nothing on the kernels written for them
+std::atomic<int> g_step_kernels{1};
+std::atomic<unsigned> g_step_launches{0};
+int counted(int rc) {
+    g_step_launches++;
+    return rc;
+}
+
 // Blocks on the matrix cores pay off from about two blocks on; single steps (stepwise inference)
 // stay on the scan kernel.
 bool delta_chunked(int L) {
@@ -103,6 +111,10 @@ int fwp_config(int key, int value) {
         g_delta_kernels = value;
         return FWP_OK;
     }
+    if (key == FWP_CFG_STEP_KERNELS && (value == 0 || value == 1)) {
+        g_step_kernels = value;
+        return FWP_OK;
+    }
     return FWP_E_SHAPE;
 }
 
@@ -131,6 +143,7 @@ int fwp_query(int what) {
         case FWP_Q_MAX_D_RNN: return generic_max_dim(0);
         case FWP_Q_MAX_D_REC: return generic_max_dim(1);
         case FWP_Q_MAX_D_LSTM: return generic_max_dim(2);
+        case FWP_Q_STEP_LAUNCHES: return (int)(g_step_launches.load() & 0x7fffffffu);
         default: return -1;
     }
 }
@@ -161,6 +174,9 @@ int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, flo
     // the output view takes part in the choice of kernels like an input read 16 bytes at a time
     const fwp_view ov = {out.ptr, out.sN, out.sH, out.sL};
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && reg_view_ok(ov) && in_range32(L, E, M, {ov});
+    if (L == 1 && !ckpt && g_step_kernels && g_delta_kernels == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
+        reg_view_ok(v) && reg_view_ok(ov) && aligned16(W))
+        return counted(step_delta_fwd(q, k, v, beta, W, out, N, H, E, M, (hipStream_t)stream));
     switch (delta_kind(false, aligned, q, k, v, beta, N, H, L, E, M)) {
         case FWP_KIND_PHASE:
             return phase_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, chunk, (hipStream_t)stream);
@@ -218,6 +234,9 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
                 int L, int E, int M, int chunk, void *stream) {
     if (bad_view(q) || bad_view(k) || bad_view(v) || !W || !out) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    if (L == 1 && !ckpt && g_step_kernels && g_delta_kernels == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
+        reg_view_ok(v) && aligned16(out) && aligned16(W))
+        return counted(step_sum_fwd(q, k, v, W, out, N, H, E, M, (hipStream_t)stream));
     if ((split_delta_dims(E, M) || sum_wide_dims(E, M)) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
         aligned16(out)) {
         // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
@@ -258,6 +277,9 @@ int fwp_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, flo
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    if (L == 1 && !ckpt && g_step_kernels && step_rec_dims(D) && reg_view_ok(z) && reg_view_ok(v) && aligned16(W) &&
+        aligned16(h) && aligned16(out))
+        return counted(step_rnn_fwd(z, k, v, beta, W, h, out, N, H, D, (hipStream_t)stream));
     if (reg_rnn_supported(D) && reg_view_ok(z) && reg_view_ok(k) && reg_view_ok(v) &&
         aligned16(vdiff) && aligned16(ckpt) && aligned16(out))
         return reg_rnn_fwd(z, k, v, beta, W, h, out, vdiff, ckpt, N, H, L, D, chunk,
@@ -299,6 +321,8 @@ int fwp_lstm_fwd(const fwp_view *z, const fwp_view *k, const fwp_view *v, const 
                aligned16(cell) && aligned16(gates) && aligned16(vdiff) && aligned16(ckpt);
     for (int a = 0; a < 3; a++)
         reg = reg && reg_view_ok(z[a]) && reg_view_ok(k[a]) && reg_view_ok(v[a]) && aligned16(W[a]);
+    if (L == 1 && saved == 0 && g_step_kernels && step_rec_dims(D) && reg)
+        return counted(step_lstm_fwd(g, h, c, out, cell, N, H, D, (hipStream_t)stream));
     if (reg)
         return reg_lstm_fwd(g, h, c, out, cell, gates, vdiff, ckpt, N, H, L, D, chunk,
                             (hipStream_t)stream);
@@ -356,6 +380,10 @@ int fwp_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float 
                       (vdiff != nullptr) + (ckpt != nullptr);
     if (saved != 0 && saved != 5) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, D, D, chunk)) return rc;
+    if (L == 1 && saved == 0 && g_step_kernels && step_rec_dims(D) && reg_view_ok(qx) && reg_view_ok(kx) &&
+        reg_view_ok(vx) && aligned16(Rq) && aligned16(Rk) && aligned16(Rv) && aligned16(W) && aligned16(h) &&
+        aligned16(out))
+        return counted(step_rec_fwd(qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, N, H, D, (hipStream_t)stream));
     if (reg_rec_supported(D) && reg_view_ok(qx) && reg_view_ok(kx) && reg_view_ok(vx) &&
         aligned16(out) && aligned16(vdiff) && aligned16(q_act) && aligned16(k_act) && aligned16(ckpt))
         return reg_rec_fwd(qx, kx, vx, bx, Rq, Rk, Rv, rb, W, h, out, q_act, k_act, beta_act, vdiff,

@@ -167,6 +167,22 @@ int reg_rec_bwd(const float *q_act, const float *k_act, const float *beta_act, c
                 float *gkx, float *gvx, float *gbx, float *workspace, int N, int H, int L, int D,
                 int chunk, hipStream_t s);
 
+// One step (L = 1) of a forward pass that saves nothing: kernels that do exactly that (rows read 16 bytes
+// at a time must be aligned, as for the register-state kernels).
+bool step_delta_dims(int E, int M);
+bool step_rec_dims(int D);
+int step_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out, int N, int H,
+                   int E, int M, hipStream_t s);
+int step_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, int N, int H, int E, int M,
+                 hipStream_t s);
+int step_rnn_fwd(fwp_view z, fwp_view k, fwp_view v, fwp_view beta, float *W, float *h, float *out, int N,
+                 int H, int D, hipStream_t s);
+int step_lstm_fwd(const LstmGates &g, float *h, float *c, float *out, float *cell, int N, int H, int D,
+                  hipStream_t s);
+int step_rec_fwd(fwp_view qx, fwp_view kx, fwp_view vx, fwp_view bx, const float *Rq, const float *Rk,
+                 const float *Rv, const float *rb, float *W, float *h, float *out, int N, int H, int D,
+                 hipStream_t s);
+
 // Fused pre-step of the Delta-Net layer and its adjoint (D in {16, 32, 64}).
 bool prep_supported(int D);
 int deltanet_prep_fwd(const float *qkvb, float *q, float *k, float *v, float *beta, int T, int B, int H,

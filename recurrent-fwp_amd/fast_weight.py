@@ -120,6 +120,8 @@ _operator = _fwp_torch.fast_weight_delta if _fwp_torch is not None else DeltaFas
 
 # Value widths the blocked kernels take for a given key width (fwp_delta_kind names the kernels).
 _FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16,)}
+# Value widths the single-step kernels take (with any of the key widths above).
+_STEP_WIDTHS = (16, 32, 64, 128)
 _plans = {}
 
 
@@ -154,6 +156,9 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
     Delta-MLP layer: cuda_fast_weight_layer.py:1474-1492,1605-1610) run on them by slices of value
     columns, see :func:`column_plan`; every other call goes straight to the autograd function."""
     plan = column_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
+    if plan is not None and Q.shape[2] == 1 and V.shape[-1] in _STEP_WIDTHS and not (
+            torch.is_grad_enabled() and any(t.requires_grad for t in (Q, K, V, beta))):
+        plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
     if plan is None:
         return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
     if W.dim() != 4 or W.shape[-1] != V.shape[-1]:
