@@ -270,6 +270,7 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
     }
 
     // ---------------------------------------------------- state wave of columns [16 mb, 16 mb + 16)
+    __builtin_amdgcn_s_setprio(3);      // the wave on the chain goes first where waves share a SIMD
     const int mb = wave;
     unsigned o_kr[4], o_vr[4];
 #pragma unroll
@@ -776,6 +777,7 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
 
     if (wave < PW) {
         // ------------------------------------------------ P
+        __builtin_amdgcn_s_setprio(2);      // ... then the role that feeds it
         const bool with_pm = wave == 0, with_rest = wave == PW - 1;
         using Raw = QuadP<NE, NM>;
         auto load = [&](Raw &w, int e) {
@@ -852,6 +854,7 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
     }
     if (wave < PW + NM) {
         // ------------------------------------------------ C of value columns [16 mb, 16 mb + 16)
+        __builtin_amdgcn_s_setprio(3);      // the chain goes first where waves share a SIMD
         const int mb = wave - PW;
         using Raw = QuadC<NE>;
         // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
@@ -1137,20 +1140,23 @@ void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp
     if constexpr (NM <= 2) {
         if (NM == 1 || (int64_t)nseq * (NM + 2) <= 1536) {
             hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), true>), dim3(nseq),
-                               dim3(64 * (NM == 1 ? 4 : NM + 2)), 0,
+                               dim3(64 * (NM == 1 ? 4 : NM + 2)),
+                               0,
                                s, q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
             return;
         }
     }
     if constexpr (NM > 1)
-        hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), false>), dim3(nseq), dim3(64 * (NM + 1)), 0, s,
+        hipLaunchKernelGGL((k_delta_fwd_split<NE, NM, fwd_ring(NE), false>), dim3(nseq), dim3(64 * (NM + 1)),
+                           0, s,
                            q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
 }
 template <int NE, int NM>
 void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go, const float *ckpt,
                 const float *aux, float *gq, float *gk, float *gv, float *gbeta, int nseq, int H, int L,
                 int chunk, int nchunk, hipStream_t s) {
-    hipLaunchKernelGGL((k_delta_bwd_split<NE, NM, bwd_ring(NE)>), dim3(nseq), dim3(64 * (NE + NM)), 0, s, q, k,
+    hipLaunchKernelGGL((k_delta_bwd_split<NE, NM, bwd_ring(NE)>), dim3(nseq), dim3(64 * (NE + NM)),
+                       0, s, q, k,
                        beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
 }
 }  // namespace
@@ -1179,10 +1185,14 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
 #define Q(ne, nm, wr, pw, pf)                                                                               \
     if (E == 16 * ne && M == 16 * nm) {                                                                     \
         static_assert(quad_lds_mats<ne, nm, wr>() * sizeof(LdsMat) + 192 <= 160 * 1024, "LDS of the hand-over"); \
-        hipLaunchKernelGGL((k_delta_bwd_quad<ne, nm, wr, pw, pf>), dim3(N * H), dim3(64 * (pw + nm + 2 * wr)), 0, \
+        hipLaunchKernelGGL((k_delta_bwd_quad<ne, nm, wr, pw, pf>), dim3(N * H), dim3(64 * (pw + nm + 2 * wr)), \
+                           0,                        \
                            s, q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);    \
         return (int)hipGetLastError();                                                                      \
     }
+    // blocks in flight per wave: short sequences start sooner with two (all sequences ask for their first rows
+    // at once, and a deeper ring puts more requests in front of them), long ones stream better with three
+    if (L <= 512) { Q(1, 1, 1, 1, 2) }
     Q(1, 1, 1, 1, 3) Q(2, 1, 1, 1, 3) Q(1, 2, 1, 1, 3) Q(2, 2, 2, 2, 3) Q(4, 1, 2, 1, 2) Q(6, 1, 3, 1, 2)
     Q(4, 2, 2, 1, 2) Q(1, 4, 1, 1, 2) Q(2, 4, 1, 1, 2) Q(6, 2, 3, 1, 1)
 #undef Q

@@ -1,6 +1,6 @@
 """Stepwise inference: one call per time step (L = 1, no gradient), the state carried from call to call in W, h
-and c as an actor or a decoder does (reference: reinforcement_learning/torchbeast/layer.py:173,256-260,342 with
-T = 1 in the actors; language_modeling/src/utils/cuda_fast_weight_layer.py:149-185 with carried `mems`).  Such calls
+and c as an actor or a decoder does (reference: the inference loop of
+reinforcement_learning/torchbeast/polybeast_learner.py:376-393 calling torchbeast/layer.py:173,256-260,342 with T = 1; language_modeling/src/utils/cuda_fast_weight_layer.py:149-185 with carried `mems`).  Such calls
 take kernels of their own; the results of a run of them are held to the float64 oracle's run over the whole
 sequence, and to the kernels written for sequences.
 
