@@ -342,18 +342,22 @@ def kernel_times(name, pkg, arrays, iters):
             h.copy_(h0)
 
     def timed(fn):
-        """Average duration of `iters` back-to-back launches between two events on the launch stream."""
-        for _ in range(3):
+        """Average duration of a launch: batches of `iters` back-to-back launches between two events on the
+        launch stream, the median batch (the first launches after an idle spell run at lower clocks)."""
+        for _ in range(50):
             L.check(fn(), "warm-up launch")
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            rc = fn()
-        e1.record()
-        L.check(rc, "timed launch")
-        e1.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / iters
+        batches = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                rc = fn()
+            e1.record()
+            L.check(rc, "timed launch")
+            e1.synchronize()
+            batches.append(e0.elapsed_time(e1) * 1e-3 / iters)
+        return sorted(batches)[len(batches) // 2]
 
     t_f = timed(fwd)       # the state carries over between launches; the work per launch is the same
     reset()
@@ -645,7 +649,7 @@ def main():
 
     # the per-kernel leg first: with few timed steps (the default command of a fresh box times a
     # millisecond of work) the step would otherwise be measured while the GPU is still waking up
-    t_f, t_b, abi_step = kernel_times(name, pkg, arrays, max(20, min(args.steps, 100)))
+    t_f, t_b, abi_step = kernel_times(name, pkg, arrays, 100)
     eager_s = timed_steps(step)
     launch = "eager calls of the autograd Function"
     step_s = eager_s
