@@ -1,7 +1,7 @@
 """Parity at the benchmark sizes, whole tensors against the float64 C oracle, default dispatch.
 
 For every output, final state and gradient the achieved error is printed (run with -s) and written to
-gpurun_out/parity_<case>.json when that directory exists:
+$FWP_REPORT_DIR/parity_<case>.json when that variable names a directory:
   max_abs          max |got - want|
   rel_scale        max_abs / max |want|                    (error relative to the tensor's scale)
   rel_elem         max |got - want| / (|want| + 1e-6)      (the measure of the reference's own self-tests,
@@ -21,7 +21,6 @@ import oracle
 from helpers import delta_inputs, lstm_inputs, rec_inputs, rnn_inputs
 
 pytestmark = pytest.mark.gpu
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 ATOL, RTOL = 1e-4, 1e-3
 
 def measures(got, want):
@@ -45,8 +44,8 @@ def report(case, rows):
     for name, m in rows.items():
         print(f"  {name:8s} {m['max_want']:10.3e} {m['max_abs']:10.3e} {m['rel_scale']:10.3e} {m['rel_elem']:10.3e} "
               f"{m['share_rel_elem_above_1e-3']:9.2e} {m['combined']:9.3f}", flush=True)
-    out_dir = os.path.join(ROOT, "gpurun_out")
-    if os.path.isdir(out_dir):
+    out_dir = os.environ.get("FWP_REPORT_DIR", "")
+    if out_dir and os.path.isdir(out_dir):
         with open(os.path.join(out_dir, f"parity_{case}.json"), "w") as f:
             json.dump(rows, f, indent=1)
     for name, m in rows.items():
