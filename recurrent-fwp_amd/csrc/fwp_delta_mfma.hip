@@ -326,10 +326,8 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_bwd_mfma(fwp_view q, f
     const ChunkOf chunk_of(chunk);
     auto load = [&](BwdRaw<NE, NM> &w, int e) {
         const int ib = nblk - 1 - e;
-        if (have_T) {
 #pragma unroll
-            for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
-        }
+        for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);      // zeros where forward left no T
         {   // always loaded, so that no load is left to be issued (and waited for) inside the block
             const unsigned cs = chunk_of(ib) * (E * M * 4);
 #pragma unroll

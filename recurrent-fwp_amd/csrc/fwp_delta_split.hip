@@ -475,10 +475,8 @@ __global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, 
         }
         auto load = [&](AdjRaw<NE> &w, int e) {
             const int ib = nblk - 1 - e;
-            if (have_T) {
 #pragma unroll
-                for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
-            }
+            for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);      // zeros where forward left no T
             const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
                            bs = ib * b_step;
             w.bcol = bb.f(o_bc, bs);
@@ -866,21 +864,20 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
         for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
         auto load = [&](Raw &w, int e) {
             const int ib = nblk - 1 - e;
-            if (have_T) {
-                if constexpr (kShareG) {
-                    w.T = tb.f4(o_tt, ib * 1024);       // rows of T, one load: T^T in the accumulator layout
-                } else {
+            // The same loads whether or not forward left T (without it the buffer has size 0 and reads zeros):
+            // with loads on some paths only, the compiler's wait before a block's first use counts the
+            // fewest loads any path issues since, and waits for loads of the round before.
+            if constexpr (kShareG) {
+                w.T = tb.f4(o_tt, ib * 1024);       // rows of T, one load: T^T in the accumulator layout
+            } else {
 #pragma unroll
-                    for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
-                }
+                for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);
             }
             const unsigned ks = ib * k_step, bs = ib * b_step;
             if constexpr (!kShareG) {
                 w.bcol = bb.f(o_bc, bs);
 #pragma unroll
                 for (int r = 0; r < 4; r++) w.brow[r] = bb.f(o_br[r], bs);
-            } else if (!have_T) {
-                w.bcol = bb.f(o_bc, bs);
             }
 #pragma unroll
             for (int b = 0; b < NE; b++) {
@@ -918,13 +915,14 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
                     __builtin_amdgcn_wave_barrier();
                 }
             } else {
+                const float bcol = kShareG ? pb[third(e)][c] : w.bcol;      // beta[t0 + c]
                 v4f G = zero, A, At;
 #pragma unroll
                 for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     A[r] = p.lo[r] ? brow[r] * G[r] : 0.f;
-                    At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
+                    At[r] = p.up[r] ? bcol * G[r] : 0.f;
                 }
                 T = inv_unit_triangular_lds(At, A, ident, inv[mb], p, lane);      // (I + A)^-1
             }
