@@ -38,6 +38,8 @@ DELTA_SHAPES = [
     (2, 2, 70, 128, 32, True),    # ... as keys: one-wave blocked kernels with 8 key tiles, two slices of 16 value columns
     (1, 3, 40, 128, 16, True),    # Performer with 64 random features
     (1, 2, 50, 96, 48, True),     # 96 keys take values of 16 or 32: slices of 32 and 16
+    (1, 2, 40, 192, 32, True),    # DPFP with nu = 3 at D = 32 (E = 2 nu D): state in LDS
+    (1, 1, 33, 256, 64, True),    # the largest state the library accepts (16384 floats)
     (1, 3, 70, 24, 8, False),     # E != M, M smaller
     (1, 1, 20, 5, 3, True),       # odd sizes
 ]
