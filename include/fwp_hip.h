@@ -93,6 +93,8 @@ int fwp_config(int key, int value);
  * arguments, touches no device.  `backward` = 0: x is v; 1: x is grad_out.  Returns FWP_KIND_* or
  * FWP_E_SHAPE.  The kernels that address a sequence with 32-bit offsets (FWP_KIND_SPLIT,
  * FWP_KIND_CHUNKED, FWP_KIND_PHASE) are never chosen for a view that could exceed them.
+ * For a forward call it answers for a contiguous output and for the kernels written for sequences;
+ * fwp_delta_fwd_kind also takes the output view and knows the single-step kernels.
  * No counterpart in the reference (its one kernel per direction takes every call).
  */
 enum {
@@ -100,10 +102,23 @@ enum {
     FWP_KIND_SCAN = 1,    /* state in registers, step by step */
     FWP_KIND_CHUNKED = 2, /* 16-step blocks on the matrix cores, one wave per sequence */
     FWP_KIND_SPLIT = 3,   /* the same blocks, roles of a block on several waves */
-    FWP_KIND_PHASE = 4    /* blocks prepared in parallel by the waves of a workgroup, short chain */
+    FWP_KIND_PHASE = 4,   /* blocks prepared in parallel by the waves of a workgroup, short chain */
+    FWP_KIND_STEP = 5     /* one step that saves nothing (fwp_delta_fwd_kind only) */
 };
 int fwp_delta_kind(int backward, fwp_view q, fwp_view k, fwp_view x, fwp_view beta, int N, int H,
                    int L, int E, int M);
+
+/*
+ * Which kernels fwp_delta_fwd_strided takes for a call with these input views, this output view and
+ * these dimensions (16-byte aligned W, vdiff and ckpt assumed); `saves` != 0: the call passes vdiff and
+ * ckpt.  The output view takes part in the choice like an input read 16 bytes at a time: rows that are
+ * not 16-byte aligned send the call to FWP_KIND_LDS, a view beyond 32-bit offsets to FWP_KIND_SCAN
+ * (64-bit addresses) where the shape has scan kernels.  A call of one step that saves nothing answers
+ * FWP_KIND_STEP when the single-step kernels take it (FWP_CFG_STEP_KERNELS on, FWP_DELTA_AUTO).
+ * A pure function, touches no device.  No counterpart in the reference.
+ */
+int fwp_delta_fwd_kind(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, fwp_out_view out, int saves,
+                       int N, int H, int L, int E, int M);
 
 /* 0 if the current HIP device is a gfx950 part, FWP_E_ARCH otherwise. */
 int fwp_check_device(void);

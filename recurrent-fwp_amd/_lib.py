@@ -49,8 +49,8 @@ _SIGNATURES = {
     "fwp_rec_bwd_static": [_P] * 6 + [_V] + [_P] * 13 + [_I] * 5 + [_P],
 }
 EXPORTS = sorted(list(_SIGNATURES) + ["fwp_strerror", "fwp_query", "fwp_check_device", "fwp_config",
-                                       "fwp_delta_ckpt_floats", "fwp_delta_kind"])
-KIND_LDS, KIND_SCAN, KIND_CHUNKED, KIND_SPLIT, KIND_PHASE = 0, 1, 2, 3, 4
+                                       "fwp_delta_ckpt_floats", "fwp_delta_kind", "fwp_delta_fwd_kind"])
+KIND_LDS, KIND_SCAN, KIND_CHUNKED, KIND_SPLIT, KIND_PHASE, KIND_STEP = 0, 1, 2, 3, 4, 5
 CFG_DELTA_KERNELS, DELTA_AUTO, DELTA_SCAN, DELTA_CHUNKED, DELTA_SPLIT, DELTA_PHASE = 0, 0, 1, 2, 3, 4
 CFG_STEP_KERNELS = 1
 
@@ -80,6 +80,8 @@ def lib():
         handle.fwp_delta_ckpt_floats.restype = ctypes.c_longlong
         handle.fwp_delta_kind.argtypes = [_I] + [_V] * 4 + [_I] * 5
         handle.fwp_delta_kind.restype = ctypes.c_int
+        handle.fwp_delta_fwd_kind.argtypes = [_V] * 4 + [OutView] + [_I] * 6
+        handle.fwp_delta_fwd_kind.restype = ctypes.c_int
         handle.fwp_config.argtypes = [ctypes.c_int, ctypes.c_int]
         handle.fwp_config.restype = ctypes.c_int
         _lib = handle

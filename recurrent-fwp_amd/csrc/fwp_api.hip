@@ -24,7 +24,9 @@ int check_dims(int N, int H, int L, int E, int M, int chunk) {
 }
 
 // fwp_config(FWP_CFG_DELTA_KERNELS, .)
-// (a test and measurement switch: one word, read once per call, written by fwp_config only)
+// (a test and measurement switch: one word, written by fwp_config only; every entry point reads it once,
+// at its top, and hands that value `dk` down, so that a call is dispatched under one setting even when
+// another thread changes it meanwhile)
 std::atomic<int> g_delta_kernels{FWP_DELTA_AUTO};
 
 // fwp_config(FWP_CFG_STEP_KERNELS, .): single steps that save nothing on the kernels written for them
@@ -37,8 +39,8 @@ int counted(int rc) {
 
 // Blocks on the matrix cores pay off from about two blocks on; single steps (stepwise inference)
 // stay on the scan kernel.
-bool delta_chunked(int L) {
-    return g_delta_kernels >= FWP_DELTA_CHUNKED || (g_delta_kernels == FWP_DELTA_AUTO && L >= 32);
+bool delta_chunked(int dk, int L) {
+    return dk >= FWP_DELTA_CHUNKED || (dk == FWP_DELTA_AUTO && L >= 32);
 }
 
 // Several waves per sequence or one, measured on MI355X (1024 SIMDs) as the time of a training step
@@ -57,14 +59,14 @@ bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
 }
 
 // Shapes that have no other fast kernel (E != M, E or M above 32) always take them.
-bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
+bool delta_split(int dk, int N, int H, int L, int E, int M, std::initializer_list<fwp_view> views,
                  const fwp_view &beta) {
     if (!split_delta_supported(L) || !split_delta_dims(E, M)) return false;
     if (!in_range32(L, E, M, {beta}) || !in_range32(L, E, M, views)) return false;
     for (const fwp_view &v : views)      // rows read 16 bytes at a time
         if (!reg_view_ok(v)) return false;
-    if (g_delta_kernels == FWP_DELTA_SPLIT || g_delta_kernels == FWP_DELTA_PHASE) return true;
-    if (g_delta_kernels != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
+    if (dk == FWP_DELTA_SPLIT || dk == FWP_DELTA_PHASE) return true;
+    if (dk != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
     if (L < 32) return false;
     return (int64_t)N * H <= 1024;
@@ -72,28 +74,36 @@ bool delta_split(bool forward, int N, int H, int L, int E, int M, std::initializ
 
 // Of the calls the several-wave kernels take (same views, same range of offsets), those that go to the
 // kernels that prepare the blocks of a sequence in parallel: 16 x 16 states, forward.
-bool delta_phase(bool backward, int L, int E, int M) {
+bool delta_phase(int dk, bool backward, int L, int E, int M) {
     if (backward || !phase_delta_dims(E, M)) return false;
-    return g_delta_kernels == FWP_DELTA_PHASE;
+    return dk == FWP_DELTA_PHASE;
 }
 
-// Which kernels a delta-rule call takes.  `x` is v for the forward pass and grad_out for the backward
-// pass (the views read 16 bytes at a time besides q and k); `aligned` says that every contiguous buffer
-// of the call is 16-byte aligned.  The kernels that read through buffer resources (split, chunked)
-// address a sequence with 32-bit byte offsets: views beyond them go to the scan or the LDS-state kernels,
-// which use 64-bit addresses, in both directions alike.
-int delta_kind(bool backward, bool aligned, const fwp_view &q, const fwp_view &k, const fwp_view &x,
-               const fwp_view &beta, int N, int H, int L, int E, int M) {
-    if (aligned && delta_split(!backward, N, H, L, E, M, {q, k, x}, beta))
-        return delta_phase(backward, L, E, M) ? FWP_KIND_PHASE : FWP_KIND_SPLIT;
-    if (aligned && reg_delta_supported(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x))
-        return delta_chunked(L) && in_range32(L, E, M, {q, k, x, beta}) ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
+// Which kernels a delta-rule call takes under the setting `dk`.  `x` is v for the forward pass and grad_out
+// for the backward pass (the views read 16 bytes at a time besides q and k); `out`, forward only, is the view
+// the output is written through, 16 bytes at a time as well; `aligned` says that every contiguous buffer of
+// the call is 16-byte aligned.  The kernels that read and write through buffer resources (split, chunked)
+// address a sequence with 32-bit byte offsets: a view beyond them sends the call to the scan kernels, which
+// use 64-bit addresses (or to the LDS-state kernels, if the shape has no scan kernel), in both directions alike.
+int delta_kind(int dk, bool backward, bool aligned, const fwp_view &q, const fwp_view &k, const fwp_view &x,
+               const fwp_view &beta, const fwp_view *out, int N, int H, int L, int E, int M) {
+    const bool rows16 = aligned && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x) && (!out || reg_view_ok(*out));
+    const bool range32 = in_range32(L, E, M, {q, k, x, beta}) && (!out || in_range32(L, E, M, {*out}));
+    if (rows16 && range32 && delta_split(dk, N, H, L, E, M, {q, k, x}, beta))
+        return delta_phase(dk, backward, L, E, M) ? FWP_KIND_PHASE : FWP_KIND_SPLIT;
+    if (rows16 && reg_delta_supported(E, M))
+        return delta_chunked(dk, L) && range32 ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
     // keys of 128 features: the one-wave blocked kernels at any length (their only alternative is the
     // LDS-state kernels)
-    if (aligned && wide_delta_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(x) &&
-        in_range32(L, E, M, {q, k, x, beta}))
-        return FWP_KIND_CHUNKED;
+    if (rows16 && range32 && wide_delta_dims(E, M)) return FWP_KIND_CHUNKED;
     return FWP_KIND_LDS;
+}
+
+// A forward call of one step that saves nothing goes to the single-step kernels.
+bool delta_single_step(int dk, const fwp_view &v, const fwp_view &ov, const float *W, const float *ckpt, int L,
+                       int E, int M) {
+    return L == 1 && !ckpt && g_step_kernels && dk == FWP_DELTA_AUTO && step_delta_dims(E, M) && reg_view_ok(v) &&
+           reg_view_ok(ov) && aligned16(W);
 }
 
 }  // namespace
@@ -103,7 +113,18 @@ extern "C" {
 int fwp_delta_kind(int backward, fwp_view q, fwp_view k, fwp_view x, fwp_view beta, int N, int H, int L,
                    int E, int M) {
     if (check_dims(N, H, L, E, M, kDefaultChunk)) return FWP_E_SHAPE;
-    return delta_kind(backward != 0, true, q, k, x, beta, N, H, L, E, M);
+    return delta_kind(g_delta_kernels, backward != 0, true, q, k, x, beta, nullptr, N, H, L, E, M);
+}
+
+int fwp_delta_fwd_kind(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, fwp_out_view out, int saves, int N,
+                       int H, int L, int E, int M) {
+    if (check_dims(N, H, L, E, M, kDefaultChunk)) return FWP_E_SHAPE;
+    const int dk = g_delta_kernels;
+    const fwp_view ov = {out.ptr, out.sN, out.sH, out.sL};
+    // a call that saves nothing passes no checkpoint buffer; any aligned address stands for one that does
+    alignas(16) static const float some_ckpt[4] = {};
+    if (delta_single_step(dk, v, ov, some_ckpt, saves ? some_ckpt : nullptr, L, E, M)) return FWP_KIND_STEP;
+    return delta_kind(dk, false, true, q, k, v, beta, &ov, N, H, L, E, M);
 }
 
 int fwp_config(int key, int value) {
@@ -171,13 +192,13 @@ int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, flo
         return FWP_E_NULL;
     if ((vdiff == nullptr) != (ckpt == nullptr)) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    const int dk = g_delta_kernels;          // the one read of the switch in this call
     // the output view takes part in the choice of kernels like an input read 16 bytes at a time
     const fwp_view ov = {out.ptr, out.sN, out.sH, out.sL};
-    const bool aligned = aligned16(vdiff) && aligned16(ckpt) && reg_view_ok(ov) && in_range32(L, E, M, {ov});
-    if (L == 1 && !ckpt && g_step_kernels && g_delta_kernels == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
-        reg_view_ok(v) && reg_view_ok(ov) && aligned16(W))
+    const bool aligned = aligned16(vdiff) && aligned16(ckpt);
+    if (delta_single_step(dk, v, ov, W, ckpt, L, E, M))
         return counted(step_delta_fwd(q, k, v, beta, W, out, N, H, E, M, (hipStream_t)stream));
-    switch (delta_kind(false, aligned, q, k, v, beta, N, H, L, E, M)) {
+    switch (delta_kind(dk, false, aligned, q, k, v, beta, &ov, N, H, L, E, M)) {
         case FWP_KIND_PHASE:
             return phase_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, chunk, (hipStream_t)stream);
         case FWP_KIND_SPLIT:
@@ -211,7 +232,7 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
     const bool aligned = aligned16(vdiff) && aligned16(ckpt) && aligned16(gq) && aligned16(gk) && aligned16(gv);
-    switch (delta_kind(true, aligned, q, k, grad_out, beta, N, H, L, E, M)) {
+    switch (delta_kind(g_delta_kernels, true, aligned, q, k, grad_out, beta, nullptr, N, H, L, E, M)) {
         case FWP_KIND_SPLIT:
             return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
                                    (hipStream_t)stream);
@@ -234,13 +255,14 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
                 int L, int E, int M, int chunk, void *stream) {
     if (bad_view(q) || bad_view(k) || bad_view(v) || !W || !out) return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if (L == 1 && !ckpt && g_step_kernels && g_delta_kernels == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
+    const int dk = g_delta_kernels;          // the one read of the switch in this call
+    if (L == 1 && !ckpt && g_step_kernels && dk == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
         reg_view_ok(v) && aligned16(out) && aligned16(W))
         return counted(step_sum_fwd(q, k, v, W, out, N, H, E, M, (hipStream_t)stream));
     if ((split_delta_dims(E, M) || sum_wide_dims(E, M)) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
         aligned16(out)) {
         // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
-        const bool blocked = in_range32(L, E, M, {q, k, v}) && (!reg_delta_supported(E, M) || delta_chunked(L));
+        const bool blocked = in_range32(L, E, M, {q, k, v}) && (!reg_delta_supported(E, M) || delta_chunked(dk, L));
         if (blocked)
             return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         if (reg_delta_supported(E, M))
@@ -259,7 +281,8 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
         const bool blocked =
-            in_range32(L, E, M, {q, k, v, grad_out}) && (!reg_delta_supported(E, M) || delta_chunked(L));
+            in_range32(L, E, M, {q, k, v, grad_out}) &&
+            (!reg_delta_supported(E, M) || delta_chunked(g_delta_kernels, L));
         if (blocked)
             return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
                                 (hipStream_t)stream);

@@ -11,16 +11,19 @@
 // Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
 
+// FWP_HOST_STUB: a build for tests of this file's host logic on a machine without a GPU (tests/host_stub/):
+// tensors may live in host memory, the stream handed to the C ABI is NULL, and the library it is linked
+// against is a stand-in whose entry points launch nothing.  The product is built without it.
+#ifndef FWP_HOST_STUB
 #include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPFunctions.h>
 #include <c10/hip/HIPStream.h>
+#endif
 
-#include <mutex>
 #include <optional>
 #include <stdexcept>
 #include <string>
 #include <tuple>
-#include <unordered_map>
 
 #include "fwp_hip.h"
 
@@ -82,17 +85,59 @@ at::Tensor rows(const at::Tensor &t_in, fwp_view &v) {
     return t;
 }
 
+#ifndef FWP_HOST_STUB
+// The device check of a GPU runs once per thread that uses it: the last device a thread saw pass is
+// remembered without a lock.
 void require_device(const at::Tensor &t) {
-    static std::mutex mu;
-    static std::unordered_map<int, bool> checked;
     if (!t.is_cuda()) fail("fast-weight operators need tensors on an MI355X GPU, got device '" + t.device().str() + "'");
+    thread_local int passed = -1;
     const int idx = t.get_device();
-    std::lock_guard<std::mutex> lock(mu);
-    if (checked.count(idx)) return;
-    c10::DeviceGuard guard(t.device());
-    check(fwp_check_device(), "device check");
-    checked[idx] = true;
+    if (idx == passed) return;
+    {
+        c10::DeviceGuard guard(t.device());
+        check(fwp_check_device(), "device check");
+    }
+    passed = idx;
 }
+
+void *stream_of(const at::Tensor &t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
+
+struct LaunchGuard {      // makes the tensors' GPU current for a launch when it is not
+    c10::OptionalDeviceGuard guard;
+    explicit LaunchGuard(const at::Tensor &t) {
+        if (t.get_device() != c10::hip::current_device()) guard.reset_device(t.device());
+    }
+};
+#else
+void require_device(const at::Tensor &) {}
+void *stream_of(const at::Tensor &) { return nullptr; }
+struct LaunchGuard {
+    explicit LaunchGuard(const at::Tensor &) {}
+};
+#endif
+
+// The view of a tensor that rows() has already passed (a saved tensor in a backward pass).
+fwp_view view_of(const at::Tensor &t) {
+    return {static_cast<const float *>(t.const_data_ptr()), t.stride(0), t.stride(1), t.stride(2)};
+}
+
+// Several contiguous fp32 results of one call in one allocation: `sizes[i]` floats each, every part
+// starting at a multiple of 4 floats (16 bytes, which the kernels that store 16 bytes at a time need).
+struct Parts {
+    at::Tensor buf;
+    int64_t at = 0;
+    Parts(std::initializer_list<int64_t> sizes, const at::TensorOptions &opts) {
+        int64_t total = 0;
+        for (int64_t n : sizes) total += (n + 3) & ~int64_t(3);
+        buf = at::empty({total}, opts);
+    }
+    // the next part, shaped [a, b, c, d] (contiguous)
+    at::Tensor take(int64_t a, int64_t b, int64_t c, int64_t d) {
+        const at::Tensor t = buf.as_strided({a, b, c, d}, {b * c * d, c * d, d, 1}, at);
+        at += (a * b * c * d + 3) & ~int64_t(3);
+        return t;
+    }
+};
 
 // Every tensor of a call lives on the first one's GPU: the kernels get raw addresses, and an address
 // of host memory or of another GPU would be a memory fault there, not an exception.
@@ -102,8 +147,6 @@ void same_device(const at::Tensor &ref, std::initializer_list<at::Tensor> others
             fail("all tensors of a call must be on the same device: got '" + t.device().str() + "' beside '" +
                  ref.device().str() + "'");
 }
-
-void *stream_of(const at::Tensor &t) { return c10::hip::getCurrentHIPStream(t.get_device()).stream(); }
 
 struct DeltaFn : torch::autograd::Function<DeltaFn> {
     static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Q_in,
@@ -141,16 +184,14 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
             ckpt = vdiff + n_vdiff;
         }
         {
-            c10::OptionalDeviceGuard guard;
-            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            LaunchGuard guard(Q);
             check(fwp_delta_fwd_strided(qv, kv, vv, bv, W.data_ptr<float>(), ov, vdiff, ckpt, (int)N, (int)H,
                                         (int)L, (int)E, (int)M, chunk, stream_of(Q)),
                   "fwp_delta_fwd_strided");
         }
         if (need_grad) {
             ctx->save_for_backward({Q, K, beta, saved});
-            ctx->saved_data["M"] = M;
-            ctx->saved_data["chunk"] = (int64_t)chunk;
+            ctx->saved_data["dims"] = (M << 32) | (int64_t)chunk;       // one entry: value width and chunk
         }
         ctx->set_materialize_grads(false);
         return out;
@@ -164,20 +205,20 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
         if (saved.size() != 4) fail("backward of a forward pass that kept nothing for it");
         const at::Tensor &Q = saved[0], &K = saved[1], &beta = saved[2], &buf = saved[3];
         const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3);
-        const int64_t M = ctx->saved_data["M"].toInt();
-        const int chunk = (int)ctx->saved_data["chunk"].toInt();
-        fwp_view qv, kv, bv, gv_;
-        rows(Q, qv);        // saved after rows(): no copies here
-        rows(K, kv);
-        rows(beta, bv);
+        const int64_t dims = ctx->saved_data.find("dims")->second.toInt();
+        const int64_t M = dims >> 32;
+        const int chunk = (int)(dims & 0xffffffff);
+        // saved after rows(): their views need no checks and no copies
+        const fwp_view qv = view_of(Q), kv = view_of(K), bv = view_of(beta);
+        fwp_view gv_;
         const at::Tensor go = rows(grads[0], gv_);
         const float *vdiff = buf.data_ptr<float>(), *ckpt = vdiff + N * H * L * M;
-        const auto opts = Q.options();
-        at::Tensor gq = at::empty({N, H, L, E}, opts), gk = at::empty({N, H, L, E}, opts),
-                   gv = at::empty({N, H, L, M}, opts), gb = at::empty({N, H, L, 1}, opts);
+        // the four gradients in one allocation
+        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M, N * H * L}, Q.options());
+        const at::Tensor gq = parts.take(N, H, L, E), gk = parts.take(N, H, L, E), gv = parts.take(N, H, L, M),
+                         gb = parts.take(N, H, L, 1);
         {
-            c10::OptionalDeviceGuard guard;
-            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            LaunchGuard guard(Q);
             check(fwp_delta_bwd(qv, kv, bv, vdiff, gv_, ckpt, gq.data_ptr<float>(), gk.data_ptr<float>(),
                                 gv.data_ptr<float>(), gb.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E,
                                 (int)M, chunk, stream_of(Q)),
@@ -211,8 +252,7 @@ struct SumFn : torch::autograd::Function<SumFn> {
             if (!exact) W_init = W.clone();
         }
         {
-            c10::OptionalDeviceGuard guard;
-            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            LaunchGuard guard(Q);
             check(fwp_sum_fwd(qv, kv, vv, W.data_ptr<float>(), out.data_ptr<float>(),
                               need_grad ? ckpt.data_ptr<float>() : nullptr, (int)N, (int)H, (int)L, (int)E, (int)M,
                               chunk, stream_of(Q)),
@@ -236,17 +276,13 @@ struct SumFn : torch::autograd::Function<SumFn> {
         const at::Tensor &Q = saved[0], &K = saved[1], &V = saved[2], &ckpt = saved[3];
         const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3), M = V.size(3);
         const int chunk = (int)ctx->saved_data["chunk"].toInt();
-        fwp_view qv, kv, vv, gv_;
-        rows(Q, qv);        // saved after rows(): no copies here
-        rows(K, kv);
-        rows(V, vv);
+        const fwp_view qv = view_of(Q), kv = view_of(K), vv = view_of(V);     // saved after rows()
+        fwp_view gv_;
         const at::Tensor go = rows(grads[0], gv_);
-        const auto opts = Q.options();
-        at::Tensor gq = at::empty({N, H, L, E}, opts), gk = at::empty({N, H, L, E}, opts),
-                   gv = at::empty({N, H, L, M}, opts);
+        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M}, Q.options());
+        const at::Tensor gq = parts.take(N, H, L, E), gk = parts.take(N, H, L, E), gv = parts.take(N, H, L, M);
         {
-            c10::OptionalDeviceGuard guard;
-            if (Q.get_device() != c10::hip::current_device()) guard.reset_device(Q.device());
+            LaunchGuard guard(Q);
             check(fwp_sum_bwd(qv, kv, vv, gv_, ckpt.data_ptr<float>(),
                               saved.size() > 4 ? saved[4].data_ptr<float>() : nullptr, gq.data_ptr<float>(),
                               gk.data_ptr<float>(), gv.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E, (int)M,
@@ -254,13 +290,6 @@ struct SumFn : torch::autograd::Function<SumFn> {
                   "fwp_sum_bwd");
         }
         return {gq, gk, gv, none, none, none};
-    }
-};
-
-struct LaunchGuard {      // makes the tensors' GPU current for a launch when it is not
-    c10::OptionalDeviceGuard guard;
-    explicit LaunchGuard(const at::Tensor &t) {
-        if (t.get_device() != c10::hip::current_device()) guard.reset_device(t.device());
     }
 };
 
@@ -315,13 +344,12 @@ struct RnnFn : torch::autograd::Function<RnnFn> {
                          &ckpt = saved[5];
         const int64_t N = K.size(0), H = K.size(1), L = K.size(2), D = K.size(3);
         const int chunk = (int)ctx->saved_data["chunk"].toInt();
-        fwp_view kv, bv, gv_;
-        rows(K, kv);
-        rows(beta, bv);
+        const fwp_view kv = view_of(K), bv = view_of(beta);     // saved after rows()
+        fwp_view gv_;
         const at::Tensor go = rows(grads[0], gv_);
-        const auto opts = K.options();
-        at::Tensor gz = at::empty({N, H, L, D}, opts), gk = at::empty({N, H, L, D}, opts),
-                   gv = at::empty({N, H, L, D}, opts), gb = at::empty({N, H, L, 1}, opts);
+        Parts parts({N * H * L * D, N * H * L * D, N * H * L * D, N * H * L}, K.options());
+        const at::Tensor gz = parts.take(N, H, L, D), gk = parts.take(N, H, L, D), gv = parts.take(N, H, L, D),
+                         gb = parts.take(N, H, L, 1);
         {
             LaunchGuard guard(K);
             check(fwp_rnn_bwd(kv, bv, vdiff.data_ptr<float>(), out.data_ptr<float>(), h_init.data_ptr<float>(), gv_,
@@ -406,11 +434,15 @@ struct RecFn : torch::autograd::Function<RecFn> {
         fwp_view gv_;
         const at::Tensor go = rows(grads[0], gv_);
         const auto opts = out.options();
-        at::Tensor gqx = at::empty({N, H, L, D}, opts), gkx = at::empty({N, H, L, D}, opts),
-                   gvx = at::empty({N, H, L, D}, opts), gbx = at::empty({N, H, L, 1}, opts),
-                   gRq = at::empty({1, H, D, D}, opts), gRk = at::empty({1, H, D, D}, opts),
-                   gRv = at::empty({1, H, D, D}, opts), grb = at::empty({1, H, 1, D}, opts),
-                   workspace = at::empty({N, H, 3 * D * D + D}, opts);
+        // the gradients of the inputs in one allocation, those of the parameters in another (they outlive
+        // the step in an optimizer), the scratch for the per-sequence partial sums in a third
+        Parts parts({N * H * L * D, N * H * L * D, N * H * L * D, N * H * L}, opts);
+        const at::Tensor gqx = parts.take(N, H, L, D), gkx = parts.take(N, H, L, D), gvx = parts.take(N, H, L, D),
+                         gbx = parts.take(N, H, L, 1);
+        Parts params({H * D * D, H * D * D, H * D * D, H * D}, opts);
+        const at::Tensor gRq = params.take(1, H, D, D), gRk = params.take(1, H, D, D), gRv = params.take(1, H, D, D),
+                         grb = params.take(1, H, 1, D);
+        const at::Tensor workspace = at::empty({N, H, 3 * D * D + D}, opts);
         {
             LaunchGuard guard(out);
             check(fwp_rec_bwd(q_act.data_ptr<float>(), k_act.data_ptr<float>(), beta_act.data_ptr<float>(),
@@ -508,9 +540,9 @@ struct LstmFn : torch::autograd::Function<LstmFn> {
         const int64_t N = out.size(0), H = out.size(1), L = out.size(2), D = out.size(3);
         const int chunk = (int)ctx->saved_data["chunk"].toInt();
         fwp_view kv[3], bv[3], gov;
-        for (int a = 0; a < 3; a++) {
-            rows(saved[a], kv[a]);
-            rows(saved[3 + a], bv[a]);
+        for (int a = 0; a < 3; a++) {       // saved after rows()
+            kv[a] = view_of(saved[a]);
+            bv[a] = view_of(saved[3 + a]);
         }
         const at::Tensor go = rows(grads[0], gov);
         const auto opts = out.options();

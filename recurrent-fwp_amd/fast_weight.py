@@ -161,9 +161,13 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
         plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
     if plan is None:
         return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
-    if W.dim() != 4 or W.shape[-1] != V.shape[-1]:
+    # the same checks on W as the whole-state path makes (there the slices would hide the caller's W from them)
+    N, H, L, E = Q.shape
+    M = V.shape[-1]
+    if W.shape != (N, H, E, M) or not W.is_contiguous() or W.dtype != torch.float32:
         raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
-    outs = []
+    _lib.same_device(Q, K, V, beta, W)
+    outs, states = [], []
     for first, last, width in plan:
         pad = width - (last - first)
         Vs, Ws = V[..., first:last], W.detach()[..., first:last]
@@ -172,9 +176,12 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
         else:
             Ws = Ws.contiguous()
         out = _operator(Q, K, Vs, beta, Ws, False)
-        with torch.no_grad():
-            W[..., first:last] = Ws[..., :last - first]         # the state after the last step, in place
+        states.append(Ws)
         outs.append(out[..., :last - first] if pad else out)
+    # the state after the last step, in place, once every slice has run: a rejected slice leaves W as it was
+    with torch.no_grad():
+        for (first, last, _), Ws in zip(plan, states):
+            W[..., first:last] = Ws[..., :last - first]
     out = torch.cat(outs, -1)
     if time_major or (time_major is None and rows_lead(Q)):
         out = out.permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)

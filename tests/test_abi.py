@@ -101,6 +101,76 @@ def test_delta_dispatch_keeps_32_bit_kernels_off_views_beyond_their_range(fwp):
     assert lib.fwp_delta_kind(0, small, small, small, beta, 0, 8, 64, D, D) == -2
 
 
+def test_forward_dispatch_knows_the_output_view_and_single_steps(fwp):
+    """fwp_delta_fwd_kind is fwp_delta_fwd_strided's choice of kernels as a pure function: the output view
+    counts like an input read 16 bytes at a time, and a single step that saves nothing has kernels of its own."""
+    L = fwp._lib
+    lib = L.lib()
+    N, H, T, D = 128, 32, 8192, 16
+    small = L.View(4096, 8 * 256 * D, 256 * D, D)
+    beta = L.View(4096, 8 * 256, 256, 1)
+    out_small = L.OutView(4096, 8 * 256 * D, 256 * D, D)
+    assert lib.fwp_delta_fwd_kind(small, small, small, beta, out_small, 1, 4, 8, 256, D, D) == L.KIND_SPLIT
+    # a time-major output whose rows pass 2 GiB: 64-bit scan kernels, not the LDS-state ones
+    big_in = L.View(4096, H * T * D, T * D, D)
+    big_beta = L.View(4096, H * T, T, 1)
+    out_huge = L.OutView(4096, H * D, D, N * H * D)
+    assert lib.fwp_delta_fwd_kind(big_in, big_in, big_in, big_beta, out_huge, 1, N, H, T, D, D) == L.KIND_SCAN
+    assert lib.fwp_delta_kind(0, big_in, big_in, big_in, big_beta, N, H, T, D, D) == L.KIND_CHUNKED
+    # output rows that are not 16-byte aligned: only the LDS-state kernels write those
+    out_odd = L.OutView(4100, 8 * 256 * D, 256 * D, D)
+    assert lib.fwp_delta_fwd_kind(small, small, small, beta, out_odd, 1, 4, 8, 256, D, D) == L.KIND_LDS
+    # one step: kernels of its own when nothing is saved, the scan kernels when the call saves for backward
+    one = L.View(4096, 8 * D, D, D)
+    one_beta = L.View(4096, 8, 1, 1)
+    out_one = L.OutView(4096, 8 * D, D, D)
+    assert lib.fwp_delta_fwd_kind(one, one, one, one_beta, out_one, 0, 4, 8, 1, D, D) == L.KIND_STEP
+    assert lib.fwp_delta_fwd_kind(one, one, one, one_beta, out_one, 1, 4, 8, 1, D, D) == L.KIND_SCAN
+    L.config(L.CFG_STEP_KERNELS, 0)
+    try:
+        assert lib.fwp_delta_fwd_kind(one, one, one, one_beta, out_one, 0, 4, 8, 1, D, D) == L.KIND_SCAN
+    finally:
+        L.config(L.CFG_STEP_KERNELS, 1)
+    assert lib.fwp_delta_fwd_kind(one, one, one, one_beta, out_one, 0, 0, 8, 1, D, D) == -2
+
+
+def test_a_call_is_dispatched_under_one_setting_while_another_thread_changes_it(fwp):
+    """Every entry point reads the FWP_CFG_DELTA_KERNELS switch once.  While a second thread flips it between
+    SCAN and SPLIT, every answer of fwp_delta_kind must be one that a single setting gives (SCAN or SPLIT for
+    16 x 16 states at L = 256): a call that saw SCAN where the several-wave kernels are chosen and SPLIT where
+    the one-wave blocks are would answer CHUNKED, which neither setting does."""
+    import threading
+    L = fwp._lib
+    lib = L.lib()
+    D = 16
+    view = L.View(4096, 8 * 256 * D, 256 * D, D)
+    beta = L.View(4096, 8 * 256, 256, 1)
+    single = {}
+    for setting in (L.DELTA_SCAN, L.DELTA_SPLIT):
+        L.config(L.CFG_DELTA_KERNELS, setting)
+        single[setting] = lib.fwp_delta_kind(0, view, view, view, beta, 96, 8, 256, D, D)
+    assert single == {L.DELTA_SCAN: L.KIND_SCAN, L.DELTA_SPLIT: L.KIND_SPLIT}
+    stop = threading.Event()
+
+    def flip():
+        while not stop.is_set():
+            lib.fwp_config(L.CFG_DELTA_KERNELS, L.DELTA_SCAN)
+            lib.fwp_config(L.CFG_DELTA_KERNELS, L.DELTA_SPLIT)
+
+    t = threading.Thread(target=flip)
+    t.start()
+    try:
+        seen = set()
+        for _ in range(50000):
+            for backward in (0, 1):
+                seen.add(lib.fwp_delta_kind(backward, view, view, view, beta, 96, 8, 256, D, D))
+    finally:
+        stop.set()
+        t.join()
+        L.config(L.CFG_DELTA_KERNELS, L.DELTA_AUTO)
+    assert seen <= set(single.values()), seen
+
+
 def test_value_columns_are_sliced_onto_the_blocked_kernels(fwp):
     """Shapes of the reference's call sites that no kernel takes whole are run by slices of value
     columns, every slice a state shape the blocked kernels take (checked against fwp_delta_kind)."""

@@ -305,6 +305,20 @@ def test_rejects_cpu_tensors_and_bad_shapes(fwp):
         fwp.fast_rnn_v2(dev(v), dev(k), dev(v), dev(W0), dev(beta), dev(v[:, :, :1, :3]))
 
 
+def test_sliced_value_columns_check_w_like_the_whole_state_path(fwp):
+    """A call that runs by slices of value columns (E = 32, M = 128) refuses a W that the whole-state
+    path refuses - wrong shape, not contiguous, not fp32 - with the same error, before anything runs:
+    the caller's W is untouched afterwards."""
+    q, k, v, beta, W0, _ = delta_inputs(77, 2, 2, 40, 32, 128, w0=True)
+    args = [dev(x) for x in (q, k, v, beta)]
+    wide = dev(np.concatenate([W0, W0], -1))
+    for bad in (wide[..., ::2], dev(W0).double(), dev(W0)[..., :64], dev(W0)[:1]):
+        before = bad.clone()
+        with pytest.raises(fwp._lib.FwpError, match="W must be a contiguous fp32"):
+            fwp.fast_weight_delta(*args, bad)
+        assert torch.equal(bad, before)
+
+
 # ------------------------------------------------------------------ output layout
 
 TIME_MAJOR_SHAPES = [

@@ -180,3 +180,65 @@ def test_softmax_of_entries_far_apart_in_a_single_step(fwp, kernels):
         outs = [fwp.fast_rnn_v2(step_of(tz, i), step_of(tk, i), step_of(tv, i), W, step_of(tb, i), h) for i in range(3)]
     check("out", torch.cat(outs, 2), want_out)
     check("h", h, want_h)
+
+
+# Beyond 2048 sequences the single-step kernels put four waves (four sequences) into a workgroup; a count
+# that is not a multiple of four leaves the last workgroup partly filled.
+MANY = 2081
+
+
+@pytest.mark.parametrize("N,H,E,M", [(MANY, 1, 16, 16), (2053, 1, 32, 64), (2052 // 4 + 1, 4, 128, 128)])
+def test_delta_rule_steps_of_many_sequences(fwp, kernels, N, H, E, M):
+    steps = 3
+    q, k, v, beta, W0, _ = delta_inputs(900 + E + M, N, H, steps, E, M, w0=True)
+    want_out, want_W = oracle.delta_fwd(q, k, v, beta, W0)
+    tq, tk, tv, tb = (dev(x) for x in (q, k, v, beta))
+    W = dev(W0)
+    before = fwp._lib.step_launches()
+    with torch.no_grad():
+        outs = [fwp.fast_weight_delta(*(step_of(t, i) for t in (tq, tk, tv, tb)), W) for i in range(steps)]
+    counted(fwp, kernels, steps, before, "delta rule")
+    check("out", torch.cat(outs, 2), want_out)
+    check("W", W, want_W)
+
+
+@pytest.mark.parametrize("D", [16, 32])
+def test_recurrent_operators_steps_of_many_sequences(fwp, kernels, D):
+    steps, N, H = 3, MANY, 1
+    L_ = fwp._lib
+    before = L_.step_launches()
+    with torch.no_grad():
+        z, k, v, W0, beta, h0, _ = rnn_inputs(910 + D, N, H, steps, D, w0=True)
+        want_out, want_W, want_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+        tz, tk, tv, tb = (dev(x) for x in (z, k, v, beta))
+        W, h = dev(W0), dev(h0)
+        outs = [fwp.fast_rnn_v2(step_of(tz, i), step_of(tk, i), step_of(tv, i), W, step_of(tb, i), h) for i in range(steps)]
+        check("rnn out", torch.cat(outs, 2), want_out)
+        check("rnn W", W, want_W)
+        check("rnn h", h, want_h)
+
+        *x, _ = rec_inputs(920 + D, N, 2, steps, D, w0=True)       # two heads: R is indexed by the head
+        want_out, want_W, want_h = oracle.rec_fwd(*x)
+        ts = [dev(a) for a in x]
+        outs = [fwp.rec_update_fwm_tanh(*(step_of(t, i) for t in ts[:4]), *ts[4:8], ts[8], ts[9]) for i in range(steps)]
+        check("rec out", torch.cat(outs, 2), want_out)
+        check("rec W", ts[8], want_W)
+        check("rec h", ts[9], want_h)
+
+        Zs, Ks, Vs, Bs, Ws, h0, c0, _ = lstm_inputs(930 + D, N, H, steps, D, w0=True)
+        want_out, want_cell, want_W, want_h, want_c = oracle.lstm_fwd(Zs, Ks, Vs, Bs, Ws, h0, c0)
+        tz, tk, tv, tb = ([dev(a) for a in xs] for xs in (Zs, Ks, Vs, Bs))
+        tw = [dev(a) for a in Ws]
+        h, c = dev(h0), dev(c0)
+        outs = []
+        for i in range(steps):
+            args = []
+            for a in range(3):
+                args += [step_of(tz[a], i), step_of(tk[a], i), step_of(tv[a], i), step_of(tb[a], i), tw[a]]
+            outs.append(fwp.fast_lstm_v4(*args, h, c)[0])
+        check("lstm out", torch.cat(outs, 2), want_out)
+        for a, gate in enumerate("iuo"):
+            check("lstm W_" + gate, tw[a], want_W[a])
+        check("lstm h", h, want_h)
+        check("lstm c", c, want_c)
+    counted(fwp, kernels, 3 * steps, before, "recurrent operators")

@@ -1,13 +1,17 @@
 """The entry point that allocates nothing (fwp_rec_bwd_static) against fwp_rec_bwd, through the C ABI:
 the same bits, on two calls in a row, the second one smaller (so that what the first left in the
-library's scratch array would show if it were read), and its size limit."""
+library's scratch array would show if it were read), and its size limit.  fwp_rec_bwd itself is held
+to the float64 oracle in test_gpu_parity.py and test_gpu_baseline_sizes.py; here the static entry
+point's gradients are compared with the oracle's directly as well
+(|hip - oracle| <= 1e-4 + 1e-3 |oracle| elementwise)."""
 import ctypes
 
 import numpy as np
 import pytest
 import torch
 
-from helpers import rec_inputs
+import oracle
+from helpers import max_abs, rec_inputs, within
 
 pytestmark = pytest.mark.gpu
 
@@ -65,6 +69,10 @@ def test_static_scratch_entry_point_matches_the_allocating_one(fwp):
         for name, g, w in zip(names, got, want):
             assert np.isfinite(w).all(), name
             assert np.array_equal(g, w), f"{name} differs between fwp_rec_bwd_static and fwp_rec_bwd"
+        exact = oracle.rec_bwd(*(np.asarray(a, np.float64) for a in arrays))
+        for name, g, w in zip(names, got, exact):
+            assert g.shape == w.shape, (name, g.shape, w.shape)
+            assert within(g, w, 1e-4, 1e-3), f"{name} of fwp_rec_bwd_static: max abs err {max_abs(g, w):.3e} against the oracle"
 
 
 def test_static_scratch_limit_is_enforced_before_any_launch(fwp):
