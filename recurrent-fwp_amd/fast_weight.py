@@ -155,12 +155,17 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
     the blocked kernels do not take whole (M = 3 D + 1 of the Delta-Delta layer, M = 128 of the
     Delta-MLP layer: cuda_fast_weight_layer.py:1474-1492,1605-1610) run on them by slices of value
     columns, see :func:`column_plan`; every other call goes straight to the autograd function."""
-    plan = column_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
+    try:        # the common case first: a width pair seen before (two size() calls and one dictionary lookup)
+        plan = _plans[(Q.size(-1), V.size(-1))]
+    except (KeyError, IndexError):
+        plan = column_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
     if plan is not None and Q.shape[2] == 1 and V.shape[-1] in _STEP_WIDTHS and not (
             torch.is_grad_enabled() and any(t.requires_grad for t in (Q, K, V, beta))):
         plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
     if plan is None:
         return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
+    if Q.dim() != 4 or V.dim() != 4:
+        raise _lib.FwpError(f"expected 4-D [N,H,L,D] tensors, got {Q.dim()}-D and {V.dim()}-D")
     # the same checks on W as the whole-state path makes (there the slices would hide the caller's W from them)
     N, H, L, E = Q.shape
     M = V.shape[-1]
