@@ -11,10 +11,9 @@
 //       need the state (X, U, S', and d); one wave prepares, four blocks ahead, what depends on K,
 //       Q, beta only ((I + A)^-T by substitution, lower(Q K^T)^T); with one or two state waves a
 //       further wave, one block behind, forms the output from the state and U handed to it.
-//   backward:  four roles, each a round behind the one before (k_delta_bwd_quad), for every shape
-//       but 64 x 64; for that one NM "adjoint" waves that own the columns of dS
-//       and walk the chain dS -> dU -> dY -> dX -> dS, and NE "state" waves, one block behind, that
-//       own rows [16 eb, 16 eb + 16) of S, rewind them and form g_q, g_k for those columns.
+//   backward:  four roles, each a round behind the one before (k_delta_bwd_quad): what does not
+//       depend on the chain, the chain dS -> dU -> dY -> dX -> dS, the rewind of the state with g_q,
+//       and g_beta with g_k.
 //
 // Hand-over is through LDS in slots used in turn, one workgroup barrier per block: every wave
 // executes the same number of barriers whatever its role.  A last block of fewer than 16 steps
@@ -390,297 +389,8 @@ __global__ __launch_bounds__(64 * (OUT ? (NM == 1 ? 4 : NM + 2) : NM + 1)) void 
 //     g_q = dO S0^T + dPm K
 //     g_k = U dS^T + dPm^T Q - dX S0^T - (M + M^T) K
 //     dS <- dS + Q^T dO - K^T dX
-// The adjoint wave of value columns mb hands over, per block: its columns of dS (before the
-// update, transposed), dX^T, and its share (the sum over its 16 value columns) of dPm, of M, both
-// also transposed, and of g_beta.  The state waves add the shares.  A matrix that is needed
-// transposed is written to LDS transposed instead of being multiplied out a second time.
-
-template <int NE>
-struct AdjRaw {
-    v4f Kt[NE], Qt[NE], Kc[NE], Qc[NE];
-    v4f Oc, Ot, Dt;          // upstream gradient and vdiff, the wave's 16 value columns
-    v4f T;                   // (I + A)^-1 when forward saved it
-    float bcol, brow[4];
-};
-
-template <int NM>
-struct StateRaw {
-    v4f Kc, Qc;                          // the wave's 16 key columns
-    v4f Ot[NM], Dc[NM], Dt[NM];
-    v4f Sck[NM];                         // checkpointed state of the block's chunk, transposed, rows of the wave
-    float bcol, brow[4];
-};
-
-template <int NE, int NM, int PF>
-__global__ __launch_bounds__(64 * (NE + NM)) void k_delta_bwd_split(fwp_view q, fwp_view k, fwp_view beta,
-                                                             const float *__restrict__ vdiff, fwp_view go,
-                                                             const float *__restrict__ ckpt,
-                                                             const float *__restrict__ aux,
-                                                             float *__restrict__ gq, float *__restrict__ gk,
-                                                             float *__restrict__ gv,
-                                                             float *__restrict__ gbeta, int H, int L,
-                                                             int chunk, int nchunk) {
-    constexpr int E = 16 * NE, M = 16 * NM;
-    constexpr int kDX = NE, kDPm = NE + 1, kDPmt = NE + 2, kNM = NE + 3, kNMt = NE + 4;
-    // lower(dO U^T): with one state wave that wave forms it itself from rows it reads anyway (the
-    // adjoint waves are the busier ones), with several the adjoint waves do it once for all
-    constexpr bool kStateDPm = NE == 1;
-    // slot, adjoint wave, matrix: blocks eb = 0..NE-1 of dS^T, then dX^T, dPm, dPm^T,
-    // -strict_lower(dX U^T) and its transpose
-    __shared__ LdsMat xch[2][NM][NE + 5];
-    __shared__ LdsMat scratch[NM][2];       // the adjoint waves'
-    __shared__ LdsMat own_[NE];             // the state waves'
-    __shared__ float gbx[2][NM][16];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
-    const int lane = threadIdx.x % 64;
-    const Geo16 p(lane);
-    const int g = p.g, c = p.c;
-    const int64_t seq = blockIdx.x;
-    const int n = (int)(seq / H), h = (int)(seq % H);
-    // rows of this sequence; lane offsets and block steps in bytes
-    const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
-        kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
-        gob(row(go, n, h, 0), (uint32_t)(((L - 1) * go.sL + M) * 4)),
-        bb(row(beta, n, h, 0), (uint32_t)(((L - 1) * beta.sL + 1) * 4)),
-        db(vdiff + seq * L * M, (uint32_t)(L * M * 4));
-    const unsigned q_step = (unsigned)(kBlk * q.sL * 4), k_step = (unsigned)(kBlk * k.sL * 4),
-                   o_step = (unsigned)(kBlk * go.sL * 4), b_step = (unsigned)(kBlk * beta.sL * 4),
-                   d_step = (unsigned)(kBlk * M * 4);
-    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-    v4f ident;
-#pragma unroll
-    for (int r = 0; r < 4; r++) ident[r] = p.di[r] ? 1.f : 0.f;
-    const int nblk = (L + kBlk - 1) / kBlk;
-    const unsigned o_bc = (unsigned)(c * beta.sL) * 4;
-    unsigned o_br[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++) o_br[r] = (unsigned)((4 * g + r) * beta.sL) * 4;
-
-    if (wave < NM) {
-        // ------------------------------------------------ adjoint wave of value columns mb
-        const int mb = wave;
-        // T = (I + A)^-1 per block as left by the blocked forward (row-major), if it ran
-        const bool have_T = aux && aux[0] == 1.f;
-        const RowBuf tb(have_T ? aux + kAuxHeader + seq * nblk * 256 : nullptr, have_T ? nblk * 1024 : 0);
-        const unsigned o_t = (unsigned)(4 * g * 16 + c) * 4;
-        const unsigned o_kt = (unsigned)(c * k.sL + 4 * g) * 4, o_qt = (unsigned)(c * q.sL + 4 * g) * 4,
-                       o_ot = (unsigned)(c * go.sL + 16 * mb + 4 * g) * 4,
-                       o_dt = (unsigned)(c * M + 16 * mb + 4 * g) * 4;
-        unsigned o_kr[4], o_qr[4], o_or[4];
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            o_kr[r] = (unsigned)((4 * g + r) * k.sL + c) * 4;
-            o_qr[r] = (unsigned)((4 * g + r) * q.sL + c) * 4;
-            o_or[r] = (unsigned)((4 * g + r) * go.sL + 16 * mb + c) * 4;
-        }
-        auto load = [&](AdjRaw<NE> &w, int e) {
-            const int ib = nblk - 1 - e;
-#pragma unroll
-            for (int r = 0; r < 4; r++) w.T[r] = tb.f(o_t + 64 * r, ib * 1024);      // zeros where forward left no T
-            const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
-                           bs = ib * b_step;
-            w.bcol = bb.f(o_bc, bs);
-            w.Ot = gob.f4(o_ot, os);
-            w.Dt = db.f4(o_dt, ds);
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                w.brow[r] = bb.f(o_br[r], bs);
-                w.Oc[r] = gob.f(o_or[r], os);
-            }
-#pragma unroll
-            for (int b = 0; b < NE; b++) {
-                w.Kt[b] = kb.f4(o_kt + 64 * b, ks);
-                w.Qt[b] = qb.f4(o_qt + 64 * b, qs);
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    w.Kc[b][r] = kb.f(o_kr[r] + 64 * b, ks);
-                    w.Qc[b][r] = qb.f(o_qr[r] + 64 * b, qs);
-                }
-            }
-        };
-
-        // dS[eb]: register r = dS[16 eb + 4g + r][16 mb + c]
-        v4f dS[NE];
-#pragma unroll
-        for (int eb = 0; eb < NE; eb++) dS[eb] = zero;
-        const RowBuf gvb(gv + seq * L * M, (uint32_t)(L * M * 4));
-        const unsigned o_gv = (unsigned)(c * M + 16 * mb + 4 * g) * 4;
-        auto block = [&](int e, const AdjRaw<NE> &w) {
-            const int ib = nblk - 1 - e;
-            LdsMat *slot = xch[ib & 1][mb];
-            v4f QK = zero;
-#pragma unroll
-            for (int b = 0; b < NE; b++) QK = tn(w.Qt[b], w.Kt[b], QK);
-            v4f Pm;
-#pragma unroll
-            for (int r = 0; r < 4; r++) Pm[r] = (p.lo[r] || p.di[r]) ? QK[r] : 0.f;
-            v4f T = w.T;
-            if (!have_T) {
-                v4f G = zero, A, At;
-#pragma unroll
-                for (int b = 0; b < NE; b++) G = tn(w.Kt[b], w.Kt[b], G);
-#pragma unroll
-                for (int r = 0; r < 4; r++) {
-                    A[r] = p.lo[r] ? w.brow[r] * G[r] : 0.f;
-                    At[r] = p.up[r] ? w.bcol * G[r] : 0.f;
-                }
-                T = inv_unit_triangular_lds(At, A, ident, scratch[mb], p, lane);      // (I + A)^-1
-            }
-            const v4f Ut = w.bcol * w.Dt;
-#pragma unroll
-            for (int eb = 0; eb < NE; eb++) slot[eb].put_t(p, dS[eb]);
-            v4f dU = tn(Pm, w.Oc, zero);
-#pragma unroll
-            for (int eb = 0; eb < NE; eb++) dU = tn(w.Kt[eb], dS[eb], dU);
-            const v4f dY = tn(T, dU, zero);
-            scratch[mb][0].put_t(p, dY);
-            v4f ndX;
-#pragma unroll
-            for (int r = 0; r < 4; r++) ndX[r] = -(w.brow[r] * dY[r]);
-#pragma unroll
-            for (int eb = 0; eb < NE; eb++) {
-                dS[eb] = tn(w.Qc[eb], w.Oc, dS[eb]);
-                dS[eb] = tn(w.Kc[eb], ndX, dS[eb]);
-            }
-            v4f Z = zero;
-            if constexpr (!kStateDPm) Z = tn(w.Ot, Ut, zero);      // dO U^T
-            __builtin_amdgcn_wave_barrier();
-            const v4f dYt = scratch[mb][0].get(lane);
-            const v4f dXt = w.bcol * dYt;
-            float gb = 0.f;
-#pragma unroll
-            for (int r = 0; r < 4; r++) gb = fmaf(dYt[r], w.Dt[r], gb);
-            // register r = g_v[t0 + c][16 mb + 4g + r]
-            gvb.st4(dXt, o_gv, ib * d_step);
-            slot[kDX].put(lane, dXt);
-            const v4f M = tn(dXt, Ut, zero);       // dX U^T
-            {   // share of g_beta[t0 + c]: the four 16-lane rows hold partial sums
-                float y = gb;
-                swap16(gb, y);
-                gb += y;
-                y = gb;
-                swap32(gb, y);
-                gb += y;
-                if (g == 0) gbx[ib & 1][mb][c] = gb;
-            }
-            v4f dPm, nM;
-#pragma unroll
-            for (int r = 0; r < 4; r++) {
-                dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-                nM[r] = p.lo[r] ? -M[r] : 0.f;
-            }
-            if constexpr (!kStateDPm) {
-                slot[kDPm].put(lane, dPm);
-                slot[kDPmt].put_t(p, dPm);
-            }
-            slot[kNM].put(lane, nM);
-            slot[kNMt].put_t(p, nM);
-        };
-        ring_loop<PF, AdjRaw<NE>>(nblk, load, block);
-        lds_barrier();        // the state waves' last block
-        return;
-    }
-
-    // ---------------------------------------------------- state wave of key columns [16 eb, 16 eb + 16)
-    const int eb = wave - NM;
-    LdsMat *own = &own_[eb];
-    const unsigned o_ot = (unsigned)(c * go.sL + 4 * g) * 4, o_dt = (unsigned)(c * M + 4 * g) * 4;
-    unsigned o_kr[4], o_qr[4], o_dr[4];
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        o_kr[r] = (unsigned)((4 * g + r) * k.sL + 16 * eb + c) * 4;
-        o_qr[r] = (unsigned)((4 * g + r) * q.sL + 16 * eb + c) * 4;
-        o_dr[r] = (unsigned)((4 * g + r) * M + c) * 4;
-    }
-    const RowBuf cb(ckpt + seq * nchunk * E * M, (uint32_t)(nchunk * E * M * 4));
-    const unsigned o_ck = (unsigned)((16 * eb + c) * M + 4 * g) * 4;
-    const ChunkOf chunk_of(chunk);
-    auto load = [&](StateRaw<NM> &w, int e) {
-        const int ib = nblk - 1 - e;
-        {   // always loaded, so that no load is left to be issued (and waited for) inside the block
-            const unsigned cs = chunk_of(ib) * (E * M * 4);
-#pragma unroll
-            for (int mb = 0; mb < NM; mb++) w.Sck[mb] = cb.f4(o_ck + 64 * mb, cs);
-        }
-        const unsigned ks = ib * k_step, qs = ib * q_step, os = ib * o_step, ds = ib * d_step,
-                       bs = ib * b_step;
-        w.bcol = bb.f(o_bc, bs);
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            w.brow[r] = bb.f(o_br[r], bs);
-            w.Kc[r] = kb.f(o_kr[r], ks);
-            w.Qc[r] = qb.f(o_qr[r], qs);
-        }
-#pragma unroll
-        for (int b = 0; b < NM; b++) {
-            w.Ot[b] = gob.f4(o_ot + 64 * b, os);
-            w.Dt[b] = db.f4(o_dt + 64 * b, ds);
-#pragma unroll
-            for (int r = 0; r < 4; r++) w.Dc[b][r] = db.f(o_dr[r] + 64 * b, ds);
-        }
-    };
-
-    // St[mb]: register r = S[16 eb + c][16 mb + 4g + r]  (block (mb, eb) of S^T)
-    v4f St[NM];
-    const RowBuf gqb(gq + seq * L * E, (uint32_t)(L * E * 4)), gkb(gk + seq * L * E, (uint32_t)(L * E * 4)),
-        gbb(gbeta + seq * L, (uint32_t)(L * 4));
-    const unsigned o_g = (unsigned)(c * E + 16 * eb + 4 * g) * 4, e_step = (unsigned)(kBlk * E * 4);
-    auto block = [&](int e, const StateRaw<NM> &w) {
-        const int ib = nblk - 1 - e;
-        if (chunk_of.closes(ib) || ib + 1 == nblk) {      // last block of a chunk: the state after it is checkpointed
-#pragma unroll
-            for (int mb = 0; mb < NM; mb++) St[mb] = w.Sck[mb];
-        }
-        // state at the start of the block, transposed: S0^T = S'^T - U^T K
-        v4f Ut[NM];
-#pragma unroll
-        for (int mb = 0; mb < NM; mb++) {
-            Ut[mb] = w.bcol * w.Dt[mb];
-            v4f nU;
-#pragma unroll
-            for (int r = 0; r < 4; r++) nU[r] = -(w.brow[r] * w.Dc[mb][r]);
-            St[mb] = tn(nU, w.Kc, St[mb]);
-        }
-        v4f gQt = zero, gKt = zero;
-#pragma unroll
-        for (int mb = 0; mb < NM; mb++) gQt = tn(St[mb], w.Ot[mb], gQt);
-        // what the adjoint waves left for this block
-        v4f dPm = zero, dPmt = zero, nMs = zero;
-        float gb = 0.f;
-        if constexpr (kStateDPm) {
-            v4f Z = zero;
-#pragma unroll
-            for (int mb = 0; mb < NM; mb++) Z = tn(w.Ot[mb], Ut[mb], Z);      // dO U^T
-#pragma unroll
-            for (int r = 0; r < 4; r++) dPm[r] = (p.lo[r] || p.di[r]) ? Z[r] : 0.f;
-            own[0].put_t(p, dPm);
-            dPmt = own[0].get(lane);
-        }
-#pragma unroll
-        for (int mb = 0; mb < NM; mb++) {
-            const LdsMat *slot = xch[ib & 1][mb];
-            if constexpr (!kStateDPm) {
-                dPm += slot[kDPm].get(lane);
-                dPmt += slot[kDPmt].get(lane);
-            }
-            nMs += slot[kNM].get(lane) + slot[kNMt].get(lane);
-            gb += gbx[ib & 1][mb][c];
-            const v4f dSt = slot[eb].get(lane), dXt = slot[kDX].get(lane);     // dSt: block (mb, eb) of dS^T
-            gKt = tn(dSt, Ut[mb], gKt);
-            gKt = tn(St[mb], -dXt, gKt);
-        }
-        gQt = tn(w.Kc, dPmt, gQt);
-        gKt = tn(w.Qc, dPm, gKt);
-        gKt = tn(w.Kc, nMs, gKt);
-        // register r = gradient[t0 + c][16 eb + 4g + r]
-        gqb.st4(gQt, o_g, ib * e_step);
-        gkb.st4(gKt, o_g, ib * e_step);
-        if (eb == 0 && g == 0) gbb.st(gb, c * 4, ib * kBlk * 4);
-    };
-
-    lds_barrier();            // the adjoint waves' first block
-    ring_loop<PF, StateRaw<NM>>(nblk, load, block);
-}
+// A matrix that is needed transposed is written to LDS transposed instead of being multiplied out a
+// second time.
 
 // ------------------------------------------------- backward in four roles
 //
@@ -1149,14 +859,6 @@ void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp
                            0, s,
                            q, k, v, beta, W, out, vdiff, ckpt, aux, H, L, chunk, nchunk);
 }
-template <int NE, int NM>
-void launch_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go, const float *ckpt,
-                const float *aux, float *gq, float *gk, float *gv, float *gbeta, int nseq, int H, int L,
-                int chunk, int nchunk, hipStream_t s) {
-    hipLaunchKernelGGL((k_delta_bwd_split<NE, NM, bwd_ring(NE)>), dim3(nseq), dim3(64 * (NE + NM)),
-                       0, s, q, k,
-                       beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, H, L, chunk, nchunk);
-}
 }  // namespace
 
 // the (NE, NM) pairs of split_delta_dims
@@ -1193,15 +895,12 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
     if (L <= 512) { Q(1, 1, 1, 1, 2) }
     Q(1, 1, 1, 1, 3) Q(2, 1, 1, 1, 3) Q(1, 2, 1, 1, 3) Q(2, 2, 2, 2, 3) Q(4, 1, 2, 1, 2) Q(6, 1, 3, 1, 2)
     Q(4, 2, 2, 1, 2) Q(1, 4, 1, 1, 2) Q(2, 4, 1, 1, 2) Q(6, 2, 3, 1, 1)
+    // 64 x 64: ten waves (two for P, four on the chain, two each for R and G with two key tiles apiece), one block
+    // in flight, 136 KB of LDS.  256 sequences of 512 steps: 111 us; with R and G on four waves each 125 us
+    // (139 us with P on one wave), on one wave each 153 us, with two blocks in flight 377 us (spills).
+    Q(4, 4, 2, 2, 1)
 #undef Q
-    // 64 x 64: adjoint and state waves (with four roles the waves that own four key tiles each spill, and
-    // 256 sequences of 512 steps take 175 against 163 us)
-#define X(ne, nm)                                                                                        \
-    if (E == 16 * ne && M == 16 * nm)                                                                    \
-        launch_bwd<ne, nm>(q, k, beta, vdiff, go, ckpt, aux, gq, gk, gv, gbeta, N * H, H, L, chunk, nchunk, s);
-    X(4, 4)
-#undef X
-    return (int)hipGetLastError();
+    return FWP_E_SHAPE;
 }
 
 }  // namespace fwp
