@@ -637,20 +637,33 @@ def main():
     torch.autograd.set_multithreading_enabled(False)
     step, _ = gpu_step_fn(name, pkg, arrays)
 
-    def timed_steps(fn):
-        for _ in range(args.warmup):
+    def timed_steps(fn, warmup=None, steps=None):
+        """(seconds per step, seconds of host time per step spent issuing) over `steps` steps after `warmup`
+        untimed ones, a synchronisation on either side."""
+        warmup = args.warmup if warmup is None else warmup
+        steps = args.steps if steps is None else steps
+        for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             fn()
+        t_issued = time.perf_counter()
         torch.cuda.synchronize()
-        return (time.perf_counter() - t0) / args.steps
+        return (time.perf_counter() - t0) / steps, (t_issued - t0) / steps
 
-    # the per-kernel leg first: with few timed steps (the default command of a fresh box times a
-    # millisecond of work) the step would otherwise be measured while the GPU is still waking up
+    # Three legs, in this order.  (1) The per-kernel leg: back-to-back launches through the C ABI.  (2) The
+    # steady state of the eager step: 2000 steps after 200, as a training loop runs them.  (3) The window the
+    # command line asks for: --warmup untimed steps, then exactly --steps timed ones; `value` is this one.
+    # With the default command of a fresh box (20 steps after 5, one millisecond of work) leg (3) on its own
+    # measured the process warming up - the first few hundred calls of the eager path issue 10-40 % slower
+    # than later ones, and the GPU runs a 1 ms burst after an idle spell 10 % slower than sustained work -
+    # so it comes last; legs (1) and (2) are reported beside it under "kernels" and "steady".
     t_f, t_b, abi_step = kernel_times(name, pkg, arrays, 100)
-    eager_s = timed_steps(step)
+    steady_steps = 2000 if w["T"] * w["B"] * w["H"] * w["D"] <= 96 * 8 * 256 * 16 * 2 else 300
+    steady_s, steady_issue_s = timed_steps(step, steady_steps // 10, steady_steps)
+    abi_s, _ = timed_steps(abi_step, 5, 20)
+    eager_s, eager_issue_s = timed_steps(step)
     launch = "eager calls of the autograd Function"
     step_s = eager_s
     if args.graph:
@@ -667,7 +680,7 @@ def main():
         torch.cuda.synchronize()
         with torch.cuda.graph(graph):
             abi_step()
-        step_s = timed_steps(graph.replay)
+        step_s, _ = timed_steps(graph.replay)
         launch = "hipGraph replay of reset+forward+backward recorded through the C ABI"
     ms = step_s * 1e3
     value = tokens / step_s
@@ -693,6 +706,13 @@ def main():
                     "hbm_frac_of_8TBps": (fwd_bytes + bwd_bytes) / kernel_s / PEAK_HBM,
                     "step_valu_frac_of_157.3TF": flops / (ms * 1e-3) / PEAK_VALU,
                     "eager_tokens_per_s": tokens / eager_s, "eager_ms_per_step": eager_s * 1e3},
+        # host time per step spent issuing the timed steps (the rest of a step's time the host waits for the GPU)
+        "issue_ms_per_step": eager_issue_s * 1e3,
+        # the same eager step in steady state, and reset + forward + backward straight through the C ABI on
+        # preallocated buffers (no allocation, no autograd engine) in a window of 20 steps after 5
+        "steady": {"steps": steady_steps, "ms_per_step": steady_s * 1e3, "tokens_per_s": tokens / steady_s,
+                   "issue_ms_per_step": steady_issue_s * 1e3},
+        "c_abi_step": {"steps": 20, "ms_per_step": abi_s * 1e3, "tokens_per_s": tokens / abi_s},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(name, arrays, w, args.cpu_reps)

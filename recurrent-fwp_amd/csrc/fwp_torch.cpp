@@ -10,6 +10,8 @@
 // time through a Python autograd.Function, and a single inference step even less GPU time.
 // Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
+#include <torch/csrc/autograd/functions/utils.h>
+#include <torch/csrc/autograd/saved_variable.h>
 
 // FWP_HOST_STUB: a build for tests of this file's host logic on a machine without a GPU (tests/host_stub/):
 // tensors may live in host memory, the stream handed to the C ABI is NULL, and the library it is linked
@@ -20,6 +22,7 @@
 #include <c10/hip/HIPStream.h>
 #endif
 
+#include <mutex>
 #include <optional>
 #include <stdexcept>
 #include <string>
@@ -148,32 +151,98 @@ void same_device(const at::Tensor &ref, std::initializer_list<at::Tensor> others
                  ref.device().str() + "'");
 }
 
-struct DeltaFn : torch::autograd::Function<DeltaFn> {
-    static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Q_in,
-                              const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &beta_in,
-                              const at::Tensor &W, bool need_grad, int64_t time_major) {
-        require_device(Q_in);
-        same_device(Q_in, {K_in, V_in, beta_in, W});
-        if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
-        const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
-        if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}) ||
-            beta_in.sizes() != at::IntArrayRef({N, H, L, 1}))
-            fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in) +
-                 " beta" + shape_of(beta_in));
-        if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
-            fail("W must be a contiguous fp32 [N,H,E,M] tensor");
-        // out follows Q's memory order unless told otherwise: steps outermost for a permuted view of
-        // [L,N,H,E] storage (the reference's layers), so that their reshape to [L,N,H*M] is a view
-        if (time_major < 0) {
-            const int64_t sN = Q_in.stride(0), sH = Q_in.stride(1), sL = Q_in.stride(2);
-            time_major = L > 1 && (N > 1 || H > 1) && (N <= 1 || sL > sN) && (H <= 1 || sL > sH);
+// The delta rule's backward as a node of the autograd graph in its own right, the way PyTorch's
+// own operators are (a saved input is a SavedVariable, the result gets the node by set_history),
+// rather than through torch::autograd::Function: a forward + backward pair of this operator takes
+// about as long on the GPU as the interpreter and the autograd engine take to issue it, and the
+// generic wrapper's bookkeeping per call (context object, maps of saved data, variable infos, the
+// demangled class name per backward call) was a tenth of that.  Same saved tensors, same results.
+struct DeltaBackward : torch::autograd::Node {
+    torch::autograd::SavedVariable Q_, K_, beta_;
+    at::Tensor buf_;             // v - v_old [N,H,L,M] and the checkpoints behind it (no graph of its own)
+    int64_t M_ = 0;
+    int chunk_ = 0;
+    bool released_ = false;
+
+    std::string name() const override { return "FwpDeltaBackward"; }
+
+    void release_variables() override {
+        std::lock_guard<std::mutex> lock(mutex_);
+        Q_.reset_data();
+        K_.reset_data();
+        beta_.reset_data();
+        buf_.reset();
+        released_ = true;
+    }
+
+    // one gradient per input edge: Q, K, V, beta
+    torch::autograd::variable_list apply(torch::autograd::variable_list &&grads) override {
+        std::lock_guard<std::mutex> lock(mutex_);      // backward passes of one graph may run on several threads
+        torch::autograd::variable_list res(4);
+        if (grads.empty() || !grads[0].defined()) return res;
+        TORCH_CHECK(!released_, torch::autograd::ERR_BACKWARD_TWICE);
+        const at::Tensor Q = Q_.unpack(), K = K_.unpack(), beta = beta_.unpack();
+        const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3), M = M_;
+        // saved after rows(): their views need no checks and no copies
+        const fwp_view qv = view_of(Q), kv = view_of(K), bv = view_of(beta);
+        same_device(Q, {grads[0]});
+        fwp_view gv_;
+        const at::Tensor go = rows(grads[0], gv_);
+        const float *vdiff = buf_.data_ptr<float>(), *ckpt = vdiff + N * H * L * M;
+        // the four gradients in one allocation
+        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M, N * H * L}, Q.options());
+        res[0] = parts.take(N, H, L, E);
+        res[1] = parts.take(N, H, L, E);
+        res[2] = parts.take(N, H, L, M);
+        res[3] = parts.take(N, H, L, 1);
+        {
+            LaunchGuard guard(Q);
+            check(fwp_delta_bwd(qv, kv, bv, vdiff, gv_, ckpt, res[0].data_ptr<float>(), res[1].data_ptr<float>(),
+                                res[2].data_ptr<float>(), res[3].data_ptr<float>(), (int)N, (int)H, (int)L, (int)E,
+                                (int)M, chunk_, stream_of(Q)),
+                  "fwp_delta_bwd");
         }
+        return res;
+    }
+};
+
+// time_major: < 0 = out's memory follows Q's, 1 = [L,N,H,M] storage, 0 = contiguous [N,H,L,M]
+at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const at::Tensor &V_in,
+                         const at::Tensor &beta_in, const at::Tensor &W, int64_t time_major) {
+    require_device(Q_in);
+    same_device(Q_in, {K_in, V_in, beta_in, W});
+    if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
+    const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
+    if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}) ||
+        beta_in.sizes() != at::IntArrayRef({N, H, L, 1}))
+        fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in) +
+             " beta" + shape_of(beta_in));
+    if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
+        fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+    const bool need_grad = at::GradMode::is_enabled() && (Q_in.requires_grad() || K_in.requires_grad() ||
+                                                          V_in.requires_grad() || beta_in.requires_grad());
+    std::shared_ptr<DeltaBackward> node;
+    if (need_grad) {
+        node = std::shared_ptr<DeltaBackward>(new DeltaBackward(), torch::autograd::deleteNode);
+        node->set_next_edges(torch::autograd::collect_next_edges(Q_in, K_in, V_in, beta_in));
+    }
+    // out follows Q's memory order unless told otherwise: steps outermost for a permuted view of
+    // [L,N,H,E] storage (the reference's layers), so that their reshape to [L,N,H*M] is a view
+    if (time_major < 0) {
+        const int64_t sN = Q_in.stride(0), sH = Q_in.stride(1), sL = Q_in.stride(2);
+        time_major = L > 1 && (N > 1 || H > 1) && (N <= 1 || sL > sN) && (H <= 1 || sL > sH);
+    }
+    at::Tensor out;
+    {
+        // what follows is below autograd: copies of unaligned views and the result's permutation record nothing
+        at::AutoDispatchBelowADInplaceOrView below;
         fwp_view qv, kv, vv, bv;
         const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), V = rows(V_in, vv), beta = rows(beta_in, bv);
         const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
         const auto opts = Q.options();
-        at::Tensor out = time_major ? at::empty({L, N, H, M}, opts).permute({1, 2, 0, 3}) : at::empty({N, H, L, M}, opts), saved;
+        out = time_major ? at::empty({L, N, H, M}, opts).permute({1, 2, 0, 3}) : at::empty({N, H, L, M}, opts);
         const fwp_out_view ov = {out.data_ptr<float>(), out.stride(0), out.stride(1), out.stride(2)};
+        at::Tensor saved;
         float *vdiff = nullptr, *ckpt = nullptr;
         if (need_grad) {
             // v - v_old [N,H,L,M] and the checkpoints behind it, one allocation
@@ -190,43 +259,18 @@ struct DeltaFn : torch::autograd::Function<DeltaFn> {
                   "fwp_delta_fwd_strided");
         }
         if (need_grad) {
-            ctx->save_for_backward({Q, K, beta, saved});
-            ctx->saved_data["dims"] = (M << 32) | (int64_t)chunk;       // one entry: value width and chunk
+            // inputs as they are (a SavedVariable of an input keeps the tensor itself), copies as plain tensors
+            node->Q_ = torch::autograd::SavedVariable(Q, false);
+            node->K_ = torch::autograd::SavedVariable(K, false);
+            node->beta_ = torch::autograd::SavedVariable(beta, false);
+            node->buf_ = std::move(saved);
+            node->M_ = M;
+            node->chunk_ = chunk;
         }
-        ctx->set_materialize_grads(false);
-        return out;
     }
-
-    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
-                                                 torch::autograd::tensor_list grads) {
-        const at::Tensor none;
-        if (!grads[0].defined()) return {none, none, none, none, none, none, none};
-        const auto saved = ctx->get_saved_variables();
-        if (saved.size() != 4) fail("backward of a forward pass that kept nothing for it");
-        const at::Tensor &Q = saved[0], &K = saved[1], &beta = saved[2], &buf = saved[3];
-        const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3);
-        const int64_t dims = ctx->saved_data.find("dims")->second.toInt();
-        const int64_t M = dims >> 32;
-        const int chunk = (int)(dims & 0xffffffff);
-        // saved after rows(): their views need no checks and no copies
-        const fwp_view qv = view_of(Q), kv = view_of(K), bv = view_of(beta);
-        fwp_view gv_;
-        const at::Tensor go = rows(grads[0], gv_);
-        const float *vdiff = buf.data_ptr<float>(), *ckpt = vdiff + N * H * L * M;
-        // the four gradients in one allocation
-        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M, N * H * L}, Q.options());
-        const at::Tensor gq = parts.take(N, H, L, E), gk = parts.take(N, H, L, E), gv = parts.take(N, H, L, M),
-                         gb = parts.take(N, H, L, 1);
-        {
-            LaunchGuard guard(Q);
-            check(fwp_delta_bwd(qv, kv, bv, vdiff, gv_, ckpt, gq.data_ptr<float>(), gk.data_ptr<float>(),
-                                gv.data_ptr<float>(), gb.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E,
-                                (int)M, chunk, stream_of(Q)),
-                  "fwp_delta_bwd");
-        }
-        return {gq, gk, gv, gb, none, none, none};
-    }
-};
+    if (need_grad) torch::autograd::set_history(out, node);
+    return out;
+}
 
 struct SumFn : torch::autograd::Function<SumFn> {
     // exact: grad_Q is the gradient of the recurrence as written; otherwise a carried-in state is left
@@ -263,7 +307,7 @@ struct SumFn : torch::autograd::Function<SumFn> {
             else ctx->save_for_backward({Q, K, V, ckpt, W_init});
             ctx->saved_data["chunk"] = (int64_t)chunk;
         }
-        ctx->set_materialize_grads(false);
+        if (ctx) ctx->set_materialize_grads(false);
         return out;
     }
 
@@ -330,7 +374,7 @@ struct RnnFn : torch::autograd::Function<RnnFn> {
             ctx->save_for_backward({K, beta, vdiff, out, h_init, ckpt});
             ctx->saved_data["chunk"] = (int64_t)chunk;
         }
-        ctx->set_materialize_grads(false);
+        if (ctx) ctx->set_materialize_grads(false);
         return out;
     }
 
@@ -366,6 +410,10 @@ at::Tensor fast_rnn_v2(const at::Tensor &Z, const at::Tensor &K, const at::Tenso
                        const at::Tensor &beta, const at::Tensor &h0) {
     const bool need_grad = at::GradMode::is_enabled() && (Z.requires_grad() || K.requires_grad() || V.requires_grad() ||
                                                           W.requires_grad() || beta.requires_grad() || h0.requires_grad());
+    if (!need_grad) {       // nothing to record: straight to the launch (single steps of an actor or a decoder)
+        at::AutoDispatchBelowADInplaceOrView below;
+        return RnnFn::forward(nullptr, Z, K, V, W, beta, h0, false);
+    }
     return RnnFn::apply(Z, K, V, W, beta, h0, need_grad);
 }
 
@@ -416,7 +464,7 @@ struct RecFn : torch::autograd::Function<RecFn> {
             ctx->save_for_backward({out, h_init, Rq, Rk, Rv, rb, q_act, k_act, beta_act, vdiff, ckpt});
             ctx->saved_data["chunk"] = (int64_t)chunk;
         }
-        ctx->set_materialize_grads(false);
+        if (ctx) ctx->set_materialize_grads(false);
         return out;
     }
 
@@ -463,7 +511,11 @@ at::Tensor rec_update_fwm_tanh(const at::Tensor &qx, const at::Tensor &kx, const
                                const at::Tensor &r_b, const at::Tensor &W, const at::Tensor &h0) {
     bool any = false;
     for (const at::Tensor *t : {&qx, &kx, &vx, &bx, &R_q, &R_k, &R_v, &r_b, &W, &h0}) any = any || t->requires_grad();
-    return RecFn::apply(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0, at::GradMode::is_enabled() && any);
+    if (!(at::GradMode::is_enabled() && any)) {
+        at::AutoDispatchBelowADInplaceOrView below;
+        return RecFn::forward(nullptr, qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0, false);
+    }
+    return RecFn::apply(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0, true);
 }
 
 struct LstmFn : torch::autograd::Function<LstmFn> {
@@ -523,8 +575,8 @@ struct LstmFn : torch::autograd::Function<LstmFn> {
             ctx->save_for_backward({Kr[0], Kr[1], Kr[2], Br[0], Br[1], Br[2], vdiff, gates, out, cell, h_init, c_init, ckpt});
             ctx->saved_data["chunk"] = (int64_t)chunk;
         }
-        ctx->mark_non_differentiable({cell});
-        ctx->set_materialize_grads(false);
+        if (ctx) ctx->mark_non_differentiable({cell});
+        if (ctx) ctx->set_materialize_grads(false);
         return {out, cell};
     }
 
@@ -575,24 +627,29 @@ std::tuple<at::Tensor, at::Tensor> fast_lstm_v4(
     bool any = false;
     for (const at::Tensor *t : {&Zi, &Ki, &Vi, &bi, &Wi, &Zu, &Ku, &Vu, &bu, &Wu, &Zo, &Ko, &Vo, &bo, &Wo, &h0, &c0})
         any = any || t->requires_grad();
-    const auto r = LstmFn::apply(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0,
-                                 at::GradMode::is_enabled() && any);
+    if (!(at::GradMode::is_enabled() && any)) {
+        at::AutoDispatchBelowADInplaceOrView below;
+        const auto r = LstmFn::forward(nullptr, Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0, false);
+        return {r[0], r[1]};
+    }
+    const auto r = LstmFn::apply(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0, true);
     return {r[0], r[1]};
 }
 
 at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
                            bool exact) {
     const bool need_grad = at::GradMode::is_enabled() && (Q.requires_grad() || K.requires_grad() || V.requires_grad());
+    if (!need_grad) {
+        at::AutoDispatchBelowADInplaceOrView below;
+        return SumFn::forward(nullptr, Q, K, V, W, exact, false);
+    }
     return SumFn::apply(Q, K, V, W, exact, need_grad);
 }
 
 // time_major: None = out's memory follows Q's, True = [L,N,H,M] storage, False = contiguous [N,H,L,M]
 at::Tensor fast_weight_delta(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V,
                              const at::Tensor &beta, const at::Tensor &W, std::optional<bool> time_major) {
-    // decided here: forward itself runs with gradient mode switched off
-    const bool need_grad = at::GradMode::is_enabled() &&
-                           (Q.requires_grad() || K.requires_grad() || V.requires_grad() || beta.requires_grad());
-    return DeltaFn::apply(Q, K, V, beta, W, need_grad, time_major.has_value() ? (int64_t)*time_major : (int64_t)-1);
+    return delta_forward(Q, K, V, beta, W, time_major.has_value() ? (int64_t)*time_major : (int64_t)-1);
 }
 
 void set_error_class(py::object cls) {
