@@ -93,9 +93,6 @@ int delta_kind(int dk, bool backward, bool aligned, const fwp_view &q, const fwp
         return delta_phase(dk, backward, L, E, M) ? FWP_KIND_PHASE : FWP_KIND_SPLIT;
     if (rows16 && reg_delta_supported(E, M))
         return delta_chunked(dk, L) && range32 ? FWP_KIND_CHUNKED : FWP_KIND_SCAN;
-    // keys of 128 features: the one-wave blocked kernels at any length (their only alternative is the
-    // LDS-state kernels)
-    if (rows16 && range32 && wide_delta_dims(E, M)) return FWP_KIND_CHUNKED;
     return FWP_KIND_LDS;
 }
 
@@ -204,8 +201,6 @@ int fwp_delta_fwd_strided(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, flo
         case FWP_KIND_SPLIT:
             return split_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         case FWP_KIND_CHUNKED:
-            if (wide_delta_dims(E, M))
-                return mfma_delta_wide_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
             return mfma_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
         case FWP_KIND_SCAN:
             return reg_delta_fwd(q, k, v, beta, W, out, vdiff, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
@@ -237,9 +232,6 @@ int fwp_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp
             return split_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M, chunk,
                                    (hipStream_t)stream);
         case FWP_KIND_CHUNKED:
-            if (wide_delta_dims(E, M))
-                return mfma_delta_wide_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, M,
-                                           chunk, (hipStream_t)stream);
             return mfma_delta_bwd(q, k, beta, vdiff, grad_out, ckpt, gq, gk, gv, gbeta, N, H, L, E, chunk,
                                   (hipStream_t)stream);
         case FWP_KIND_SCAN:

@@ -113,14 +113,6 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
                    const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
                    int L, int D, int chunk, hipStream_t s);
 
-// Delta rule with keys of 128 features and 16 value columns, one wave per sequence.
-bool wide_delta_dims(int E, int M);
-int mfma_delta_wide_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
-                        float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s);
-int mfma_delta_wide_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
-                        const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
-                        int L, int E, int M, int chunk, hipStream_t s);
-
 // the widest sum-rule shapes, built in a translation unit of their own
 bool sum_wide_dims(int E, int M);
 int mfma_sum_wide_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,

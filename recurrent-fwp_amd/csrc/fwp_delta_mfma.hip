@@ -491,7 +491,7 @@ float *delta_aux_of(const float *ckpt, int N, int H, int L, int E, int M, int ch
 }
 
 // Shapes whose checkpoint buffer has the auxiliary part: those the blocked kernels take.
-bool delta_has_aux(int E, int M) { return reg_delta_supported(E, M) || split_delta_dims(E, M) || wide_delta_dims(E, M); }
+bool delta_has_aux(int E, int M) { return reg_delta_supported(E, M) || split_delta_dims(E, M); }
 
 namespace {
 __global__ void k_store_float(float *dst, float x) { *dst = x; }
@@ -539,37 +539,6 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
     return (int)hipGetLastError();
 }
 
-// Keys of 128 features (Performer with 64 random features, DPFP, the Delta-MLP layer's wide side:
-// language_modeling/src/utils/cuda_fast_weight_layer.py:421-423,973-975,1474-1492) with 16 value
-// columns: the one-wave kernels with a state of 8 x 1 tiles.  (8 x 2 tiles spill in the forward kernel.)
-// Wider values need no kernel of their own: the columns of the state are independent of each other, and
-// the bindings run the operator on slices of them.
-bool wide_delta_dims(int E, int M) { return E == 128 && M == 16; }
-
-int mfma_delta_wide_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
-                        float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s) {
-    const int nchunk = (L + chunk - 1) / chunk;
-    float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
-    const int spw = seq_per_wg(N * H);
-    const dim3 grid((N * H + spw - 1) / spw), block(64 * spw);
-    const size_t lds = spw * sizeof(FwdLds);
-    hipLaunchKernelGGL((k_delta_fwd_mfma<8, 1>), grid, block, lds, s, q, k, v, beta, W, out, vdiff, ckpt, aux,
-                       N * H, H, L, chunk, nchunk);
-    return (int)hipGetLastError();
-}
-
-int mfma_delta_wide_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,
-                        const float *ckpt, float *gq, float *gk, float *gv, float *gbeta, int N, int H,
-                        int L, int E, int M, int chunk, hipStream_t s) {
-    const int nchunk = (L + chunk - 1) / chunk;
-    const float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
-    const int spw = seq_per_wg(N * H);
-    const dim3 grid((N * H + spw - 1) / spw), block(64 * spw);
-    const size_t lds = spw * 4 * sizeof(LdsMat);
-    hipLaunchKernelGGL((k_delta_bwd_mfma<8, 1>), grid, block, lds, s, q, k, beta, vdiff, go, ckpt, aux, gq, gk,
-                       gv, gbeta, N * H, H, L, chunk, nchunk);
-    return (int)hipGetLastError();
-}
 
 // the state shapes the blocked sum-rule kernels are instantiated for here (those of the split delta
 // kernels); the wider ones are built in fwp_sum_wide.hip

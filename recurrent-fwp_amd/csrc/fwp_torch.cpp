@@ -27,6 +27,7 @@
 #include <stdexcept>
 #include <string>
 #include <tuple>
+#include <vector>
 
 #include "fwp_hip.h"
 
@@ -151,15 +152,54 @@ void same_device(const at::Tensor &ref, std::initializer_list<at::Tensor> others
                  ref.device().str() + "'");
 }
 
+// A run of value columns [first, last) of the delta rule's state, run as a state of `width` value columns
+// (zero padded when width > last - first).
+struct Slice {
+    int64_t first, last, width;
+};
+
+// How a state of E x M is run when no blocked kernel takes it whole (fwp_delta_kind names the kernels):
+// one slice [0, M) for the shapes that run as they are, else slices of the widths the blocked kernels
+// take for this key width, widest first, the last one padded.  The columns of the delta rule's state
+// never mix - v_old[m], the written value, W[:, m] and out[m] depend on column m and on the shared q, k,
+// beta only (fast_weight_cuda.cu:101-143) - so the operator on a slice of V and W is exact, the gradients
+// of Q, K and beta are the sums over the slices, and a padded column (v = 0, W = 0) stays zero.
+std::vector<Slice> column_plan(int64_t E, int64_t M) {
+    static const int64_t narrow[] = {64, 32, 16}, wide[] = {32, 16};      // value widths, widest first
+    const int64_t *widths = nullptr;
+    int n = 0;
+    if (E == 16 || E == 32 || E == 64) widths = narrow, n = 3;
+    else if (E == 96 || E == 128) widths = wide, n = 2;
+    std::vector<Slice> plan;
+    for (int i = 0; i < n; i++)
+        if (M == widths[i]) n = 0;
+    if (n == 0) {
+        plan.push_back({0, M, M});
+        return plan;
+    }
+    for (int64_t first = 0; first < M;) {
+        const int64_t left = M - first;
+        int64_t width = widths[n - 1];          // the narrowest, padded, when nothing fits
+        for (int i = n - 1; i >= 0; i--)
+            if (widths[i] <= left) width = widths[i];
+        const int64_t last = std::min(M, first + width);
+        plan.push_back({first, last, width});
+        first = last;
+    }
+    return plan;
+}
+
 // The delta rule's backward as a node of the autograd graph in its own right, the way PyTorch's
 // own operators are (a saved input is a SavedVariable, the result gets the node by set_history),
 // rather than through torch::autograd::Function: a forward + backward pair of this operator takes
 // about as long on the GPU as the interpreter and the autograd engine take to issue it, and the
 // generic wrapper's bookkeeping per call (context object, maps of saved data, variable infos, the
 // demangled class name per backward call) was a tenth of that.  Same saved tensors, same results.
+// A state that runs by slices of value columns keeps one saved buffer per slice.
 struct DeltaBackward : torch::autograd::Node {
     torch::autograd::SavedVariable Q_, K_, beta_;
-    at::Tensor buf_;             // v - v_old [N,H,L,M] and the checkpoints behind it (no graph of its own)
+    std::vector<Slice> plan_;
+    std::vector<at::Tensor> bufs_;      // per slice: v - v_old [N,H,L,width] and the checkpoints behind it
     int64_t M_ = 0;
     int chunk_ = 0;
     bool released_ = false;
@@ -171,7 +211,7 @@ struct DeltaBackward : torch::autograd::Node {
         Q_.reset_data();
         K_.reset_data();
         beta_.reset_data();
-        buf_.reset();
+        bufs_.clear();
         released_ = true;
     }
 
@@ -186,21 +226,39 @@ struct DeltaBackward : torch::autograd::Node {
         // saved after rows(): their views need no checks and no copies
         const fwp_view qv = view_of(Q), kv = view_of(K), bv = view_of(beta);
         same_device(Q, {grads[0]});
-        fwp_view gv_;
-        const at::Tensor go = rows(grads[0], gv_);
-        const float *vdiff = buf_.data_ptr<float>(), *ckpt = vdiff + N * H * L * M;
         // the four gradients in one allocation
         Parts parts({N * H * L * E, N * H * L * E, N * H * L * M, N * H * L}, Q.options());
         res[0] = parts.take(N, H, L, E);
         res[1] = parts.take(N, H, L, E);
         res[2] = parts.take(N, H, L, M);
         res[3] = parts.take(N, H, L, 1);
-        {
-            LaunchGuard guard(Q);
-            check(fwp_delta_bwd(qv, kv, bv, vdiff, gv_, ckpt, res[0].data_ptr<float>(), res[1].data_ptr<float>(),
-                                res[2].data_ptr<float>(), res[3].data_ptr<float>(), (int)N, (int)H, (int)L, (int)E,
-                                (int)M, chunk_, stream_of(Q)),
+        const bool whole = plan_.size() == 1;
+        at::Tensor tq, tk, tb;      // a later slice's share of the gradients of Q, K and beta
+        LaunchGuard guard(Q);
+        for (size_t i = 0; i < plan_.size(); i++) {
+            const Slice &sl = plan_[i];
+            const int64_t cols = sl.last - sl.first, pad = sl.width - cols;
+            at::Tensor go_s = whole ? grads[0] : grads[0].slice(3, sl.first, sl.last);
+            if (pad) go_s = at::constant_pad_nd(go_s, {0, pad});
+            fwp_view gv_;
+            const at::Tensor go = rows(go_s, gv_);
+            const float *vdiff = bufs_[i].data_ptr<float>(), *ckpt = vdiff + N * H * L * sl.width;
+            const at::Tensor gv_s = whole ? res[2] : at::empty({N, H, L, sl.width}, Q.options());
+            at::Tensor gq = res[0], gk = res[1], gb = res[3];
+            if (i > 0) {
+                if (!tq.defined()) tq = at::empty_like(res[0]), tk = at::empty_like(res[1]), tb = at::empty_like(res[3]);
+                gq = tq, gk = tk, gb = tb;
+            }
+            check(fwp_delta_bwd(qv, kv, bv, vdiff, gv_, ckpt, gq.data_ptr<float>(), gk.data_ptr<float>(),
+                                gv_s.data_ptr<float>(), gb.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E,
+                                (int)sl.width, chunk_, stream_of(Q)),
                   "fwp_delta_bwd");
+            if (!whole) res[2].slice(3, sl.first, sl.last).copy_(pad ? gv_s.slice(3, 0, cols) : gv_s);
+            if (i > 0) {
+                res[0].add_(tq);
+                res[1].add_(tk);
+                res[3].add_(tb);
+            }
         }
         return res;
     }
@@ -221,6 +279,10 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
         fail("W must be a contiguous fp32 [N,H,E,M] tensor");
     const bool need_grad = at::GradMode::is_enabled() && (Q_in.requires_grad() || K_in.requires_grad() ||
                                                           V_in.requires_grad() || beta_in.requires_grad());
+    // a single step that saves nothing: the single-step kernels take the widths of the slices whole
+    const bool step_whole = L == 1 && !need_grad && (M == 16 || M == 32 || M == 64 || M == 128);
+    std::vector<Slice> plan = step_whole ? std::vector<Slice>{{0, M, M}} : column_plan(E, M);
+    const bool whole = plan.size() == 1;
     std::shared_ptr<DeltaBackward> node;
     if (need_grad) {
         node = std::shared_ptr<DeltaBackward>(new DeltaBackward(), torch::autograd::deleteNode);
@@ -236,34 +298,59 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
     {
         // what follows is below autograd: copies of unaligned views and the result's permutation record nothing
         at::AutoDispatchBelowADInplaceOrView below;
-        fwp_view qv, kv, vv, bv;
-        const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), V = rows(V_in, vv), beta = rows(beta_in, bv);
+        fwp_view qv, kv, bv;
+        const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), beta = rows(beta_in, bv);
         const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
         const auto opts = Q.options();
         out = time_major ? at::empty({L, N, H, M}, opts).permute({1, 2, 0, 3}) : at::empty({N, H, L, M}, opts);
-        const fwp_out_view ov = {out.data_ptr<float>(), out.stride(0), out.stride(1), out.stride(2)};
-        at::Tensor saved;
-        float *vdiff = nullptr, *ckpt = nullptr;
-        if (need_grad) {
-            // v - v_old [N,H,L,M] and the checkpoints behind it, one allocation
-            const int64_t n_vdiff = N * H * L * M, n_ckpt = fwp_delta_ckpt_floats(N, H, L, E, M, chunk);
-            if (n_ckpt < 0) fail("invalid dimensions");
-            saved = at::empty({n_vdiff + n_ckpt}, opts);
-            vdiff = saved.data_ptr<float>();
-            ckpt = vdiff + n_vdiff;
-        }
-        {
-            LaunchGuard guard(Q);
-            check(fwp_delta_fwd_strided(qv, kv, vv, bv, W.data_ptr<float>(), ov, vdiff, ckpt, (int)N, (int)H,
-                                        (int)L, (int)E, (int)M, chunk, stream_of(Q)),
+        std::vector<at::Tensor> bufs, states;
+        LaunchGuard guard(Q);
+        for (const Slice &sl : plan) {
+            const int64_t cols = sl.last - sl.first, pad = sl.width - cols;
+            // a slice of V and of the result is passed as the strided view it is when its rows can be read
+            // and written 16 bytes at a time; a padded slice, or one of rows that are not, goes through a
+            // contiguous copy
+            at::Tensor V_s = whole ? V_in : V_in.slice(3, sl.first, sl.last), W_s = W, out_s = out;
+            if (!whole) {
+                W_s = W.slice(3, sl.first, sl.last);
+                if (pad) {
+                    V_s = at::constant_pad_nd(V_s, {0, pad});
+                    W_s = at::constant_pad_nd(W_s, {0, pad});
+                } else {
+                    W_s = W_s.contiguous();
+                }
+                out_s = (pad || M % 4) ? at::empty({N, H, L, sl.width}, opts) : out.slice(3, sl.first, sl.last);
+                states.push_back(W_s);
+            }
+            fwp_view vv;
+            const at::Tensor V = rows(V_s, vv);
+            const fwp_out_view ov = {out_s.data_ptr<float>(), out_s.stride(0), out_s.stride(1), out_s.stride(2)};
+            at::Tensor saved;
+            float *vdiff = nullptr, *ckpt = nullptr;
+            if (need_grad) {
+                // v - v_old [N,H,L,width] and the checkpoints behind it, one allocation
+                const int64_t n_vdiff = N * H * L * sl.width, n_ckpt = fwp_delta_ckpt_floats(N, H, L, E, sl.width, chunk);
+                if (n_ckpt < 0) fail("invalid dimensions");
+                saved = at::empty({n_vdiff + n_ckpt}, opts);
+                vdiff = saved.data_ptr<float>();
+                ckpt = vdiff + n_vdiff;
+                bufs.push_back(saved);
+            }
+            check(fwp_delta_fwd_strided(qv, kv, vv, bv, W_s.data_ptr<float>(), ov, vdiff, ckpt, (int)N, (int)H,
+                                        (int)L, (int)E, (int)sl.width, chunk, stream_of(Q)),
                   "fwp_delta_fwd_strided");
+            if (!whole && (pad || M % 4)) out.slice(3, sl.first, sl.last).copy_(out_s.slice(3, 0, cols));
         }
+        // the state after the last step, in place, once every slice has run: a rejected slice leaves W as it was
+        for (size_t i = 0; i < states.size(); i++)
+            W.slice(3, plan[i].first, plan[i].last).copy_(states[i].slice(3, 0, plan[i].last - plan[i].first));
         if (need_grad) {
             // inputs as they are (a SavedVariable of an input keeps the tensor itself), copies as plain tensors
             node->Q_ = torch::autograd::SavedVariable(Q, false);
             node->K_ = torch::autograd::SavedVariable(K, false);
             node->beta_ = torch::autograd::SavedVariable(beta, false);
-            node->buf_ = std::move(saved);
+            node->plan_ = std::move(plan);
+            node->bufs_ = std::move(bufs);
             node->M_ = M;
             node->chunk_ = chunk;
         }

@@ -119,7 +119,7 @@ _fwp_torch = _native()
 _operator = _fwp_torch.fast_weight_delta if _fwp_torch is not None else DeltaFastWeight.apply
 
 # Value widths the blocked kernels take for a given key width (fwp_delta_kind names the kernels).
-_FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16,)}
+_FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16, 32)}
 # Value widths the single-step kernels take (with any of the key widths above).
 _STEP_WIDTHS = (16, 32, 64, 128)
 _plans = {}
@@ -154,7 +154,16 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
     (algorithmic/fast_weight/__init__.py:96).  Key widths of 16, 32, 64, 96 and 128 with value widths
     the blocked kernels do not take whole (M = 3 D + 1 of the Delta-Delta layer, M = 128 of the
     Delta-MLP layer: cuda_fast_weight_layer.py:1474-1492,1605-1610) run on them by slices of value
-    columns, see :func:`column_plan`; every other call goes straight to the autograd function."""
+    columns, see :func:`column_plan`: inside the C++ autograd function when it is built (one graph node,
+    results written in place), by :func:`fast_weight_delta_sliced` otherwise."""
+    if _fwp_torch is not None:      # the C++ function cuts the value columns itself (csrc/fwp_torch.cpp column_plan)
+        return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
+    return fast_weight_delta_sliced(Q, K, V, beta, W, time_major)
+
+
+def fast_weight_delta_sliced(Q, K, V, beta, W, time_major=None, operator=DeltaFastWeight.apply):
+    """The operator with the slices of value columns cut here, one call of the autograd Function per
+    slice (what runs when the C++ function has not been built)."""
     try:        # the common case first: a width pair seen before (two size() calls and one dictionary lookup)
         plan = _plans[(Q.size(-1), V.size(-1))]
     except (KeyError, IndexError):
@@ -163,7 +172,7 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
             torch.is_grad_enabled() and any(t.requires_grad for t in (Q, K, V, beta))):
         plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
     if plan is None:
-        return _operator(Q, K, V, beta, W) if time_major is None else _operator(Q, K, V, beta, W, time_major)
+        return operator(Q, K, V, beta, W) if time_major is None else operator(Q, K, V, beta, W, time_major)
     if Q.dim() != 4 or V.dim() != 4:
         raise _lib.FwpError(f"expected 4-D [N,H,L,D] tensors, got {Q.dim()}-D and {V.dim()}-D")
     # the same checks on W as the whole-state path makes (there the slices would hide the caller's W from them)
@@ -180,7 +189,7 @@ def fast_weight_delta(Q, K, V, beta, W, time_major=None):
             Vs, Ws = torch.nn.functional.pad(Vs, (0, pad)), torch.nn.functional.pad(Ws, (0, pad))
         else:
             Ws = Ws.contiguous()
-        out = _operator(Q, K, Vs, beta, Ws, False)
+        out = operator(Q, K, Vs, beta, Ws, False)
         states.append(Ws)
         outs.append(out[..., :last - first] if pad else out)
     # the state after the last step, in place, once every slice has run: a rejected slice leaves W as it was

@@ -119,6 +119,10 @@ def worker(m, seed, results):
         for tm in (None, True, False):
             for views in (False, True):
                 acc += delta_case(m, 2 + rep % 2, 3, 33 + rep, 16, 16 + 16 * (rep % 2), tm, views)
+        # value widths that run by slices of value columns: 3 D + 1 (a padded last slice, rows that are not
+        # 16-byte aligned), 128 (two slices written in place), 128 keys with 64 values
+        for E, M in ((32, 97), (32, 128), (128, 64)):
+            acc += delta_case(m, 2, 2, 20 + rep, E, M, (None, True, False)[rep % 3], rep % 2 == 1)
         acc += others_case(m, 2, 2, 17 + rep, 16)
     results[seed] = acc
 

@@ -179,12 +179,13 @@ def test_value_columns_are_sliced_onto_the_blocked_kernels(fwp):
     L = fwp._lib
     lib = L.lib()
     assert fw.column_plan(32, 32) is None and fw.column_plan(96, 16) is None and fw.column_plan(128, 16) is None
+    assert fw.column_plan(128, 32) is None
     assert fw.column_plan(24, 8) is None and fw.column_plan(5, 3) is None          # no fast kernel for these keys
     assert fw.column_plan(32, 97) == [(0, 64, 64), (64, 96, 32), (96, 97, 16)]
     assert fw.column_plan(32, 128) == [(0, 64, 64), (64, 128, 64)]
-    assert fw.column_plan(128, 32) == [(0, 16, 16), (16, 32, 16)]
+    assert fw.column_plan(128, 64) == [(0, 32, 32), (32, 64, 32)]
     assert fw.column_plan(96, 48) == [(0, 32, 32), (32, 48, 16)]
-    for E, M in ((32, 97), (32, 128), (128, 32), (96, 48), (64, 100), (16, 1)):
+    for E, M in ((32, 97), (32, 128), (128, 64), (96, 48), (64, 100), (16, 1)):
         plan = fw.column_plan(E, M)
         assert plan[0][0] == 0 and plan[-1][1] == M and all(a[1] == b[0] for a, b in zip(plan, plan[1:]))
         for first, last, width in plan:

@@ -35,7 +35,8 @@ DELTA_SHAPES = [
     (1, 2, 1, 16, 16, True),      # single step (RL-style stepping)
     (2, 2, 37, 32, 97, True),     # E != M (Delta-Delta layer: M = 3D+1): slices of 64, 32 and a padded 1 value columns
     (2, 2, 70, 32, 128, True),    # Delta-MLP layer, wide side as values: two slices of 64 value columns
-    (2, 2, 70, 128, 32, True),    # ... as keys: one-wave blocked kernels with 8 key tiles, two slices of 16 value columns
+    (2, 2, 70, 128, 32, True),    # ... as keys: eight key tiles on the several-wave kernels
+    (1, 2, 50, 128, 64, True),    # ... two slices of 32 value columns
     (1, 3, 40, 128, 16, True),    # Performer with 64 random features
     (1, 2, 50, 96, 48, True),     # 96 keys take values of 16 or 32: slices of 32 and 16
     (1, 2, 40, 192, 32, True),    # DPFP with nu = 3 at D = 32 (E = 2 nu D): state in LDS
@@ -62,7 +63,7 @@ def test_delta(fwp, delta_kernels, N, H, L, E, M, w0):
 
 # every state shape E x M (multiples of 16) that the kernels with several waves per sequence are built for
 RECTANGULAR = [(16, 16), (16, 32), (16, 64), (32, 16), (32, 32), (32, 64), (64, 16), (64, 32), (64, 64),
-               (96, 16), (96, 32)]
+               (96, 16), (96, 32), (128, 16), (128, 32)]
 
 
 @pytest.mark.parametrize("E,M", RECTANGULAR)

@@ -155,3 +155,31 @@ def test_delta_lstm_same_as_python_function(fwp, N, H, L, D):
         assert torch.equal(a, b)
     with pytest.raises(fwp._lib.FwpError, match="h0 and c0"):
         fwp.fast_lstm_v4(*args, h[:, :, 0], c)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N,H,L,E,M", [(2, 2, 37, 32, 97), (2, 2, 70, 32, 128), (1, 2, 50, 128, 64), (1, 2, 1, 32, 97)])
+@pytest.mark.parametrize("time_major", [None, True])
+def test_slices_of_value_columns_cut_in_cpp_and_in_python_agree(fwp, N, H, L, E, M, time_major):
+    """Value widths that no kernel takes whole: the C++ function cuts them into slices inside one graph node,
+    the Python path (what runs without the C++ function) makes one call of the autograd Function per slice.
+    Same kernels on the same slices; the sums over the slices (gradients of Q, K, beta) may be taken in
+    another order, so those are held to 1e-6 relative to the tensor's scale instead of bit for bit."""
+    fw = importlib.import_module(fwp.__name__ + ".fast_weight")
+    q, k, v, beta, W0, go = (torch.from_numpy(a).cuda() for a in delta_inputs(9, N, H, L, E, M, dtype=np.float32, w0=True))
+    results = []
+    for f in (native(fwp).fast_weight_delta, fw.fast_weight_delta_sliced):
+        ins = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+        W = W0.clone()
+        out = f(*ins, W) if time_major is None else f(*ins, W, time_major)
+        grads = torch.autograd.grad(out, ins, go)
+        results.append([out, W, *grads])
+    names = ("out", "W", "gq", "gk", "gv", "gbeta")
+    for name, a, b in zip(names, *results):
+        assert a.shape == b.shape, name
+        if name in ("out", "W", "gv"):
+            assert torch.equal(a, b), name
+        else:
+            assert float((a - b).abs().max()) <= 1e-6 * float(b.abs().max()), name
+    a, b = results[0][0], results[1][0]      # the same memory order (a stride of an axis of one element says nothing)
+    assert [s for s, n in zip(a.stride(), a.shape) if n > 1] == [s for s, n in zip(b.stride(), b.shape) if n > 1]
