@@ -825,18 +825,20 @@ __global__ __launch_bounds__(64 * (PW + NM + 2 * WR)) void k_delta_bwd_quad(
 }  // namespace
 
 // Supported state shapes: E = 16 NE, M = 16 NM with NE in {1, 2, 4, 6}, NM in {1, 2, 4} and NE + NM <= 8,
-// and keys of 128 features (NE = 8) with NM in {1, 2}: what the backward pass's hand-over fits into the LDS.
+// keys of 128 features (NE = 8) with NM in {1, 2} and of 192 (NE = 12) with NM = 1: what the backward pass's
+// hand-over fits into the LDS.
 bool split_delta_dims(int E, int M) {
     const int ne = E / 16, nm = M / 16;
     if (E % 16 != 0 || M % 16 != 0) return false;
     if (ne == 8) return nm == 1 || nm == 2;
+    if (ne == 12) return nm == 1;
     return (ne == 1 || ne == 2 || ne == 4 || ne == 6) && (nm == 1 || nm == 2 || nm == 4) && ne + nm <= 8;
 }
 
 bool split_delta_supported(int L) { return L >= 1; }
 
 namespace {
-constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : 2; }     // (NE = 8: 56 us with two, 67 with one)
+constexpr int fwd_ring(int ne) { return ne <= 2 ? 4 : ne <= 4 ? 3 : ne <= 8 ? 2 : 1; }     // (NE = 8: 56 us with two, 67 with one)
 constexpr int bwd_ring(int ne) { return ne <= 2 ? 3 : ne <= 4 ? 2 : 1; }
 
 // The output wave is built for one or two state waves; with one (a workgroup of four waves, one per
@@ -863,7 +865,7 @@ void launch_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp
 }  // namespace
 
 // the (NE, NM) pairs of split_delta_dims
-#define FWP_SPLIT_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2) X(8, 1) X(8, 2)
+#define FWP_SPLIT_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2) X(8, 1) X(8, 2) X(12, 1)
 
 int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, fwp_out_view out,
                     float *vdiff, float *ckpt, int N, int H, int L, int E, int M, int chunk, hipStream_t s) {
@@ -904,6 +906,9 @@ int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, f
     // (104 on two, 112 with P on two waves), values of 32 in 120 us with R and G on two waves each and P on two
     // (136 on four, 141 with P on one); the one-wave kernels took 216 us for values of 16
     Q(8, 1, 4, 1, 1) Q(8, 2, 2, 2, 1)
+    // keys of 192 features, values of 16: 139 us with R and G on two waves each and P on two (143 with three and
+    // one, 275 with four and two, 302 with four and one, 725 with six and two; the LDS-state kernels take 7.9 ms)
+    Q(12, 1, 2, 2, 1)
 #undef Q
     return FWP_E_SHAPE;
 }

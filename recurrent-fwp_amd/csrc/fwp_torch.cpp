@@ -165,11 +165,12 @@ struct Slice {
 // beta only (fast_weight_cuda.cu:101-143) - so the operator on a slice of V and W is exact, the gradients
 // of Q, K and beta are the sums over the slices, and a padded column (v = 0, W = 0) stays zero.
 std::vector<Slice> column_plan(int64_t E, int64_t M) {
-    static const int64_t narrow[] = {64, 32, 16}, wide[] = {32, 16};      // value widths, widest first
+    static const int64_t narrow[] = {64, 32, 16}, wide[] = {32, 16}, widest[] = {16};      // value widths, widest first
     const int64_t *widths = nullptr;
     int n = 0;
     if (E == 16 || E == 32 || E == 64) widths = narrow, n = 3;
     else if (E == 96 || E == 128) widths = wide, n = 2;
+    else if (E == 192) widths = widest, n = 1;
     std::vector<Slice> plan;
     for (int i = 0; i < n; i++)
         if (M == widths[i]) n = 0;
@@ -189,6 +190,16 @@ std::vector<Slice> column_plan(int64_t E, int64_t M) {
     return plan;
 }
 
+// Key widths the blocked kernels take.  Another width up to the largest runs zero padded to the next one:
+// a key feature that is zero in every q and k reads and writes nothing of the state, so the padded rows of
+// the state stay zero and the results are those of the narrow state; the padded columns of grad_Q and
+// grad_K are dropped.  (The kernels that take any width keep the state in LDS and are 10 to 100 times slower.)
+int64_t padded_keys(int64_t E) {
+    for (int64_t w : {16, 32, 64, 96, 128, 192})
+        if (E <= w) return w;
+    return E;
+}
+
 // The delta rule's backward as a node of the autograd graph in its own right, the way PyTorch's
 // own operators are (a saved input is a SavedVariable, the result gets the node by set_history),
 // rather than through torch::autograd::Function: a forward + backward pair of this operator takes
@@ -200,7 +211,7 @@ struct DeltaBackward : torch::autograd::Node {
     torch::autograd::SavedVariable Q_, K_, beta_;
     std::vector<Slice> plan_;
     std::vector<at::Tensor> bufs_;      // per slice: v - v_old [N,H,L,width] and the checkpoints behind it
-    int64_t M_ = 0;
+    int64_t E_ = 0, M_ = 0;             // widths of the caller's tensors (the saved Q and K may be padded)
     int chunk_ = 0;
     bool released_ = false;
 
@@ -232,7 +243,7 @@ struct DeltaBackward : torch::autograd::Node {
         res[1] = parts.take(N, H, L, E);
         res[2] = parts.take(N, H, L, M);
         res[3] = parts.take(N, H, L, 1);
-        const bool whole = plan_.size() == 1;
+        const bool whole = plan_.size() == 1 && plan_[0].width == M;       // the state runs as it is
         at::Tensor tq, tk, tb;      // a later slice's share of the gradients of Q, K and beta
         LaunchGuard guard(Q);
         for (size_t i = 0; i < plan_.size(); i++) {
@@ -260,6 +271,10 @@ struct DeltaBackward : torch::autograd::Node {
                 res[3].add_(tb);
             }
         }
+        if (E_ != E) {      // keys that ran zero padded
+            res[0] = res[0].slice(3, 0, E_);
+            res[1] = res[1].slice(3, 0, E_);
+        }
         return res;
     }
 };
@@ -270,19 +285,21 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
     require_device(Q_in);
     same_device(Q_in, {K_in, V_in, beta_in, W});
     if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
-    const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
+    const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E_in = Q_in.size(3), M = V_in.size(3);
     if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}) ||
         beta_in.sizes() != at::IntArrayRef({N, H, L, 1}))
         fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in) +
              " beta" + shape_of(beta_in));
-    if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
+    if (W.sizes() != at::IntArrayRef({N, H, E_in, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
         fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+    if (Q_in.scalar_type() != at::kFloat || K_in.scalar_type() != at::kFloat) fail("fast-weight operators are fp32 only");
     const bool need_grad = at::GradMode::is_enabled() && (Q_in.requires_grad() || K_in.requires_grad() ||
                                                           V_in.requires_grad() || beta_in.requires_grad());
+    const int64_t E = padded_keys(E_in);
     // a single step that saves nothing: the single-step kernels take the widths of the slices whole
-    const bool step_whole = L == 1 && !need_grad && (M == 16 || M == 32 || M == 64 || M == 128);
+    const bool step_whole = L == 1 && !need_grad && E <= 128 && (M == 16 || M == 32 || M == 64 || M == 128);
     std::vector<Slice> plan = step_whole ? std::vector<Slice>{{0, M, M}} : column_plan(E, M);
-    const bool whole = plan.size() == 1;
+    const bool whole = plan.size() == 1 && plan[0].width == M;         // the state runs as it is
     std::shared_ptr<DeltaBackward> node;
     if (need_grad) {
         node = std::shared_ptr<DeltaBackward>(new DeltaBackward(), torch::autograd::deleteNode);
@@ -299,7 +316,10 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
         // what follows is below autograd: copies of unaligned views and the result's permutation record nothing
         at::AutoDispatchBelowADInplaceOrView below;
         fwp_view qv, kv, bv;
-        const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), beta = rows(beta_in, bv);
+        const bool wider = E != E_in;       // keys zero padded to a width the blocked kernels take
+        const at::Tensor Q = rows(wider ? at::constant_pad_nd(Q_in, {0, E - E_in}) : Q_in, qv),
+                         K = rows(wider ? at::constant_pad_nd(K_in, {0, E - E_in}) : K_in, kv), beta = rows(beta_in, bv);
+        const at::Tensor Wk = wider ? at::constant_pad_nd(W, {0, 0, 0, E - E_in}) : W;     // [N,H,E,M]
         const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
         const auto opts = Q.options();
         out = time_major ? at::empty({L, N, H, M}, opts).permute({1, 2, 0, 3}) : at::empty({N, H, L, M}, opts);
@@ -310,9 +330,9 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
             // a slice of V and of the result is passed as the strided view it is when its rows can be read
             // and written 16 bytes at a time; a padded slice, or one of rows that are not, goes through a
             // contiguous copy
-            at::Tensor V_s = whole ? V_in : V_in.slice(3, sl.first, sl.last), W_s = W, out_s = out;
+            at::Tensor V_s = whole ? V_in : V_in.slice(3, sl.first, sl.last), W_s = Wk, out_s = out;
             if (!whole) {
-                W_s = W.slice(3, sl.first, sl.last);
+                W_s = Wk.slice(3, sl.first, sl.last);
                 if (pad) {
                     V_s = at::constant_pad_nd(V_s, {0, pad});
                     W_s = at::constant_pad_nd(W_s, {0, pad});
@@ -343,7 +363,8 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
         }
         // the state after the last step, in place, once every slice has run: a rejected slice leaves W as it was
         for (size_t i = 0; i < states.size(); i++)
-            W.slice(3, plan[i].first, plan[i].last).copy_(states[i].slice(3, 0, plan[i].last - plan[i].first));
+            Wk.slice(3, plan[i].first, plan[i].last).copy_(states[i].slice(3, 0, plan[i].last - plan[i].first));
+        if (wider) W.copy_(Wk.slice(2, 0, E_in));
         if (need_grad) {
             // inputs as they are (a SavedVariable of an input keeps the tensor itself), copies as plain tensors
             node->Q_ = torch::autograd::SavedVariable(Q, false);
@@ -351,6 +372,7 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
             node->beta_ = torch::autograd::SavedVariable(beta, false);
             node->plan_ = std::move(plan);
             node->bufs_ = std::move(bufs);
+            node->E_ = E_in;
             node->M_ = M;
             node->chunk_ = chunk;
         }

@@ -119,8 +119,9 @@ _fwp_torch = _native()
 _operator = _fwp_torch.fast_weight_delta if _fwp_torch is not None else DeltaFastWeight.apply
 
 # Value widths the blocked kernels take for a given key width (fwp_delta_kind names the kernels).
-_FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16, 32)}
-# Value widths the single-step kernels take (with any of the key widths above).
+_FAST_WIDTHS = {16: (16, 32, 64), 32: (16, 32, 64), 64: (16, 32, 64), 96: (16, 32), 128: (16, 32),
+                192: (16,)}
+# Value widths the single-step kernels take (with any of the key widths above up to 128).
 _STEP_WIDTHS = (16, 32, 64, 128)
 _plans = {}
 
@@ -168,7 +169,7 @@ def fast_weight_delta_sliced(Q, K, V, beta, W, time_major=None, operator=DeltaFa
         plan = _plans[(Q.size(-1), V.size(-1))]
     except (KeyError, IndexError):
         plan = column_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
-    if plan is not None and Q.shape[2] == 1 and V.shape[-1] in _STEP_WIDTHS and not (
+    if plan is not None and Q.shape[2] == 1 and Q.shape[-1] <= 128 and V.shape[-1] in _STEP_WIDTHS and not (
             torch.is_grad_enabled() and any(t.requires_grad for t in (Q, K, V, beta))):
         plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
     if plan is None:

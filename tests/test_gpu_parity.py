@@ -39,7 +39,9 @@ DELTA_SHAPES = [
     (1, 2, 50, 128, 64, True),    # ... two slices of 32 value columns
     (1, 3, 40, 128, 16, True),    # Performer with 64 random features
     (1, 2, 50, 96, 48, True),     # 96 keys take values of 16 or 32: slices of 32 and 16
-    (1, 2, 40, 192, 32, True),    # DPFP with nu = 3 at D = 32 (E = 2 nu D): state in LDS
+    (1, 2, 40, 192, 32, True),    # DPFP with nu = 3 at D = 32 (E = 2 nu D): twelve key tiles, two slices of 16 value columns
+    (2, 1, 50, 160, 16, True),    # Performer with 80 random features: keys zero padded to 192
+    (1, 2, 33, 200, 24, True),    # keys beyond 192: state in LDS
     (1, 1, 33, 256, 64, True),    # the largest state the library accepts (16384 floats)
     (1, 3, 70, 24, 8, False),     # E != M, M smaller
     (1, 1, 20, 5, 3, True),       # odd sizes
@@ -63,7 +65,7 @@ def test_delta(fwp, delta_kernels, N, H, L, E, M, w0):
 
 # every state shape E x M (multiples of 16) that the kernels with several waves per sequence are built for
 RECTANGULAR = [(16, 16), (16, 32), (16, 64), (32, 16), (32, 32), (32, 64), (64, 16), (64, 32), (64, 64),
-               (96, 16), (96, 32), (128, 16), (128, 32)]
+               (96, 16), (96, 32), (128, 16), (128, 32), (192, 16)]
 
 
 @pytest.mark.parametrize("E,M", RECTANGULAR)
