@@ -579,6 +579,12 @@ def main():
     ap.add_argument("--delta-kernels", choices=["auto", "scan", "chunked", "split", "phase"], default="auto",
                     help="delta-rule kernels for D=16/32: step-by-step register-state scan or 16-step blocks "
                          "on the matrix cores (default: the library's choice)")
+    ap.add_argument("--lib", metavar="PATH",
+                    help="take the kernel-timing leg's launches from this build of libfwp_hip.so (a variant built "
+                         "for a measurement); the eager step still runs on the package's own library")
+    ap.add_argument("--kernel-leg-only", action="store_true",
+                    help="only the per-kernel leg (back-to-back launches through the C ABI): for profiles of a "
+                         "build given with --lib, whose kernels must not mix with the package's own in a trace")
     ap.add_argument("--graph", action="store_true",
                     help="time a HIP graph replay of the step recorded through the C ABI instead of eager calls")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -617,6 +623,10 @@ def main():
     import torch
     from __graft_entry__ import package
     pkg = package()
+    if args.lib:
+        # the C++ functions are linked against the package's own library and keep using it; the ctypes binding,
+        # which the per-kernel leg and the C-ABI window go through, loads the given one
+        pkg._lib.SO_PATH = os.path.abspath(args.lib)
     pkg._lib.lib()                       # fails loudly if the HIP library is not built
     pkg._lib.config(pkg._lib.CFG_DELTA_KERNELS, {"auto": 0, "scan": 1, "chunked": 2, "split": 3, "phase": 4}[args.delta_kernels])
     name = args.workload
@@ -660,6 +670,11 @@ def main():
     # than later ones, and the GPU runs a 1 ms burst after an idle spell 10 % slower than sustained work -
     # so it comes last; legs (1) and (2) are reported beside it under "kernels" and "steady".
     t_f, t_b, abi_step = kernel_times(name, pkg, arrays, 100)
+    if args.kernel_leg_only:
+        th = B * H * T
+        print(json.dumps({"workload": w["label"], "lib": pkg._lib.SO_PATH, "fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
+                          "fwd_GBps": w["fwd_bytes"](D) * th / t_f / 1e9, "bwd_GBps": w["bwd_bytes"](D) * th / t_b / 1e9}))
+        return
     steady_steps = 2000 if w["T"] * w["B"] * w["H"] * w["D"] <= 96 * 8 * 256 * 16 * 2 else 300
     steady_s, steady_issue_s = timed_steps(step, steady_steps // 10, steady_steps)
     abi_s, _ = timed_steps(abi_step, 5, 20)

@@ -1,10 +1,12 @@
 #!/bin/bash
 # Builds libfwp_hip.so for gfx950 next to the package (in-tree, so it travels with the tree).
 # Every source file is compiled to an object of its own, FWP_JOBS at a time (default 8), then linked.
+# Arguments go to every compile line; FWP_OUT names another output file (a build for a measurement, e.g.
+# FWP_OUT=/tmp/libfwp_nb.so build.sh -DFWP_TIMING_WITHOUT_BARRIERS, timed with bench.py --lib).
 set -euo pipefail
 here="$(cd "$(dirname "${BASH_SOURCE[0]}")" && pwd)"
 root="$(cd "$here/../.." && pwd)"
-out="$here/../libfwp_hip.so"
+out="${FWP_OUT:-$here/../libfwp_hip.so}"
 export HIPCC="${HIPCC:-/opt/rocm/bin/hipcc}"
 export FWP_OBJ="$(mktemp -d)"
 trap 'rm -rf "$FWP_OBJ"' EXIT

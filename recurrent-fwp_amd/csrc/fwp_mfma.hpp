@@ -78,8 +78,15 @@ struct RowBuf {
 
 // Workgroup barrier that orders the LDS hand-over only.  __syncthreads() also waits for every
 // global load and store of the wave, the prefetches of the coming blocks included.
+// FWP_TIMING_WITHOUT_BARRIERS (measurement only, never the product's build): the waves keep every instruction
+// and every LDS wait but do not wait for each other, which bounds what any hand-over protocol without a
+// workgroup barrier could gain.  Results are wrong; no address depends on data, so such a build is safe to time.
 __device__ __forceinline__ void lds_barrier() {
+#ifdef FWP_TIMING_WITHOUT_BARRIERS
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#else
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#endif
 }
 
 __device__ __forceinline__ float4 as_float4(const v4f &x) { return make_float4(x[0], x[1], x[2], x[3]); }
