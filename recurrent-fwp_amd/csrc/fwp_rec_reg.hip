@@ -121,10 +121,11 @@ __global__ __launch_bounds__(kWave * WPB) void k_rec_fwd_reg(
         const float y_m = fast_tanh(hcur);
         float y[NP], kp[NP], qp[NP];
         to_periodic<D>(y_m, y, lane);
+        // (needs no periodic operand: runs while the conversion above is on its way)
+        const float b = pinned(fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum())));
         const float qa = o.qx + group_sum<S>(dot_rot<D>(Rqc, y));
         const float ka = o.kx + group_sum<S>(dot_rot<D>(Rkc, y));
         const float va = o.vx + group_sum<S>(dot_rot<D>(Rvc, y));
-        const float b = fast_sigmoid(o.bx + across_groups<S>(rb_m * y_m, OpSum()));
         const float eq = __expf(softmax_shifted<S>(qa));
         const float ek = __expf(softmax_shifted<S>(ka));
         // The softmaxes are eq / sum(eq) and ek / sum(ek); the state is read and written with eq and
@@ -315,17 +316,20 @@ __device__ __forceinline__ void rec_bwd_pair_x(RecPairLds<D> &M, const float *__
     };
     auto compute = [&](const RecBwdOps<D> &o, int it, int tt) {
         const float g_i = dh_i + o.go_i;                      // gradient of out_t
-        float g[NP], a[NP], gqp[NP], gkp[NP], gvp[NP];
+        float g[NP], a[NP], gqp[NP], gkp[NP];
+        // Every conversion of a grouped vector into a periodic operand (ds_bpermute, 60 cycles before its
+        // result can be used) is issued as soon as its input exists, with work that does not need it behind it.
         to_periodic<D>(g_i, g, lane);
-        // gradient of q (after softmax) = W_t g, then through the softmax
-        const float dq_i = group_sum<S>(dot_rot<D>(Wr, g));
         // G' = G + q (x) g (both layouts);  r = G'^T k
         rank1_rot<D>(Gc, o.q, g_i);
         const float r_i = group_sum<S>(dot_rot<D>(Gc, o.k));
-        const float gqx_i = o.q_i * (dq_i - across_groups<S>(dq_i * o.q_i, OpSum()));
         const float gvx_i = o.b * r_i;
         const float a_i = -gvx_i;                             // gradient w.r.t. v_old
         to_periodic<D>(a_i, a, lane);
+        // gradient of q (after softmax) = W_t g, then through the softmax
+        const float dq_i = group_sum<S>(dot_rot<D>(Wr, g));
+        const float gqx_i = o.q_i * (dq_i - across_groups<S>(dq_i * o.q_i, OpSum()));
+        to_periodic<D>(gqx_i, gqp, lane);
         const float gb = across_groups<S>(r_i * o.d_i, OpSum());
         const float gbx_t = gb * o.b * (1.f - o.b);           // through the sigmoid
         rank1_rot<D>(Gr, g, o.q_i);
@@ -334,14 +338,12 @@ __device__ __forceinline__ void rec_bwd_pair_x(RecPairLds<D> &M, const float *__
         float dk_i = dot_rot<D>(Gr, o.u);                     // G' u + W_{t-1} a
         dk_i = group_sum<S>(dot_rot<D>(Wr, a, dk_i));
         rank1_rot<D>(Gr, a, o.k_i);
+        // back through the slow recurrent weights to tanh(out_{t-1}) and to out_{t-1}: the terms of q and v
+        // (grad_vx = -a, already periodic) while grad_kx is still on its way
+        float acc = dot_rot<D>(Rqr, gqp) - dot_rot<D>(Rvr, a);
         const float gkx_i = o.k_i * (dk_i - across_groups<S>(dk_i * o.k_i, OpSum()));
-        // back through the slow recurrent weights to tanh(out_{t-1}) and to out_{t-1}
-        to_periodic<D>(gqx_i, gqp, lane);
         to_periodic<D>(gkx_i, gkp, lane);
-        to_periodic<D>(gvx_i, gvp, lane);
-        float acc = dot_rot<D>(Rqr, gqp);
-        acc = dot_rot<D>(Rkr, gkp, acc);
-        acc = group_sum<S>(dot_rot<D>(Rvr, gvp, acc));
+        acc = group_sum<S>(dot_rot<D>(Rkr, gkp, acc));
         acc = fmaf(rb_i, gbx_t, acc);
         dh_i = (1.f - o.y_i * o.y_i) * acc;
         const float o_q = pinned(gqx_i), o_k = pinned(gkx_i), o_v = pinned(gvx_i);
