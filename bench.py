@@ -105,7 +105,7 @@ def make_inputs(name, w):
     from helpers import delta_inputs, lstm_inputs, rec_inputs, rnn_inputs
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
     if name.startswith("delta") or name == "sum":
-        return delta_inputs(0, B, H, T, D, D, dtype=np.float32)
+        return delta_inputs(0, B, H, T, w.get("E", D), w.get("M", D), dtype=np.float32)
     if name == "rnn":
         return rnn_inputs(0, B, H, T, D, dtype=np.float32)
     if name == "lstm":
@@ -582,6 +582,9 @@ def main():
     ap.add_argument("--lib", metavar="PATH",
                     help="take the kernel-timing leg's launches from this build of libfwp_hip.so (a variant built "
                          "for a measurement); the eager step still runs on the package's own library")
+    ap.add_argument("--dims", nargs=5, type=int, metavar=("B", "H", "T", "E", "M"),
+                    help="with --workload delta --kernel-leg-only: another batch and state shape (E key features, "
+                         "M value columns) for the per-kernel leg, e.g. 32 8 512 64 64")
     ap.add_argument("--kernel-leg-only", action="store_true",
                     help="only the per-kernel leg (back-to-back launches through the C ABI): for profiles of a "
                          "build given with --lib, whose kernels must not mix with the package's own in a trace")
@@ -637,6 +640,11 @@ def main():
         print(json.dumps(run_single_steps(args, pkg)))
         return
     w = WORKLOADS[name]
+    if args.dims:
+        if name != "delta" or not args.kernel_leg_only:
+            sys.exit("bench.py: --dims goes with --workload delta --kernel-leg-only")
+        B, H, T, E, M = args.dims
+        w = dict(w, B=B, H=H, T=T, E=E, M=M, label=f"delta-rule fast_weight fwd+bwd, B={B} H={H} T={T} E={E} M={M}, fp32")
     arrays = make_inputs(name, w)
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
     tokens = B * T
@@ -672,8 +680,10 @@ def main():
     t_f, t_b, abi_step = kernel_times(name, pkg, arrays, 100)
     if args.kernel_leg_only:
         th = B * H * T
+        E, M = w.get("E", D), w.get("M", D)      # algorithmic bytes per token-head: fwd 2E + 2M + 1, bwd 4E + 3M + 2 floats
         print(json.dumps({"workload": w["label"], "lib": pkg._lib.SO_PATH, "fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
-                          "fwd_GBps": w["fwd_bytes"](D) * th / t_f / 1e9, "bwd_GBps": w["bwd_bytes"](D) * th / t_b / 1e9}))
+                          "fwd_GBps": (2 * E + 2 * M + 1) * 4 * th / t_f / 1e9,
+                          "bwd_GBps": (4 * E + 3 * M + 2) * 4 * th / t_b / 1e9}))
         return
     steady_steps = 2000 if w["T"] * w["B"] * w["H"] * w["D"] <= 96 * 8 * 256 * 16 * 2 else 300
     steady_s, steady_issue_s = timed_steps(step, steady_steps // 10, steady_steps)
