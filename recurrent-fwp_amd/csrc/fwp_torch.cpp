@@ -8,6 +8,8 @@
 // language_modeling/src/utils/fast_lstm_v4/__init__.py:36-208).  They exist because a
 // forward + backward pair of the benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter
 // time through a Python autograd.Function, and a single inference step even less GPU time.
+// The delta rule, whose step is the shortest, is a graph node of its own (DeltaBackward) that also cuts value
+// widths no kernel takes whole into slices of columns and pads key widths; the others are autograd Functions.
 // Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
 #include <torch/csrc/autograd/functions/utils.h>
