@@ -251,7 +251,7 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
     if (L == 1 && !ckpt && g_step_kernels && dk == FWP_DELTA_AUTO && step_delta_dims(E, M) &&
         reg_view_ok(v) && aligned16(out) && aligned16(W))
         return counted(step_sum_fwd(q, k, v, W, out, N, H, E, M, (hipStream_t)stream));
-    if ((split_delta_dims(E, M) || sum_wide_dims(E, M)) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
+    if (sum_blocked_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) && aligned16(ckpt) &&
         aligned16(out)) {
         // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
         const bool blocked = in_range32(L, E, M, {q, k, v}) && (!reg_delta_supported(E, M) || delta_chunked(dk, L));
@@ -269,7 +269,7 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(grad_out) || !ckpt || !gq || !gk || !gv)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
-    if ((split_delta_dims(E, M) || sum_wide_dims(E, M)) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
+    if (sum_blocked_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
         const bool blocked =

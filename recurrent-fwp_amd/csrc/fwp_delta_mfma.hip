@@ -544,14 +544,22 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
 // kernels); the wider ones are built in fwp_sum_wide.hip
 #define FWP_SUM_SHAPES(X) X(1, 1) X(1, 2) X(1, 4) X(2, 1) X(2, 2) X(2, 4) X(4, 1) X(4, 2) X(4, 4) X(6, 1) X(6, 2)
 
+bool sum_blocked_dims(int E, int M) {
+    if (sum_wide_dims(E, M)) return true;
+#define X(ne, nm) if (E == 16 * ne && M == 16 * nm) return true;
+    FWP_SUM_SHAPES(X)
+#undef X
+    return false;
+}
+
 int mfma_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                  int L, int E, int M, int chunk, hipStream_t s) {
     if (sum_wide_dims(E, M)) return mfma_sum_wide_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, s);
 #define X(ne, nm)                                                                                          \
-    if (E == 16 * ne && M == 16 * nm) launch_sum_fwd<ne, nm>(q, k, v, W, out, ckpt, N, H, L, chunk, s);
+    if (E == 16 * ne && M == 16 * nm) return launch_sum_fwd<ne, nm>(q, k, v, W, out, ckpt, N, H, L, chunk, s);
     FWP_SUM_SHAPES(X)
 #undef X
-    return (int)hipGetLastError();
+    return FWP_E_SHAPE;
 }
 
 int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
@@ -561,10 +569,10 @@ int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *c
         return mfma_sum_wide_bwd(q, k, v, go, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk, s);
 #define X(ne, nm)                                                                                          \
     if (E == 16 * ne && M == 16 * nm)                                                                      \
-        launch_sum_bwd<ne, nm>(q, k, v, go, ckpt, W_init, gq, gk, gv, N, H, L, chunk, s);
+        return launch_sum_bwd<ne, nm>(q, k, v, go, ckpt, W_init, gq, gk, gv, N, H, L, chunk, s);
     FWP_SUM_SHAPES(X)
 #undef X
-    return (int)hipGetLastError();
+    return FWP_E_SHAPE;
 }
 
 }  // namespace fwp

@@ -872,11 +872,13 @@ int split_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W,
     const int nchunk = (L + chunk - 1) / chunk;
     float *aux = delta_aux_of(ckpt, N, H, L, E, M, chunk);
 #define X(ne, nm)                                                                                        \
-    if (E == 16 * ne && M == 16 * nm)                                                                    \
-        launch_fwd<ne, nm>(q, k, v, beta, W, out, vdiff, ckpt, aux, N * H, H, L, chunk, nchunk, s);
+    if (E == 16 * ne && M == 16 * nm) {                                                                  \
+        launch_fwd<ne, nm>(q, k, v, beta, W, out, vdiff, ckpt, aux, N * H, H, L, chunk, nchunk, s);      \
+        return (int)hipGetLastError();                                                                   \
+    }
     FWP_SPLIT_SHAPES(X)
 #undef X
-    return (int)hipGetLastError();
+    return FWP_E_SHAPE;
 }
 
 int split_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fwp_view go,

@@ -281,20 +281,22 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_sum_bwd_mfma(fwp_view q, fwp
 
 
 template <int NE, int NM>
-void launch_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H, int L,
+int launch_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H, int L,
                     int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, spw = seq_per_wg(N * H);
     hipLaunchKernelGGL((k_sum_fwd_mfma<NE, NM>), dim3((N * H + spw - 1) / spw), dim3(64 * spw), 0, s, q, k, v, W,
                        out, ckpt, N * H, H, L, chunk, nchunk);
+    return (int)hipGetLastError();
 }
 
 template <int NE, int NM>
-void launch_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt, const float *W_init,
+int launch_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt, const float *W_init,
                     float *gq, float *gk, float *gv, int N, int H, int L, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, spw = seq_per_wg(N * H);
     hipLaunchKernelGGL((k_sum_bwd_mfma<NE, NM>), dim3((N * H + spw - 1) / spw), dim3(64 * spw),
                        spw * 4 * sizeof(LdsMat), s, q, k, v, go, ckpt, W_init, gq, gk, gv, N * H, H, L, chunk,
                        nchunk);
+    return (int)hipGetLastError();
 }
 
 }  // namespace

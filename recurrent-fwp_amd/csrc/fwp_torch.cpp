@@ -182,8 +182,13 @@ std::vector<Slice> column_plan(int64_t E, int64_t M) {
     }
     for (int64_t first = 0; first < M;) {
         const int64_t left = M - first;
-        int64_t width = widths[n - 1];          // the narrowest, padded, when nothing fits
-        for (int i = n - 1; i >= 0; i--)
+        // the narrowest width that holds all that is left when at most a third of it is padding (one launch
+        // instead of two), else the widest that fits, else the narrowest, padded
+        int64_t width = widths[n - 1];
+        bool holds = false;
+        for (int i = n - 1; i >= 0 && !holds; i--)
+            if (widths[i] >= left && 2 * (widths[i] - left) <= left) width = widths[i], holds = true;
+        for (int i = n - 1; i >= 0 && !holds; i--)
             if (widths[i] <= left) width = widths[i];
         const int64_t last = std::min(M, first + width);
         plan.push_back({first, last, width});

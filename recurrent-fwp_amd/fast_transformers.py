@@ -4,7 +4,7 @@ language-modelling and RL copies are identical)."""
 import torch
 
 from . import _lib
-from .fast_weight import _fwp_torch, _nchunk
+from .fast_weight import _fwp_torch, _nchunk, pick_width
 
 
 class FastWeightSum(torch.autograd.Function):
@@ -85,4 +85,77 @@ def _native_sum(Q, K, V, W):
     return _fwp_torch.fast_weight_sum(Q, K, V, W, mode == "exact")
 
 
-fast_weight_sum = _native_sum if _fwp_torch is not None else FastWeightSum.apply
+_operator = _native_sum if _fwp_torch is not None else FastWeightSum.apply
+
+# Value widths the blocked kernels take for a given key width, and those the single-step kernels take.
+_FAST_WIDTHS = {16: (16, 32, 64, 128), 32: (16, 32, 64, 128), 64: (16, 32, 64), 96: (16, 32), 128: (16, 32),
+                192: (16,)}
+_STEP_WIDTHS = (16, 32, 64, 128)
+_plans = {}
+
+
+def sum_plan(E, M):
+    """How a state of E x M is run when no fast kernel takes it whole: ``None`` (as it is), or
+    ``(keys, slices)``: the keys zero padded to ``keys`` features and value columns [first, last) run as a
+    state of keys x width for every ``(first, last, width)`` of ``slices``.  Both are exact for the sum rule:
+    a column of ``W += k (x) v`` and of ``out = W^T q`` depends on that column of V and W only
+    (causal_product_cuda.cu:15-96), the gradients of Q and K are sums over the columns, and a key feature
+    that is zero in q and k adds nothing to any of them."""
+    key = (E, M)
+    if key not in _plans:
+        keys = next((w for w in sorted(_FAST_WIDTHS) if w >= E), None)
+        plan = None
+        if keys is not None and not (keys == E and M in _FAST_WIDTHS[keys]):
+            widths, slices, first = _FAST_WIDTHS[keys], [], 0
+            while first < M:
+                left = M - first
+                width = pick_width(widths, left)
+                last = min(M, first + width)
+                slices.append((first, last, width))
+                first = last
+            plan = (keys, slices)
+        _plans[key] = plan
+    return _plans[key]
+
+
+def fast_weight_sum(Q, K, V, W):
+    """``out = fast_weight_sum(Q, K, V, W)``, the reference's operator
+    (algorithmic/fast_transformers/__init__.py:84).  State shapes no blocked kernel takes whole (keys of
+    192 features with values of 32, values of 128 with keys of 64, widths that are not multiples of 16)
+    run on them by slices of value columns with zero padded keys, see :func:`sum_plan`."""
+    try:        # the common case first: a width pair seen before
+        plan = _plans[(Q.size(-1), V.size(-1))]
+    except (KeyError, IndexError):
+        plan = sum_plan(Q.shape[-1], V.shape[-1]) if Q.dim() == 4 and V.dim() == 4 else None
+    if plan is not None and Q.shape[2] == 1 and Q.shape[-1] in _FAST_WIDTHS and Q.shape[-1] <= 128 and \
+            V.shape[-1] in _STEP_WIDTHS and not (torch.is_grad_enabled() and any(t.requires_grad for t in (Q, K, V))):
+        plan = None     # a single step that saves nothing: the single-step kernels take these widths whole
+    if plan is None:
+        return _operator(Q, K, V, W)
+    N, H, L, E = Q.shape
+    M = V.shape[-1]
+    # the checks the whole-state path makes on the caller's W, which the slices would hide from it
+    if K.shape != Q.shape or V.shape[:3] != Q.shape[:3]:
+        raise _lib.FwpError(f"shape mismatch: Q{tuple(Q.shape)} K{tuple(K.shape)} V{tuple(V.shape)}")
+    if W.shape != (N, H, E, M) or not W.is_contiguous() or W.dtype != torch.float32:
+        raise _lib.FwpError("W must be a contiguous fp32 [N,H,E,M] tensor")
+    _lib.same_device(Q, K, V, W)
+    keys, slices = plan
+    pad = torch.nn.functional.pad
+    if keys > E:
+        Q, K = pad(Q, (0, keys - E)), pad(K, (0, keys - E))
+    outs, states = [], []
+    for first, last, width in slices:
+        extra = width - (last - first)
+        Vs = V[..., first:last]
+        Ws = pad(W.detach()[..., first:last], (0, extra, 0, keys - E))      # a copy, contiguous
+        if extra:
+            Vs = pad(Vs, (0, extra))
+        out = _operator(Q, K, Vs, Ws)
+        states.append(Ws)
+        outs.append(out[..., :last - first] if extra else out)
+    # the state after the last step, in place, once every slice has run: a rejected slice leaves W as it was
+    with torch.no_grad():
+        for (first, last, _), Ws in zip(slices, states):
+            W[..., first:last] = Ws[:, :, :E, :last - first]
+    return torch.cat(outs, -1) if len(outs) > 1 else outs[0]

@@ -126,6 +126,17 @@ _STEP_WIDTHS = (16, 32, 64, 128)
 _plans = {}
 
 
+def pick_width(widths, left):
+    """The width of the next slice when ``left`` value columns remain: the narrowest that holds them all when
+    at most a third of it is padding (one launch instead of two), else the widest that fits, else the
+    narrowest, padded."""
+    holds = [w for w in widths if w >= left and 2 * (w - left) <= left]
+    if holds:
+        return min(holds)
+    fits = [w for w in widths if w <= left]
+    return max(fits) if fits else min(widths)
+
+
 def column_plan(E, M):
     """How a state of E x M is run when no fast kernel takes it whole: ``None`` (run it as it is) or a
     list of ``(first, last, width)``: value columns [first, last) run as a state of E x width, zero
@@ -141,8 +152,7 @@ def column_plan(E, M):
             plan, first = [], 0
             while first < M:
                 left = M - first
-                fits = [w for w in widths if w <= left]
-                width = max(fits) if fits else min(w for w in widths if w >= left)
+                width = pick_width(widths, left)
                 last = min(M, first + width)
                 plan.append((first, last, width))
                 first = last

@@ -185,7 +185,17 @@ def test_value_columns_are_sliced_onto_the_blocked_kernels(fwp):
     assert fw.column_plan(32, 128) == [(0, 64, 64), (64, 128, 64)]
     assert fw.column_plan(128, 64) == [(0, 32, 32), (32, 64, 32)]
     assert fw.column_plan(96, 48) == [(0, 32, 32), (32, 48, 16)]
-    for E, M in ((32, 97), (32, 128), (128, 64), (96, 48), (64, 100), (16, 1)):
+    # one padded launch where at most a third of it is padding: 3 D + 1 at D = 16, and 24 or 48 columns
+    assert fw.column_plan(16, 49) == [(0, 49, 64)] and fw.column_plan(32, 24) == [(0, 24, 32)]
+    assert fw.column_plan(64, 48) == [(0, 48, 64)] and fw.column_plan(64, 40) == [(0, 32, 32), (32, 40, 16)]
+    assert fw.column_plan(192, 24) == [(0, 16, 16), (16, 24, 16)]
+    # the sum rule: its own table of widths, keys padded as well
+    ft = fwp.fast_transformers
+    assert ft.sum_plan(32, 128) is None and ft.sum_plan(192, 16) is None and ft.sum_plan(200, 16) is None
+    assert ft.sum_plan(192, 32) == (192, [(0, 16, 16), (16, 32, 16)])
+    assert ft.sum_plan(64, 128) == (64, [(0, 64, 64), (64, 128, 64)])
+    assert ft.sum_plan(48, 24) == (64, [(0, 24, 32)]) and ft.sum_plan(11, 4) == (16, [(0, 4, 16)])
+    for E, M in ((32, 97), (32, 128), (128, 64), (96, 48), (64, 100), (16, 1), (16, 49), (64, 48)):
         plan = fw.column_plan(E, M)
         assert plan[0][0] == 0 and plan[-1][1] == M and all(a[1] == b[0] for a, b in zip(plan, plan[1:]))
         for first, last, width in plan:

@@ -98,7 +98,7 @@ def off_by_one_float(t):
 
 
 @pytest.mark.parametrize("B,H,T,E,M", [(96, 8, 100, 32, 128), (96, 8, 100, 128, 32), (64, 4, 130, 16, 128),
-                                       (33, 9, 47, 128, 16)])
+                                       (33, 9, 47, 128, 16), (40, 8, 100, 192, 16)])
 def test_sum_widest_states_blocked_against_generic_kernels(fwp, B, H, T, E, M):
     """The fast-net layers' memories (d_head x 4 d_head and back) at hundreds of sequences: the
     blocked kernels against the generic ones, which a misaligned q selects.  Tolerance as for the
