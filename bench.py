@@ -683,8 +683,10 @@ def main():
         fwd_bytes, bwd_bytes = w["fwd_bytes"](D), w["bwd_bytes"](D)
         if args.dims:       # the delta rule at E x M, per token-head: forward 2E + 2M + 1 floats, backward 4E + 3M + 2
             fwd_bytes, bwd_bytes = (2 * w["E"] + 2 * w["M"] + 1) * 4, (4 * w["E"] + 3 * w["M"] + 2) * 4
+        t_step, _ = timed_steps(abi_step, 20, 200)      # state reset + forward + backward, through the C ABI
         print(json.dumps({"workload": w["label"], "lib": pkg._lib.SO_PATH, "fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
-                          "fwd_GBps": fwd_bytes * th / t_f / 1e9, "bwd_GBps": bwd_bytes * th / t_b / 1e9}))
+                          "fwd_GBps": fwd_bytes * th / t_f / 1e9, "bwd_GBps": bwd_bytes * th / t_b / 1e9,
+                          "c_abi_step_us": t_step * 1e6}))
         return
     steady_steps = 2000 if w["T"] * w["B"] * w["H"] * w["D"] <= 96 * 8 * 256 * 16 * 2 else 300
     steady_s, steady_issue_s = timed_steps(step, steady_steps // 10, steady_steps)

@@ -45,11 +45,13 @@ bool delta_chunked(int dk, int L) {
 
 // Several waves per sequence or one, measured on MI355X (1024 SIMDs) as the time of a training step
 // (what runs before a kernel changes where its waves land, so kernels timed alone mislead): the split
-// kernels up to 1024 sequences, one wave per sequence beyond.  D = 16, step of forward + backward at
+// kernels up to 1024 sequences, one wave per sequence beyond, at D = 16: step of forward + backward at
 // 512 / 768 / 1024 sequences of 256 steps: 41 / 44 / 49 us split, 44 / 47 / 50 us one wave; at
-// 1280 / 1536 / 2048 sequences: 74 / 80 / 124 us split, 71 / 74 / 97 us one wave.  D = 32, 256 sequences
-// of 1024 steps: 55 + 106 us split, 117 + 233 us one wave; 1280 sequences of 256 steps: 218 us split,
-// 203 us one wave.
+// 1280 / 1536 / 2048 sequences: 74 / 80 / 124 us split, 71 / 74 / 97 us one wave.  D = 32: the split
+// kernels up to 512 sequences, which is what the chip holds of them at once (two workgroups per CU);
+// 512 / 576 / 768 / 1024 sequences of 256 steps: 79 / 109 / 117 / 154 us split, 95 / 96 / 98 / 124 us
+// one wave; of 1024 steps: 279 / 396 / 431 / 543 us split, 386 / 394 / 411 / 447 us one wave; of 64 steps
+// 33 / - / 49 / - us split, 35 / - / 36 / - us one wave.
 // The kernels that read through buffer resources address a sequence with 32-bit byte offsets, and
 // may ask for rows up to two blocks past its end (which must not wrap around to rows that exist).
 bool in_range32(int L, int E, int M, std::initializer_list<fwp_view> views) {
@@ -69,7 +71,7 @@ bool delta_split(int dk, int N, int H, int L, int E, int M, std::initializer_lis
     if (dk != FWP_DELTA_AUTO) return !reg_delta_supported(E, M);
     if (!reg_delta_supported(E, M)) return true;
     if (L < 32) return false;
-    return (int64_t)N * H <= 1024;
+    return (int64_t)N * H <= (E == 32 ? 512 : 1024);
 }
 
 // Of the calls the several-wave kernels take (same views, same range of offsets), those that go to the

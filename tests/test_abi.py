@@ -96,6 +96,12 @@ def test_delta_dispatch_keeps_32_bit_kernels_off_views_beyond_their_range(fwp):
             L.config(L.CFG_DELTA_KERNELS, L.DELTA_AUTO)
     # short sequences stay on the scan kernels, shapes without a fast kernel on the LDS kernels
     assert lib.fwp_delta_kind(0, small, small, small, beta, 4, 8, 8, D, D) == L.KIND_SCAN
+    # several waves per sequence while the chip holds every sequence's workgroup at once, one wave beyond
+    for D_, most in ((16, 1024), (32, 512)):
+        rows = L.View(4096, 8 * 256 * D_, 256 * D_, D_)
+        for backward in (0, 1):
+            assert lib.fwp_delta_kind(backward, rows, rows, rows, beta, most // 8, 8, 256, D_, D_) == L.KIND_SPLIT
+            assert lib.fwp_delta_kind(backward, rows, rows, rows, beta, most // 8 + 1, 8, 256, D_, D_) == L.KIND_CHUNKED
     odd = L.View(4096, 8 * 64 * 24, 64 * 24, 24)
     assert lib.fwp_delta_kind(1, odd, odd, odd, beta, 4, 8, 64, 24, 24) == L.KIND_LDS
     assert lib.fwp_delta_kind(0, small, small, small, beta, 0, 8, 64, D, D) == -2

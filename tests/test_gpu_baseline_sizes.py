@@ -63,7 +63,8 @@ def f64(arrays):
     return [np.asarray(a, np.float64) for a in arrays]
 
 
-# The last two lie beyond 1024 sequences, where the default dispatch is the one-wave blocked kernels.
+# The last two lie beyond 1024 (D = 16) and 512 (D = 32) sequences, where the default dispatch is the one-wave
+# blocked kernels.
 @pytest.mark.parametrize("case,shape", [("delta_B96H8T256D16", (96, 8, 256, 16)),
                                         ("delta_B32H8T1024D32", (32, 8, 1024, 32)),
                                         ("delta_B160H8T256D16", (160, 8, 256, 16)),
@@ -73,7 +74,7 @@ def test_delta_rule_whole_batch_against_the_oracle(fwp, case, shape):
     L_ = fwp._lib
     view = L_.View(4096, H * T * D, T * D, D)
     kind = L_.lib().fwp_delta_kind(0, view, view, view, L_.View(4096, H * T, T, 1), N, H, T, D, D)
-    assert kind == (L_.KIND_SPLIT if N * H <= 1024 else L_.KIND_CHUNKED), (case, kind)
+    assert kind == (L_.KIND_SPLIT if N * H <= (1024 if D == 16 else 512) else L_.KIND_CHUNKED), (case, kind)
     q, k, v, beta, W0, go = delta_inputs(2, N, H, T, D, D, dtype=np.float32)
     ts = [dev(a, True) for a in (q, k, v, beta)]
     W = dev(W0)
