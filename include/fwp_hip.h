@@ -127,8 +127,8 @@ int fwp_check_device(void);
  * Number of floats the delta rule's `ckpt` buffer must hold (-1 for invalid dimensions):
  * the N*H*nchunk*E*M checkpointed states and, for the state shapes the matrix-core kernels take
  * (E in {16,32,64,96} with M in {16,32,64} and E/16 + M/16 <= 8; E = 128 with M in {16,32}; E = 192
- * with M = 16), a header and one 16x16 matrix per 16
- * steps that the blocked forward kernel leaves for the blocked backward.
+ * with M = 16), a header and room for one 16x16 matrix per 16
+ * steps that the blocked forward kernel leaves for the blocked backward (the header says whether it did).
  * No counterpart in the reference.
  */
 long long fwp_delta_ckpt_floats(int N, int H, int L, int E, int M, int chunk);

@@ -61,8 +61,8 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
                                                        fwp_out_view out,
                                                        float *__restrict__ vdiff,
                                                        float *__restrict__ ckpt,
-                                                       float *__restrict__ aux, int nseq, int H,
-                                                       int L, int chunk, int nchunk) {
+                                                       float *__restrict__ aux, int keep_T, int nseq,
+                                                       int H, int L, int chunk, int nchunk) {
     constexpr int E = 16 * NE, M = 16 * NM;
     extern __shared__ __align__(16) unsigned char dyn_lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -79,8 +79,10 @@ __global__ __launch_bounds__(64 * kSeqPerWg) void k_delta_fwd_mfma(fwp_view q, f
     const int n = (int)(seq / H), h = (int)(seq % H);
     const int nblk = (L + kBlk - 1) / kBlk, ngrp = (nblk + kGrp - 1) / kGrp;
     // aux (with ckpt): a header whose first float says that the per-block matrices T = (I + A)^-1
-    // follow, row-major, [sequence][block][16][16]; backward then does not invert.
-    if (aux && seq == 0 && lane == 0) aux[0] = 1.f;
+    // follow, row-major, [sequence][block][16][16]; backward then does not invert.  Without keep_T the header
+    // says that none follow, and the stores of T are dropped (a buffer of no bytes).
+    if (aux && seq == 0 && lane == 0) aux[0] = keep_T ? 1.f : 0.f;
+    if (!keep_T) aux = nullptr;
     const RowBuf qb(row(q, n, h, 0), (uint32_t)(((L - 1) * q.sL + E) * 4)),
         kb(row(k, n, h, 0), (uint32_t)(((L - 1) * k.sL + E) * 4)),
         vb(row(v, n, h, 0), (uint32_t)(((L - 1) * v.sL + M) * 4)),
@@ -511,14 +513,21 @@ int mfma_delta_fwd(fwp_view q, fwp_view k, fwp_view v, fwp_view beta, float *W, 
     // whole workgroups of four: in a training step (after the backward kernels of the step before) 47.3 us
     // per step at 768 sequences against 48.2 us with three waves per workgroup and 50.3 us with one
     const int spw = N * H >= kSeqPerWg ? kSeqPerWg : N * H;
+    // The inverses T (64 bytes per step and sequence, a seventh of the forward pass's traffic) are left for the
+    // backward pass while the launch is bound by the latency of a sequence's chain; from 2048 sequences on both
+    // kernels are bound by HBM and the backward pass inverts again at no cost in time.  Forward + backward
+    // with / without them, 256 steps: D = 16, 1280 / 2048 / 3072 / 12288 sequences 74 / 99 / 150 / 595 us with,
+    // 83 / 99 / 142 / 544 us without (2048 sequences of 1024 steps: 411 / 377 us); D = 32, 1536 / 2048 / 4096
+    // sequences 206 / 230 / 450 us with, 202 / 221 / 434 us without.
+    const int keep_T = (int64_t)N * H < 2048;
     const dim3 grid((N * H + spw - 1) / spw), block(64 * spw);
     const size_t lds = spw * sizeof(FwdLds);
     if (D == 16)
         hipLaunchKernelGGL((k_delta_fwd_mfma<1, 1>), grid, block, lds, s, q, k, v, beta, W, out, vdiff, ckpt, aux,
-                           N * H, H, L, chunk, nchunk);
+                           keep_T, N * H, H, L, chunk, nchunk);
     else
         hipLaunchKernelGGL((k_delta_fwd_mfma<2, 2>), grid, block, lds, s, q, k, v, beta, W, out, vdiff, ckpt, aux,
-                           N * H, H, L, chunk, nchunk);
+                           keep_T, N * H, H, L, chunk, nchunk);
     return (int)hipGetLastError();
 }
 

@@ -68,7 +68,10 @@ def f64(arrays):
 @pytest.mark.parametrize("case,shape", [("delta_B96H8T256D16", (96, 8, 256, 16)),
                                         ("delta_B32H8T1024D32", (32, 8, 1024, 32)),
                                         ("delta_B160H8T256D16", (160, 8, 256, 16)),
-                                        ("delta_B48H32T256D32", (48, 32, 256, 32))])
+                                        ("delta_B48H32T256D32", (48, 32, 256, 32)),
+                                        # from 2048 sequences on forward leaves no inverses and backward inverts
+                                        ("delta_B256H8T80D16", (256, 8, 80, 16)),
+                                        ("delta_B96H32T72D32", (96, 32, 72, 32))])
 def test_delta_rule_whole_batch_against_the_oracle(fwp, case, shape):
     N, H, T, D = shape
     L_ = fwp._lib
