@@ -4,7 +4,7 @@ import ctypes
 
 import torch
 
-from . import _lib
+from . import _lib, _padding
 from .fast_weight import _fwp_torch, _nchunk
 
 
@@ -97,4 +97,40 @@ class FastLSTMv4(torch.autograd.Function):
 
 
 # the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
-fast_lstm_v4 = _fwp_torch.fast_lstm_v4 if _fwp_torch is not None else FastLSTMv4.apply
+_operator = _fwp_torch.fast_lstm_v4 if _fwp_torch is not None else FastLSTMv4.apply
+
+
+def fast_lstm_v4(Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0):
+    """``rnn_out, cell_out = fast_lstm_v4(Zi, Ki, Vi, bi, Wi, Zu, ..., Wo, h0, c0)``, the reference's
+    operator (language_modeling/src/utils/fast_lstm_v4/__init__.py:208).  A head size below 32 that is
+    not 16 runs on the kernels of the next of the two.  The padded entries of h must be -BIG for the
+    softmax to give them exactly zero (see _padding.py): h0 is padded with -BIG, Zi and Zo with +BIG (both
+    gates exactly one) and Zu with -BIG, so that every later c = i u + (1 - i) c and h = o c of a padded
+    entry is -BIG again; K, V, W and c0 are padded with zeros.  The states come back in W, h0, c0."""
+    args = (Zi, Ki, Vi, bi, Wi, Zu, Ku, Vu, bu, Wu, Zo, Ko, Vo, bo, Wo, h0, c0)
+    D = Vi.shape[-1] if Vi.dim() == 4 else 0
+    width = _padding.padded_width(D)
+    if width is None or Zi.dim() != 4:
+        return _operator(*args)
+    N, H, L, _ = Zi.shape
+    gates = ((Zi, Ki, Vi, bi, Wi), (Zu, Ku, Vu, bu, Wu), (Zo, Ko, Vo, bo, Wo))
+    for Z, K, V, b, W in gates:
+        if not (Z.shape == K.shape == V.shape == (N, H, L, D) and b.shape == (N, H, L, 1)
+                and _padding.state_ok(W, (N, H, D, D))):
+            return _operator(*args)      # raises what the operator raises for these
+    if not (_padding.state_ok(h0, (N, H, 1, D)) and _padding.state_ok(c0, (N, H, 1, D))):
+        return _operator(*args)
+    n = width - D
+    padded, states = [], []
+    for (Z, K, V, b, W), z_fill in zip(gates, (_padding.BIG, -_padding.BIG, _padding.BIG)):
+        Wp = _padding.square(W.detach(), n)
+        states.append(Wp)
+        padded += [_padding.last(Z, n, z_fill), _padding.last(K, n), _padding.last(V, n), b, Wp]
+    hp, cp = _padding.last(h0.detach(), n, -_padding.BIG), _padding.last(c0.detach(), n)
+    out, cell = _operator(*padded, hp, cp)
+    with torch.no_grad():
+        for (_, _, _, _, W), Wp in zip(gates, states):
+            W.copy_(Wp[:, :, :D, :D])
+        h0.copy_(hp[..., :D])
+        c0.copy_(cp[..., :D])
+    return out[..., :D], cell[..., :D]

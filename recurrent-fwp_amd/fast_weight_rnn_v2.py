@@ -2,7 +2,7 @@
 ``fast_weight_rnn_v2`` package (algorithmic/fast_weight_rnn_v2/__init__.py:29-121)."""
 import torch
 
-from . import _lib
+from . import _lib, _padding
 from .fast_weight import _fwp_torch, _nchunk
 
 
@@ -79,4 +79,26 @@ class FastRNNv2(torch.autograd.Function):
 
 
 # the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
-fast_rnn_v2 = _fwp_torch.fast_rnn_v2 if _fwp_torch is not None else FastRNNv2.apply
+_operator = _fwp_torch.fast_rnn_v2 if _fwp_torch is not None else FastRNNv2.apply
+
+
+def fast_rnn_v2(Z, K, V, W, beta, h0):
+    """``rnn_out = fast_rnn_v2(Z, K, V, W, beta, h0)``, the reference's operator
+    (algorithmic/fast_weight_rnn_v2/__init__.py:121).  A head size below 32 that is not 16 runs on the
+    kernels of the next of the two: K, V and W zero padded, Z and h0 padded with -BIG, so that the padded
+    entries of softmax(h) are exactly zero (see _padding.py); W and h0 take the states back."""
+    D = V.shape[-1] if V.dim() == 4 else 0
+    width = _padding.padded_width(D)
+    if width is None or Z.dim() != 4:
+        return _operator(Z, K, V, W, beta, h0)
+    N, H, L, _ = Z.shape
+    if not (Z.shape == K.shape == V.shape and beta.shape == (N, H, L, 1) and _padding.state_ok(W, (N, H, D, D))
+            and _padding.state_ok(h0, (N, H, 1, D))):
+        return _operator(Z, K, V, W, beta, h0)      # raises what the operator raises for these
+    n = width - D
+    Wp, hp = _padding.square(W.detach(), n), _padding.last(h0.detach(), n, -_padding.BIG)
+    out = _operator(_padding.last(Z, n, -_padding.BIG), _padding.last(K, n), _padding.last(V, n), Wp, beta, hp)
+    with torch.no_grad():
+        W.copy_(Wp[:, :, :D, :D])
+        h0.copy_(hp[..., :D])
+    return out[..., :D]

@@ -2,7 +2,7 @@
 ``rec_update_fwm_tanh`` package (algorithmic/rec_update_fwm_tanh/__init__.py:31-139)."""
 import torch
 
-from . import _lib
+from . import _lib, _padding
 from .fast_weight import _fwp_torch, _nchunk
 
 
@@ -94,4 +94,30 @@ class FastWeightRecUpdateTanh(torch.autograd.Function):
 
 
 # the same operator as a C++ autograd function (csrc/fwp_torch.cpp) when that has been built
-rec_update_fwm_tanh = _fwp_torch.rec_update_fwm_tanh if _fwp_torch is not None else FastWeightRecUpdateTanh.apply
+_operator = _fwp_torch.rec_update_fwm_tanh if _fwp_torch is not None else FastWeightRecUpdateTanh.apply
+
+
+def rec_update_fwm_tanh(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0):
+    """``out = rec_update_fwm_tanh(qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0)``, the reference's operator
+    (algorithmic/rec_update_fwm_tanh/__init__.py:139).  A head size below 32 that is not 16 runs on the
+    kernels of the next of the two: qx and kx padded with -BIG, so that the padded entries of the two
+    softmaxes are exactly zero (see _padding.py), everything else with zeros; W and h0 take the states back."""
+    args = (qx, kx, vx, bx, R_q, R_k, R_v, r_b, W, h0)
+    D = vx.shape[-1] if vx.dim() == 4 else 0
+    width = _padding.padded_width(D)
+    if width is None or qx.dim() != 4:
+        return _operator(*args)
+    N, H, L, _ = qx.shape
+    if not (qx.shape == kx.shape == vx.shape == (N, H, L, D) and bx.shape == (N, H, L, 1)
+            and R_q.shape == R_k.shape == R_v.shape == (1, H, D, D) and r_b.shape == (1, H, 1, D)
+            and _padding.state_ok(W, (N, H, D, D)) and _padding.state_ok(h0, (N, H, 1, D))):
+        return _operator(*args)      # raises what the operator raises for these
+    n = width - D
+    Wp, hp = _padding.square(W.detach(), n), _padding.last(h0.detach(), n)
+    out = _operator(_padding.last(qx, n, -_padding.BIG), _padding.last(kx, n, -_padding.BIG), _padding.last(vx, n),
+                    bx, _padding.square(R_q, n), _padding.square(R_k, n), _padding.square(R_v, n),
+                    _padding.last(r_b, n), Wp, hp)
+    with torch.no_grad():
+        W.copy_(Wp[:, :, :D, :D])
+        h0.copy_(hp[..., :D])
+    return out[..., :D]

@@ -42,6 +42,8 @@ SHAPES = [
     (1, 2, 1, 32, True),       # single step
     (2, 2, 70, 8, True),
     (1, 1, 19, 5, True),
+    (2, 2, 40, 24, True),      # 18, 8, 5 and 24 run padded to 16 or 32
+    (1, 2, 20, 40, True),      # wider than any register kernel: the kernels that keep the state in LDS
 ]
 
 

@@ -191,7 +191,8 @@ def test_delta_no_grad_path(fwp, delta_kernels, E, M, L):
 
 RNN_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 64, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
               (3, 5, 40, 32, True), (1, 3, 100, 16, True),
-              (2, 3, 77, 8, True), (1, 1, 19, 5, True)]
+              (2, 3, 77, 8, True), (1, 1, 19, 5, True),
+              (2, 2, 50, 24, True), (1, 2, 1, 18, True)]     # head sizes that run padded to 16 or 32: these four
 
 
 @pytest.mark.parametrize("N,H,L,D,w0", RNN_SHAPES)
@@ -211,7 +212,8 @@ def test_rnn(fwp, N, H, L, D, w0):
 
 REC_SHAPES = [(2, 2, 64, 16, False), (3, 5, 11, 32, False), (2, 2, 256, 32, True), (1, 2, 1, 32, True),
               (1, 3, 100, 16, True),
-              (2, 3, 77, 8, True), (1, 1, 19, 5, True), (1, 2, 30, 64, False)]
+              (2, 3, 77, 8, True), (1, 1, 19, 5, True), (1, 2, 30, 64, False),
+              (2, 2, 50, 24, True), (1, 2, 1, 18, True)]     # 8, 5, 24 and 18 run padded to 16 or 32
 
 
 @pytest.mark.parametrize("N,H,L,D,w0", REC_SHAPES)
@@ -228,6 +230,56 @@ def test_rec(fwp, N, H, L, D, w0):
     names = "qx kx vx bx R_q R_k R_v r_b".split()
     for name, t, r in zip(names, ts, oracle.rec_bwd(*x, go)):
         check("grad_" + name, t.grad, r)
+
+
+def test_lds_state_kernels_of_the_recurrent_operators_at_a_small_head_size(fwp):
+    """The operators pad head sizes below 32; the autograd Functions under them do not, and send D = 5 to
+    the kernels that keep the state in LDS."""
+    N, H, L, D = 1, 2, 19, 5
+    z, k, v, W0, beta, h0, go = rnn_inputs(5, N, H, L, D, w0=True)
+    tz, tk, tv, tb = (dev(x, True) for x in (z, k, v, beta))
+    W, h = dev(W0), dev(h0)
+    out = fwp.FastRNNv2.apply(tz, tk, tv, W, tb, h)
+    ref_out, ref_W, ref_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+    check("rnn out", out, ref_out)
+    check("rnn W", W, ref_W)
+    out.backward(dev(go))
+    for name, t, r in zip("z k v beta".split(), (tz, tk, tv, tb), oracle.rnn_bwd(z, k, v, W0, beta, h0, go)):
+        check("rnn grad_" + name, t.grad, r)
+    *x, go = rec_inputs(6, N, H, L, D, w0=True)
+    ts = [dev(a, True) for a in x[:8]]
+    W, h = dev(x[8]), dev(x[9])
+    out = fwp.FastWeightRecUpdateTanh.apply(*ts, W, h)
+    ref_out, ref_W, ref_h = oracle.rec_fwd(*x)
+    check("rec out", out, ref_out)
+    check("rec h", h, ref_h)
+    out.backward(dev(go))
+    for name, t, r in zip("qx kx vx bx R_q R_k R_v r_b".split(), ts, oracle.rec_bwd(*x, go)):
+        check("rec grad_" + name, t.grad, r)
+
+
+@pytest.mark.parametrize("D", [24, 9])
+def test_padded_head_sizes_carry_their_states_and_keep_the_operators_errors(fwp, D):
+    """Head sizes that run padded: two calls with W and h carried over equal the oracle's whole run (the
+    states that come back are the narrow ones), outputs that differ by hundreds do not reach the padding,
+    and a state the operator refuses is refused with the operator's own message, W and h untouched."""
+    N, H, L = 2, 3, 44
+    z, k, v, W0, beta, h0, go = rnn_inputs(31 + D, N, H, L, D, w0=True)
+    z, h0 = z * 60.0, h0 * 60.0
+    ref_out, ref_W, ref_h = oracle.rnn_fwd(z, k, v, W0, beta, h0)
+    W, h = dev(W0), dev(h0)
+    a, b = slice(0, 20), slice(20, L)
+    outs = [fwp.fast_rnn_v2(dev(z[:, :, s]), dev(k[:, :, s]), dev(v[:, :, s]), W, dev(beta[:, :, s]), h) for s in (a, b)]
+    assert W.shape == (N, H, D, D) and h.shape == (N, H, 1, D)
+    check("out", torch.cat(outs, 2), ref_out)
+    check("W", W, ref_W)
+    check("h", h, ref_h)
+    before = W.clone()
+    with pytest.raises(fwp._lib.FwpError, match="contiguous"):
+        fwp.fast_rnn_v2(dev(z), dev(k), dev(v), W.transpose(2, 3), dev(beta), h)
+    with pytest.raises(AssertionError):
+        fwp.fast_rnn_v2(dev(z), dev(k[:, :, :-1]), dev(v), W, dev(beta), h)
+    assert torch.equal(W, before)
 
 
 @pytest.mark.parametrize("N,H,L,D", [(2, 3, 40, 32), (1, 2, 50, 16), (130, 8, 20, 32)])
