@@ -583,7 +583,7 @@ def main():
                     help="take the kernel-timing leg's launches from this build of libfwp_hip.so (a variant built "
                          "for a measurement); the eager step still runs on the package's own library")
     ap.add_argument("--dims", nargs=5, type=int, metavar=("B", "H", "T", "E", "M"),
-                    help="with --workload delta --kernel-leg-only: another batch and state shape (E key features, "
+                    help="with --workload delta or sum and --kernel-leg-only: another batch and state shape (E key features, "
                          "M value columns) for the per-kernel leg, e.g. 32 8 512 64 64")
     ap.add_argument("--kernel-leg-only", action="store_true",
                     help="only the per-kernel leg (back-to-back launches through the C ABI): for profiles of a "
@@ -641,10 +641,10 @@ def main():
         return
     w = WORKLOADS[name]
     if args.dims:
-        if name != "delta" or not args.kernel_leg_only:
-            sys.exit("bench.py: --dims goes with --workload delta --kernel-leg-only")
+        if name not in ("delta", "sum") or not args.kernel_leg_only:
+            sys.exit("bench.py: --dims goes with --workload delta or sum and --kernel-leg-only")
         B, H, T, E, M = args.dims
-        w = dict(w, B=B, H=H, T=T, E=E, M=M, label=f"delta-rule fast_weight fwd+bwd, B={B} H={H} T={T} E={E} M={M}, fp32")
+        w = dict(w, B=B, H=H, T=T, E=E, M=M, label=w["label"].split(",")[0] + f", B={B} H={H} T={T} E={E} M={M}, fp32")
     arrays = make_inputs(name, w)
     B, H, T, D = w["B"], w["H"], w["T"], w["D"]
     tokens = B * T
@@ -681,8 +681,9 @@ def main():
     if args.kernel_leg_only:
         th = B * H * T
         fwd_bytes, bwd_bytes = w["fwd_bytes"](D), w["bwd_bytes"](D)
-        if args.dims:       # the delta rule at E x M, per token-head: forward 2E + 2M + 1 floats, backward 4E + 3M + 2
-            fwd_bytes, bwd_bytes = (2 * w["E"] + 2 * w["M"] + 1) * 4, (4 * w["E"] + 3 * w["M"] + 2) * 4
+        if args.dims:       # at E x M, per token-head: forward 2E + 2M (+ 1: beta) floats, backward 4E + 3M (+ 2)
+            extra = name == "delta"
+            fwd_bytes, bwd_bytes = (2 * w["E"] + 2 * w["M"] + extra) * 4, (4 * w["E"] + 3 * w["M"] + 2 * extra) * 4
         t_step, _ = timed_steps(abi_step, 20, 200)      # state reset + forward + backward, through the C ABI
         print(json.dumps({"workload": w["label"], "lib": pkg._lib.SO_PATH, "fwd_us": t_f * 1e6, "bwd_us": t_b * 1e6,
                           "fwd_GBps": fwd_bytes * th / t_f / 1e9, "bwd_GBps": bwd_bytes * th / t_b / 1e9,

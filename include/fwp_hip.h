@@ -74,8 +74,8 @@ int fwp_query(int what);
  * FWP_CFG_DELTA_KERNELS selects the delta-rule kernels for E = M in {16, 32}:
  * FWP_DELTA_AUTO (default: the fastest), FWP_DELTA_SCAN (step-by-step register-state
  * kernels), FWP_DELTA_CHUNKED (16-step blocks on the matrix cores, one wave per sequence),
- * FWP_DELTA_SPLIT (the same blocks, a sequence's work split over several waves; the sum rule
- * takes the one-wave blocks), FWP_DELTA_PHASE (16 x 16 states: the blocks of a sequence prepared in
+ * FWP_DELTA_SPLIT (the same blocks, a sequence's work split over several waves; the sum rule's
+ * states of more than one 16 x 16 tile likewise, by key tiles and value tiles), FWP_DELTA_PHASE (16 x 16 states: the blocks of a sequence prepared in
  * parallel, one product per block on the sequential chain; other shapes as FWP_DELTA_SPLIT).  All give the same results within the fp32 tolerance.
  * FWP_CFG_STEP_KERNELS: 1 (default) sends forward calls of one step (L = 1) that save nothing for a
  * backward pass - stepwise inference, state carried from call to call - to kernels that do exactly

@@ -258,7 +258,7 @@ int fwp_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float 
         // square states of 16 or 32 also have the step-by-step kernels (short sequences, or on request)
         const bool blocked = in_range32(L, E, M, {q, k, v}) && (!reg_delta_supported(E, M) || delta_chunked(dk, L));
         if (blocked)
-            return mfma_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
+            return mfma_sum_fwd(dk, q, k, v, W, out, ckpt, N, H, L, E, M, chunk, (hipStream_t)stream);
         if (reg_delta_supported(E, M))
             return reg_sum_fwd(q, k, v, W, out, ckpt, N, H, L, E, chunk, (hipStream_t)stream);
     }
@@ -271,14 +271,15 @@ int fwp_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view grad_out, const flo
     if (bad_view(q) || bad_view(k) || bad_view(v) || bad_view(grad_out) || !ckpt || !gq || !gk || !gv)
         return FWP_E_NULL;
     if (int rc = check_dims(N, H, L, E, M, chunk)) return rc;
+    const int dk = g_delta_kernels;          // the one read of the switch in this call
     if (sum_blocked_dims(E, M) && reg_view_ok(q) && reg_view_ok(k) && reg_view_ok(v) &&
         reg_view_ok(grad_out) && aligned16(ckpt) && aligned16(W_init) && aligned16(gq) &&
         aligned16(gk) && aligned16(gv)) {
         const bool blocked =
             in_range32(L, E, M, {q, k, v, grad_out}) &&
-            (!reg_delta_supported(E, M) || delta_chunked(g_delta_kernels, L));
+            (!reg_delta_supported(E, M) || delta_chunked(dk, L));
         if (blocked)
-            return mfma_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
+            return mfma_sum_bwd(dk, q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, M, chunk,
                                 (hipStream_t)stream);
         if (reg_delta_supported(E, M))
             return reg_sum_bwd(q, k, v, grad_out, ckpt, W_init, gq, gk, gv, N, H, L, E, chunk,

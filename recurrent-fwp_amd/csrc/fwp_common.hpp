@@ -114,17 +114,18 @@ int mfma_delta_bwd(fwp_view q, fwp_view k, fwp_view beta, const float *vdiff, fw
                    int L, int D, int chunk, hipStream_t s);
 
 // the widest sum-rule shapes, built in a translation unit of their own
+// `mode` of the four below: the setting of FWP_CFG_DELTA_KERNELS (one wave per sequence or several)
 bool sum_wide_dims(int E, int M);
 // the state shapes the blocked sum-rule kernels are built for (a subset of the delta rule's plus the widest)
 bool sum_blocked_dims(int E, int M);
-int mfma_sum_wide_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+int mfma_sum_wide_fwd(int mode, fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                       int L, int E, int M, int chunk, hipStream_t s);
-int mfma_sum_wide_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+int mfma_sum_wide_bwd(int mode, fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
                       const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E,
                       int M, int chunk, hipStream_t s);
-int mfma_sum_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+int mfma_sum_fwd(int mode, fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                  int L, int E, int M, int chunk, hipStream_t s);
-int mfma_sum_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+int mfma_sum_bwd(int mode, fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
                  const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E, int M,
                  int chunk, hipStream_t s);
 

@@ -12,21 +12,21 @@ bool sum_wide_dims(int E, int M) {
 
 #define FWP_SUM_WIDE_SHAPES(X) X(1, 8) X(2, 8) X(8, 1) X(8, 2) X(12, 1)
 
-int mfma_sum_wide_fwd(fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
+int mfma_sum_wide_fwd(int mode, fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                       int L, int E, int M, int chunk, hipStream_t s) {
 #define X(ne, nm)                                                                                          \
-    if (E == 16 * ne && M == 16 * nm) return launch_sum_fwd<ne, nm>(q, k, v, W, out, ckpt, N, H, L, chunk, s);
+    if (E == 16 * ne && M == 16 * nm) return launch_sum_fwd<ne, nm>(mode, q, k, v, W, out, ckpt, N, H, L, chunk, s);
     FWP_SUM_WIDE_SHAPES(X)
 #undef X
     return FWP_E_SHAPE;
 }
 
-int mfma_sum_wide_bwd(fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
+int mfma_sum_wide_bwd(int mode, fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
                       const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int E,
                       int M, int chunk, hipStream_t s) {
 #define X(ne, nm)                                                                                          \
     if (E == 16 * ne && M == 16 * nm)                                                                      \
-        return launch_sum_bwd<ne, nm>(q, k, v, go, ckpt, W_init, gq, gk, gv, N, H, L, chunk, s);
+        return launch_sum_bwd<ne, nm>(mode, q, k, v, go, ckpt, W_init, gq, gk, gv, N, H, L, chunk, s);
     FWP_SUM_WIDE_SHAPES(X)
 #undef X
     return FWP_E_SHAPE;

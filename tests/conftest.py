@@ -24,7 +24,8 @@ def delta_kernels(request, fwp):
     """The kinds of delta-rule kernels for D = 16/32: the step-by-step scan, 16-step blocks on the
     matrix cores with one wave per sequence, those blocks split over several waves, and (16 x 16
     states) the blocks of a sequence prepared in parallel with a one-product chain.  The sum rule
-    has the first two; other shapes take the LDS kernels whatever the setting."""
+    has the first two and, for states of more than one 16 x 16 tile, several waves per sequence under the
+    last two; other shapes take the LDS kernels whatever the setting."""
     L_ = fwp._lib
     L_.config(L_.CFG_DELTA_KERNELS, {"scan": L_.DELTA_SCAN, "chunked": L_.DELTA_CHUNKED, "split": L_.DELTA_SPLIT,
                                       "phase": L_.DELTA_PHASE}[request.param])

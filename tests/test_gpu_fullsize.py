@@ -98,11 +98,14 @@ def off_by_one_float(t):
 
 
 @pytest.mark.parametrize("B,H,T,E,M", [(96, 8, 100, 32, 128), (96, 8, 100, 128, 32), (64, 4, 130, 16, 128),
-                                       (33, 9, 47, 128, 16), (40, 8, 100, 192, 16)])
+                                       (33, 9, 47, 128, 16), (40, 8, 100, 192, 16),
+                                       # up to 512 sequences: several waves per sequence (key tiles x value tiles)
+                                       (40, 8, 100, 32, 128), (40, 8, 100, 128, 32), (32, 8, 130, 64, 64),
+                                       (64, 8, 70, 16, 128), (50, 8, 90, 96, 32), (32, 16, 50, 32, 64)])
 def test_sum_widest_states_blocked_against_generic_kernels(fwp, B, H, T, E, M):
     """The fast-net layers' memories (d_head x 4 d_head and back) at hundreds of sequences: the
-    blocked kernels against the generic ones, which a misaligned q selects.  Tolerance as for the
-    oracle parity: |a - b| <= 1e-4 + 1e-3 |b|."""
+    blocked kernels (one wave per sequence beyond 512 sequences, several up to there) against the generic
+    ones, which a misaligned q selects.  Tolerance as for the oracle parity: |a - b| <= 1e-4 + 1e-3 |b|."""
     q, k, v, _, W0, go = (dev(a) for a in delta_inputs(5, B, H, T, E, M, dtype=np.float32, w0=True))
     res = []
     for misaligned in (False, True):
