@@ -383,31 +383,33 @@ inline bool sum_several_waves(int mode, int team, int nseq) {
     return mode != FWP_DELTA_AUTO || nseq <= kSumWavesMaxSeq;
 }
 
-template <int NE, int NM>
+// TEAM_ONLY: shapes too wide for one wave's registers, which take the team whatever the mode and the batch
+template <int NE, int NM, bool TEAM_ONLY = false>
 int launch_sum_fwd(int mode, fwp_view q, fwp_view k, fwp_view v, float *W, float *out, float *ckpt, int N, int H,
                    int L, int chunk, hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, spw = seq_per_wg(N * H);
     constexpr int WV = sum_waves(NE, NM), CV = sum_col_waves(NE, NM);
-    if (sum_several_waves(mode, WV * CV, N * H))
+    static_assert(!TEAM_ONLY || WV * CV > 1, "a shape without a one-wave kernel needs a team");
+    if (TEAM_ONLY || sum_several_waves(mode, WV * CV, N * H))
         hipLaunchKernelGGL((k_sum_fwd_mfma<NE, NM, WV, CV>), dim3(N * H), dim3(64 * WV * CV), 0, s, q, k, v, W, out,
                            ckpt, N * H, H, L, chunk, nchunk);
-    else
+    else if constexpr (!TEAM_ONLY)
         hipLaunchKernelGGL((k_sum_fwd_mfma<NE, NM>), dim3((N * H + spw - 1) / spw), dim3(64 * spw), 0, s, q, k, v,
                            W, out, ckpt, N * H, H, L, chunk, nchunk);
     return (int)hipGetLastError();
 }
 
-template <int NE, int NM>
+template <int NE, int NM, bool TEAM_ONLY = false>
 int launch_sum_bwd(int mode, fwp_view q, fwp_view k, fwp_view v, fwp_view go, const float *ckpt,
                    const float *W_init, float *gq, float *gk, float *gv, int N, int H, int L, int chunk,
                    hipStream_t s) {
     const int nchunk = (L + chunk - 1) / chunk, spw = seq_per_wg(N * H);
     constexpr int WV = sum_waves(NE, NM), CV = sum_col_waves(NE, NM);
-    if (sum_several_waves(mode, WV * CV, N * H))
+    if (TEAM_ONLY || sum_several_waves(mode, WV * CV, N * H))
         hipLaunchKernelGGL((k_sum_bwd_mfma<NE, NM, WV, CV>), dim3(N * H), dim3(64 * WV * CV),
                            WV * CV * 4 * sizeof(LdsMat), s, q, k, v, go, ckpt, W_init, gq, gk, gv, N * H, H, L,
                            chunk, nchunk);
-    else
+    else if constexpr (!TEAM_ONLY)
         hipLaunchKernelGGL((k_sum_bwd_mfma<NE, NM>), dim3((N * H + spw - 1) / spw), dim3(64 * spw),
                            spw * 4 * sizeof(LdsMat), s, q, k, v, go, ckpt, W_init, gq, gk, gv, N * H, H, L, chunk,
                            nchunk);

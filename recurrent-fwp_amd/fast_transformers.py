@@ -88,8 +88,8 @@ def _native_sum(Q, K, V, W):
 _operator = _native_sum if _fwp_torch is not None else FastWeightSum.apply
 
 # Value widths the blocked kernels take for a given key width, and those the single-step kernels take.
-_FAST_WIDTHS = {16: (16, 32, 64, 128), 32: (16, 32, 64, 128), 64: (16, 32, 64), 96: (16, 32), 128: (16, 32),
-                192: (16,)}
+_FAST_WIDTHS = {16: (16, 32, 64, 128), 32: (16, 32, 64, 128), 64: (16, 32, 64, 128), 96: (16, 32),
+                128: (16, 32, 64), 192: (16, 32)}
 _STEP_WIDTHS = (16, 32, 64, 128)
 _plans = {}
 
@@ -120,8 +120,8 @@ def sum_plan(E, M):
 
 def fast_weight_sum(Q, K, V, W):
     """``out = fast_weight_sum(Q, K, V, W)``, the reference's operator
-    (algorithmic/fast_transformers/__init__.py:84).  State shapes no blocked kernel takes whole (keys of
-    192 features with values of 32, values of 128 with keys of 64, widths that are not multiples of 16)
+    (algorithmic/fast_transformers/__init__.py:84).  State shapes no blocked kernel takes whole (keys and values of 128, values of
+    64 with keys of 96, widths that are not multiples of 16)
     run on them by slices of value columns with zero padded keys, see :func:`sum_plan`."""
     try:        # the common case first: a width pair seen before
         plan = _plans[(Q.size(-1), V.size(-1))]

@@ -198,8 +198,9 @@ def test_value_columns_are_sliced_onto_the_blocked_kernels(fwp):
     # the sum rule: its own table of widths, keys padded as well
     ft = fwp.fast_transformers
     assert ft.sum_plan(32, 128) is None and ft.sum_plan(192, 16) is None and ft.sum_plan(200, 16) is None
-    assert ft.sum_plan(192, 32) == (192, [(0, 16, 16), (16, 32, 16)])
-    assert ft.sum_plan(64, 128) == (64, [(0, 64, 64), (64, 128, 64)])
+    assert ft.sum_plan(192, 32) is None and ft.sum_plan(64, 128) is None and ft.sum_plan(128, 64) is None
+    assert ft.sum_plan(128, 128) == (128, [(0, 64, 64), (64, 128, 64)])
+    assert ft.sum_plan(96, 64) == (96, [(0, 32, 32), (32, 64, 32)])
     assert ft.sum_plan(48, 24) == (64, [(0, 24, 32)]) and ft.sum_plan(11, 4) == (16, [(0, 4, 16)])
     for E, M in ((32, 97), (32, 128), (128, 64), (96, 48), (64, 100), (16, 1), (16, 49), (64, 48)):
         plan = fw.column_plan(E, M)

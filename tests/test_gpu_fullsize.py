@@ -101,7 +101,9 @@ def off_by_one_float(t):
                                        (33, 9, 47, 128, 16), (40, 8, 100, 192, 16),
                                        # up to 512 sequences: several waves per sequence (key tiles x value tiles)
                                        (40, 8, 100, 32, 128), (40, 8, 100, 128, 32), (32, 8, 130, 64, 64),
-                                       (64, 8, 70, 16, 128), (50, 8, 90, 96, 32), (32, 16, 50, 32, 64)])
+                                       (64, 8, 70, 16, 128), (50, 8, 90, 96, 32), (32, 16, 50, 32, 64),
+                                       # only the several-wave form takes these, at any number of sequences
+                                       (40, 8, 60, 192, 32), (96, 8, 40, 64, 128), (24, 8, 70, 128, 64)])
 def test_sum_widest_states_blocked_against_generic_kernels(fwp, B, H, T, E, M):
     """The fast-net layers' memories (d_head x 4 d_head and back) at hundreds of sequences: the
     blocked kernels (one wave per sequence beyond 512 sequences, several up to there) against the generic

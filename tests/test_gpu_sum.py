@@ -59,8 +59,11 @@ SHAPES = [
     (1, 1, 31, 32, 16, False),
     # keys of 192 features whole; by slices of value columns and with zero padded keys
     (2, 2, 40, 192, 16, True),
-    (1, 2, 50, 192, 32, True),
+    (1, 2, 50, 192, 32, True),   # 192 x 32, 64 x 128, 128 x 64: whole, on several waves whatever the setting
     (2, 1, 40, 64, 128, True),
+    (1, 2, 70, 128, 64, False),
+    (1, 1, 40, 128, 128, True),  # two slices of 128 x 64
+    (2, 1, 33, 96, 64, True),    # two slices of 96 x 32
     (1, 2, 33, 48, 24, True),
     (1, 1, 70, 160, 40, False),
     (2, 2, 1, 64, 128, True),
@@ -129,13 +132,13 @@ def test_sum_equals_delta_rule_on_orthonormal_keys(fwp):
 def test_sum_by_slices_checks_the_state_it_is_given(fwp):
     """A state shape that runs by slices of value columns makes the checks of the whole-state path on the
     caller's W before anything runs, and leaves W alone when it raises."""
-    q, k, v, W0, _ = inputs(9, 1, 2, 20, 64, 128, True)
+    q, k, v, W0, _ = inputs(9, 1, 2, 20, 128, 128, True)
     tq, tk, tv, W = dev(q), dev(k), dev(v), dev(W0)
-    assert fwp.fast_transformers.sum_plan(64, 128) is not None
+    assert fwp.fast_transformers.sum_plan(128, 128) is not None
     with pytest.raises(fwp._lib.FwpError, match="W must be"):
         fwp.fast_weight_sum(tq, tk, tv, W.transpose(2, 3))
     with pytest.raises(fwp._lib.FwpError, match="W must be"):
-        fwp.fast_weight_sum(tq, tk, tv, W[:, :, :32])
+        fwp.fast_weight_sum(tq, tk, tv, W[:, :, :64])
     with pytest.raises(fwp._lib.FwpError, match="shape mismatch"):
         fwp.fast_weight_sum(tq, tk[:, :, :-1], tv, W)
     assert torch.equal(W, dev(W0))
