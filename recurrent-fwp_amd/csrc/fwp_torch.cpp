@@ -9,7 +9,8 @@
 // forward + backward pair of the benchmark shape takes 40-50 us on the GPU and ~57 us of interpreter
 // time through a Python autograd.Function, and a single inference step even less GPU time.
 // The delta rule, whose step is the shortest, is a graph node of its own (DeltaBackward) that also cuts value
-// widths no kernel takes whole into slices of columns and pads key widths; the others are autograd Functions.
+// widths no kernel takes whole into slices of columns and pads key widths; so is the sum rule (SumBackward); the
+// others are autograd Functions.
 // Host code only: tensors are PyTorch's, every kernel is behind the C ABI.
 #include <torch/extension.h>
 #include <torch/csrc/autograd/functions/utils.h>
@@ -388,25 +389,80 @@ at::Tensor delta_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const a
     return out;
 }
 
-struct SumFn : torch::autograd::Function<SumFn> {
-    // exact: grad_Q is the gradient of the recurrence as written; otherwise a carried-in state is left
-    // out of it, as the reference's backward does (causal_product_cuda.cu:385)
-    static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Q_in,
-                              const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &W, bool exact,
-                              bool need_grad) {
-        require_device(Q_in);
-        same_device(Q_in, {K_in, V_in, W});
-        if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
-        const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
-        if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}))
-            fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in));
-        if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
-            fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+// The sum rule's backward as a node of its own, like the delta rule's (its step is as short).
+struct SumBackward : torch::autograd::Node {
+    torch::autograd::SavedVariable Q_, K_, V_;
+    at::Tensor ckpt_, W_init_;          // the checkpointed states; the carried-in state unless `exact`
+    int chunk_ = 0;
+    bool released_ = false;
+
+    std::string name() const override { return "FwpSumBackward"; }
+
+    void release_variables() override {
+        std::lock_guard<std::mutex> lock(mutex_);
+        Q_.reset_data();
+        K_.reset_data();
+        V_.reset_data();
+        ckpt_.reset();
+        W_init_.reset();
+        released_ = true;
+    }
+
+    // one gradient per input edge: Q, K, V
+    torch::autograd::variable_list apply(torch::autograd::variable_list &&grads) override {
+        std::lock_guard<std::mutex> lock(mutex_);
+        torch::autograd::variable_list res(3);
+        if (grads.empty() || !grads[0].defined()) return res;
+        TORCH_CHECK(!released_, torch::autograd::ERR_BACKWARD_TWICE);
+        const at::Tensor Q = Q_.unpack(), K = K_.unpack(), V = V_.unpack();
+        const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3), M = V.size(3);
+        const fwp_view qv = view_of(Q), kv = view_of(K), vv = view_of(V);     // saved after rows()
+        same_device(Q, {grads[0]});
+        fwp_view gv_;
+        const at::Tensor go = rows(grads[0], gv_);
+        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M}, Q.options());
+        res[0] = parts.take(N, H, L, E);
+        res[1] = parts.take(N, H, L, E);
+        res[2] = parts.take(N, H, L, M);
+        LaunchGuard guard(Q);
+        check(fwp_sum_bwd(qv, kv, vv, gv_, ckpt_.data_ptr<float>(),
+                          W_init_.defined() ? W_init_.data_ptr<float>() : nullptr, res[0].data_ptr<float>(),
+                          res[1].data_ptr<float>(), res[2].data_ptr<float>(), (int)N, (int)H, (int)L, (int)E, (int)M,
+                          chunk_, stream_of(Q)),
+              "fwp_sum_bwd");
+        return res;
+    }
+};
+
+// exact: grad_Q is the gradient of the recurrence as written; otherwise a carried-in state is left out of
+// it, as the reference's backward does (causal_product_cuda.cu:385)
+at::Tensor sum_forward(const at::Tensor &Q_in, const at::Tensor &K_in, const at::Tensor &V_in, const at::Tensor &W,
+                       bool exact) {
+    require_device(Q_in);
+    same_device(Q_in, {K_in, V_in, W});
+    if (Q_in.dim() != 4 || V_in.dim() != 4) fail("expected 4-D [N,H,L,D] tensors");
+    const int64_t N = Q_in.size(0), H = Q_in.size(1), L = Q_in.size(2), E = Q_in.size(3), M = V_in.size(3);
+    if (K_in.sizes() != Q_in.sizes() || V_in.sizes() != at::IntArrayRef({N, H, L, M}))
+        fail("shape mismatch: Q" + shape_of(Q_in) + " K" + shape_of(K_in) + " V" + shape_of(V_in));
+    if (W.sizes() != at::IntArrayRef({N, H, E, M}) || !W.is_contiguous() || W.scalar_type() != at::kFloat)
+        fail("W must be a contiguous fp32 [N,H,E,M] tensor");
+    const bool need_grad =
+        at::GradMode::is_enabled() && (Q_in.requires_grad() || K_in.requires_grad() || V_in.requires_grad());
+    std::shared_ptr<SumBackward> node;
+    if (need_grad) {
+        node = std::shared_ptr<SumBackward>(new SumBackward(), torch::autograd::deleteNode);
+        node->set_next_edges(torch::autograd::collect_next_edges(Q_in, K_in, V_in));
+    }
+    at::Tensor out;
+    {
+        // below autograd: copies of unaligned views and of the carried-in state record nothing
+        at::AutoDispatchBelowADInplaceOrView below;
         fwp_view qv, kv, vv;
         const at::Tensor Q = rows(Q_in, qv), K = rows(K_in, kv), V = rows(V_in, vv);
         const int chunk = fwp_query(FWP_Q_DEFAULT_CHUNK);
         const auto opts = Q.options();
-        at::Tensor out = at::empty({N, H, L, M}, opts), ckpt, W_init;
+        out = at::empty({N, H, L, M}, opts);
+        at::Tensor ckpt, W_init;
         if (need_grad) {
             ckpt = at::empty({N, H, (L + chunk - 1) / chunk, E, M}, opts);
             if (!exact) W_init = W.clone();
@@ -419,39 +475,17 @@ struct SumFn : torch::autograd::Function<SumFn> {
                   "fwp_sum_fwd");
         }
         if (need_grad) {
-            if (exact) ctx->save_for_backward({Q, K, V, ckpt});
-            else ctx->save_for_backward({Q, K, V, ckpt, W_init});
-            ctx->saved_data["chunk"] = (int64_t)chunk;
+            node->Q_ = torch::autograd::SavedVariable(Q, false);
+            node->K_ = torch::autograd::SavedVariable(K, false);
+            node->V_ = torch::autograd::SavedVariable(V, false);
+            node->ckpt_ = std::move(ckpt);
+            node->W_init_ = std::move(W_init);
+            node->chunk_ = chunk;
         }
-        if (ctx) ctx->set_materialize_grads(false);
-        return out;
     }
-
-    static torch::autograd::tensor_list backward(torch::autograd::AutogradContext *ctx,
-                                                 torch::autograd::tensor_list grads) {
-        const at::Tensor none;
-        if (!grads[0].defined()) return {none, none, none, none, none, none};
-        const auto saved = ctx->get_saved_variables();
-        if (saved.size() < 4) fail("backward of a forward pass that kept nothing for it");
-        const at::Tensor &Q = saved[0], &K = saved[1], &V = saved[2], &ckpt = saved[3];
-        const int64_t N = Q.size(0), H = Q.size(1), L = Q.size(2), E = Q.size(3), M = V.size(3);
-        const int chunk = (int)ctx->saved_data["chunk"].toInt();
-        const fwp_view qv = view_of(Q), kv = view_of(K), vv = view_of(V);     // saved after rows()
-        fwp_view gv_;
-        const at::Tensor go = rows(grads[0], gv_);
-        Parts parts({N * H * L * E, N * H * L * E, N * H * L * M}, Q.options());
-        const at::Tensor gq = parts.take(N, H, L, E), gk = parts.take(N, H, L, E), gv = parts.take(N, H, L, M);
-        {
-            LaunchGuard guard(Q);
-            check(fwp_sum_bwd(qv, kv, vv, gv_, ckpt.data_ptr<float>(),
-                              saved.size() > 4 ? saved[4].data_ptr<float>() : nullptr, gq.data_ptr<float>(),
-                              gk.data_ptr<float>(), gv.data_ptr<float>(), (int)N, (int)H, (int)L, (int)E, (int)M,
-                              chunk, stream_of(Q)),
-                  "fwp_sum_bwd");
-        }
-        return {gq, gk, gv, none, none, none};
-    }
-};
+    if (need_grad) torch::autograd::set_history(out, node);
+    return out;
+}
 
 struct RnnFn : torch::autograd::Function<RnnFn> {
     static at::Tensor forward(torch::autograd::AutogradContext *ctx, const at::Tensor &Z_in, const at::Tensor &K_in,
@@ -754,12 +788,7 @@ std::tuple<at::Tensor, at::Tensor> fast_lstm_v4(
 
 at::Tensor fast_weight_sum(const at::Tensor &Q, const at::Tensor &K, const at::Tensor &V, const at::Tensor &W,
                            bool exact) {
-    const bool need_grad = at::GradMode::is_enabled() && (Q.requires_grad() || K.requires_grad() || V.requires_grad());
-    if (!need_grad) {
-        at::AutoDispatchBelowADInplaceOrView below;
-        return SumFn::forward(nullptr, Q, K, V, W, exact, false);
-    }
-    return SumFn::apply(Q, K, V, W, exact, need_grad);
+    return sum_forward(Q, K, V, W, exact);
 }
 
 // time_major: None = out's memory follows Q's, True = [L,N,H,M] storage, False = contiguous [N,H,L,M]
